@@ -1,0 +1,187 @@
+/*
+ * pluto_oracle.h -- CPU restatement of the reference's attention hot path.
+ *
+ * THIS IS TEST INFRASTRUCTURE, NOT PRODUCT CODE.  Only the test-suite, the
+ * smoke check and the benchmark's cpu_baseline leg may link or call it, and
+ * only as the checker.  Nothing that ships computes through this library.
+ *
+ * Every function restates, in scalar C, a function of the reference
+ * (sanjoy/pluto); the reference file:line it follows is cited at each
+ * declaration.  Arithmetic is done in the same precision and order as the
+ * cited code so results agree to the last bit wherever the cited code is
+ * itself deterministic scalar code.
+ *
+ * Pinning status (which independent evidence fixes each function):
+ *   mha_fwd / mha_bwd        closed form (attention_test.cc:282-360), float64
+ *                            scaled_dot_product_attention + autograd, brute
+ *                            force, causality invariants.
+ *   gqa_*                    known answers of cached_attention_test.cc:108-156,
+ *                            exact gate expectation and uniform 1/L rows of
+ *                            cached_attention_ops_test.cc:364-398,472-503,
+ *                            an independent float64 numpy restatement.
+ *   gdn_*                    textbook delta rule special cases (beta=0, g=0
+ *                            with orthonormal keys), softplus extremes,
+ *                            independent float64 numpy recurrence.
+ */
+#ifndef PLUTO_ORACLE_H_
+#define PLUTO_ORACLE_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Storage type of activations.  The reference's DataType::FP16 policy keeps
+ * FP32 storage (src/llm/layer.h:86-88); DataType::BF16 stores bfloat16. */
+enum { PLUTO_ORACLE_F32 = 0, PLUTO_ORACLE_BF16 = 1 };
+
+/* src/llm/layers/reference_internal.h:109-119 (round to nearest even). */
+uint16_t pluto_oracle_f32_to_bf16(float value);
+float pluto_oracle_bf16_to_f32(uint16_t value);
+float pluto_oracle_bf16_round(float value);
+
+/* ---- GPT-2 style causal multi-head attention -------------------------- */
+
+/* src/llm/layers/attention_reference.cc:36-114.  qkv is the packed
+ * [rows, 3*E] activation, out is [rows, E].  Additionally reports the
+ * per-(sequence, head, position) maximum and normalizer of the softmax row
+ * ([rows/T * H, T] each, nullable), which the reference's device layer saves
+ * (src/llm/layers/attention.cc:448-451) and the CPU class does not.
+ * Only sequences [seq_begin, seq_end) and heads [head_begin, head_end) are
+ * computed; other outputs are left untouched.  Returns 0, or -1 on a shape
+ * the reference rejects. */
+int pluto_oracle_mha_fwd(int dtype, const void* qkv, int rows,
+                         int context_length, int num_heads, int embedding_dim,
+                         void* out, float* maxima, float* normalizers,
+                         int seq_begin, int seq_end, int head_begin,
+                         int head_end);
+
+/* src/llm/layers/attention_reference.cc:116-230.  d_qkv must be zeroed by
+ * the caller ([rows, 3*E] fp32); d_out is fp32 [rows, E]; out is the stored
+ * forward output. */
+int pluto_oracle_mha_bwd(int dtype, const void* qkv, const void* out,
+                         const float* d_out, int rows, int context_length,
+                         int num_heads, int embedding_dim, float* d_qkv,
+                         int seq_begin, int seq_end, int head_begin,
+                         int head_end);
+
+/* ---- Qwen style grouped-query attention ------------------------------- */
+
+/* src/llm/layers/util/cached_attention_ops.h:13-22 */
+typedef struct {
+  int query_heads;
+  int key_value_heads;
+  int head_dim;
+  int rotary_dim;
+  int capacity;
+  float rms_norm_epsilon;
+  float rope_theta;
+  int round_to_bfloat16;
+} pluto_oracle_attention_params;
+
+/* Per-head RMSNorm with (1 + weight) and split-half partial RoPE at
+ * `position`: src/llm/layers/util/cached_attention_ops_test.cc:56-78 (scalar
+ * specification of cached_attention_ops.cc:30-79). */
+void pluto_oracle_gqa_normalize_rotate(const pluto_oracle_attention_params* p,
+                                       int position, const float* input,
+                                       const float* weight, float* output);
+
+/* One cached decode step: cached_attention_ops_test.cc:46-118 (scalar
+ * specification of CachedAttentionStep, cached_attention_ops.cc:308-353).
+ * cache_keys / cache_values are FP32 [capacity, kv_heads, head_dim]
+ * (src/llm/key_value_cache.h:13-16); `position` rows are valid on entry and
+ * row `position` is written.  q_gate is [qh, 2, d], k/v are [kh, d], output
+ * is [qh, d], probabilities (nullable) is [qh, position + 1].
+ * Returns 0, -1 for invalid parameters, -2 when the cache is full. */
+int pluto_oracle_gqa_cached_step(const pluto_oracle_attention_params* p,
+                                 float* cache_keys, float* cache_values,
+                                 int position, const float* q_gate,
+                                 const float* k, const float* v,
+                                 const float* q_norm, const float* k_norm,
+                                 float* output, float* probabilities);
+
+/* Whole-sequence attention with the semantics of
+ * QwenAttentionLayer::SequenceForward (src/llm/layers/qwen_attention.cc:
+ * 414-448; scalar specification qwen_attention_test.cc:26-95): row t is the
+ * cached step at position t.  qg is [T, qh, 2, d], k/v are [T, kh, d]; all
+ * inputs are FP32 holding the (bf16 representable) activations.  Writes the
+ * prepared keys and rounded values for every row < row_end into key_out /
+ * value_out ([T, kh, d], nullable) and the gated output [T, qh, d] for rows
+ * [row_begin, row_end) and heads [head_begin, head_end).  lse (nullable,
+ * [T, qh]) receives max + log(normalizer) of each softmax row. */
+int pluto_oracle_gqa_sequence(const pluto_oracle_attention_params* p,
+                              int length, const float* qg, const float* k,
+                              const float* v, const float* q_norm,
+                              const float* k_norm, float* out, float* key_out,
+                              float* value_out, float* lse, int row_begin,
+                              int row_end, int head_begin, int head_end);
+
+/* Attention of prepared queries against an existing cache, used for the
+ * batched decode configuration: q is [qh, d] already normalised and rotated,
+ * gate is [qh, d] raw logits, keys/values are [kh, length, d] head-major FP32
+ * views of a bf16 cache (row stride = stride_tokens rows per head).  Softmax
+ * and gating follow cached_attention_ops_test.cc:86-114. */
+int pluto_oracle_gqa_attend(const pluto_oracle_attention_params* p, int length,
+                            size_t head_stride, const float* q,
+                            const float* gate, const float* keys,
+                            const float* values, float* output);
+
+/* ---- Gated delta-net --------------------------------------------------- */
+
+/* src/llm/layers/util/cached_attention_ops.h:49-57 */
+typedef struct {
+  int key_heads;
+  int value_heads;
+  int key_head_dim;
+  int value_head_dim;
+  int conv_kernel_dim;
+  float rms_norm_epsilon;
+  int round_to_bfloat16;
+} pluto_oracle_delta_params;
+
+/* The recurrence alone: sequence_delta_net_test.cc:100-141 (scalar
+ * specification of RecurrenceForward, sequence_delta_net.cc:55-102).
+ * q, k are [T, kh, kd]; v is [T, vh, vd]; log_decay and beta are [T, vh]
+ * (decay = exp(log_decay); beta is used as given).  When normalize_qk is
+ * nonzero q and k are L2-normalised as the reference does (1e-6 added to the
+ * sum of squares); q is always multiplied by q_scale (the reference uses
+ * 1/sqrt(kd)).  state is FP64 [vh, kd, vd], read as the initial state and
+ * overwritten with the final state.  core is [T, vh, vd], rounded to bf16
+ * when p->round_to_bfloat16.  Heads [head_begin, head_end) only. */
+int pluto_oracle_gdn_scan(const pluto_oracle_delta_params* p, int length,
+                          const float* q, const float* k, const float* v,
+                          const float* log_decay, const float* beta,
+                          int normalize_qk, double q_scale, double* state,
+                          float* core, int head_begin, int head_end);
+
+/* Whole layer over a sequence: sequence_delta_net_test.cc:66-159 (scalar
+ * specification of SequenceDeltaNetLayer::fwd_impl, sequence_delta_net.cc:
+ * 435-480).  qkv is [T, 2*kh*kd + vh*vd] packed [all Q | all K | all V],
+ * z is [T, vh*vd], a and b are [T, vh]; conv_weight is [channels, kernel];
+ * a_log, dt_bias are [vh]; norm is [vd].  output is [T, vh*vd].  core
+ * (nullable) receives the pre-norm recurrence output, final_state (nullable)
+ * the FP64 [vh, kd, vd] state after the last token. */
+int pluto_oracle_gdn_sequence(const pluto_oracle_delta_params* p, int length,
+                              const float* qkv, const float* z, const float* a,
+                              const float* b, const float* conv_weight,
+                              const float* a_log, const float* dt_bias,
+                              const float* norm, float* output, float* core,
+                              double* final_state);
+
+/* Single-token step with persistent state: cached_attention_ops_test.cc:
+ * 133-220 (scalar specification of DeltaNetState::Step,
+ * cached_attention_ops.cc:401-431).  conv_state is FP32 [channels, kernel],
+ * recurrent_state is FP64 [vh, kd, vd]; both are updated in place. */
+int pluto_oracle_gdn_step(const pluto_oracle_delta_params* p,
+                          float* conv_state, double* recurrent_state,
+                          const float* qkv, const float* z, const float* a,
+                          const float* b, const float* conv_weight,
+                          const float* a_log, const float* dt_bias,
+                          const float* norm, float* output);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PLUTO_ORACLE_H_ */
