@@ -1,0 +1,281 @@
+/*
+ * pluto_hip.h -- C ABI of the MI355X (gfx950) attention path.
+ *
+ * This is the boundary a maintainer of the reference (sanjoy/pluto) binds to
+ * replace the execution pieces of its attention hot path: the stream/buffer
+ * runtime of src/cuda and the device kernels of src/llm/layers/{attention,
+ * qwen_attention,sequence_delta_net,delta_net}.cc and
+ * src/llm/layers/util/cached_attention_ops.cc.  Every entry point cites the
+ * reference interface it stands in for.
+ *
+ * Conventions
+ *   - plain C types only: device/host pointers, sizes, ints, floats.
+ *   - every function returns 0 on success.  Positive values are hipError_t
+ *     codes reported by the HIP runtime; negative values are the PLUTO_HIP_E*
+ *     codes below (argument validation, done before any GPU work is queued).
+ *   - `stream` is a hipStream_t passed as void*.  Nothing synchronises with
+ *     the host and nothing uses the default stream; all work is queued on the
+ *     given stream, and calls on different streams may run concurrently.
+ *   - kernels never allocate: scratch memory is passed in as `workspace`, whose
+ *     required size the matching *_workspace_bytes function reports.
+ */
+#ifndef PLUTO_HIP_H_
+#define PLUTO_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PLUTO_HIP_EINVAL (-1)       /* invalid argument (absl::InvalidArgument) */
+#define PLUTO_HIP_ERANGE (-2)       /* capacity exhausted (absl::ResourceExhausted) */
+#define PLUTO_HIP_EUNSUPPORTED (-3) /* not implemented (absl::Unimplemented) */
+#define PLUTO_HIP_EWORKSPACE (-4)   /* workspace missing or too small */
+
+/* Storage type of an activation buffer.  The reference's DataType::FP16
+ * compute policy keeps FP32 storage (src/llm/layer.h:86-88). */
+#define PLUTO_HIP_F32 0
+#define PLUTO_HIP_BF16 1
+
+/* Human readable text for any value returned by this library. */
+const char* pluto_hip_error_name(int code);
+const char* pluto_hip_error_string(int code);
+
+/* Library/ABI version and the gfx target the kernels were compiled for. */
+int pluto_hip_abi_version(void);
+const char* pluto_hip_target_arch(void);
+
+/* ------------------------------------------------------------------------
+ * Runtime: replaces src/cuda/executor.{h,cc}, buffer.{h,cc} and
+ * page_locked_host_buffer.{h,cc} for this path.
+ * --------------------------------------------------------------------- */
+
+typedef struct pluto_hip_executor pluto_hip_executor;
+
+/* cuda::Executor::Create (src/cuda/executor.cc:35-96): one non-blocking
+ * compute stream, one non-blocking immediate stream, a pinned-host block
+ * cache.  Uses the calling thread's current device. */
+int pluto_hip_executor_create(pluto_hip_executor** executor);
+/* cuda::Executor::~Executor (src/cuda/executor.cc:98-116): drains both
+ * streams, releases cached pinned blocks, destroys the streams. */
+int pluto_hip_executor_destroy(pluto_hip_executor* executor);
+/* cuda::Executor::Synchronize (src/cuda/executor.cc:118-120). */
+int pluto_hip_executor_synchronize(pluto_hip_executor* executor);
+/* cuda::Executor::stream / immediate_stream (src/cuda/executor.h:42-51). */
+void* pluto_hip_executor_stream(pluto_hip_executor* executor);
+void* pluto_hip_executor_immediate_stream(pluto_hip_executor* executor);
+
+/* cuda::Buffer::Allocate (src/cuda/buffer.cc:53-68): stream-ordered device
+ * allocation on the compute stream.  bytes == 0 yields *data == NULL. */
+int pluto_hip_malloc_async(pluto_hip_executor* executor, size_t bytes,
+                           void** data);
+/* cuda::Buffer::Allocation::~Allocation (src/cuda/buffer.cc:33-47): the free
+ * is ordered after all work queued so far on the compute stream. */
+int pluto_hip_free_async(pluto_hip_executor* executor, void* data);
+
+/* cuda::PageLockedHostBuffer::Allocate
+ * (src/cuda/page_locked_host_buffer.h:27-29): pinned host memory that the CPU
+ * may touch as soon as the call returns, without waiting for compute. */
+int pluto_hip_host_alloc(pluto_hip_executor* executor, size_t bytes,
+                         void** data);
+/* Release of a pinned block: it is recycled only after the work queued on
+ * the compute stream at the time of this call has finished
+ * (src/cuda/page_locked_host_buffer.h:13-24). */
+int pluto_hip_host_free_async(pluto_hip_executor* executor, void* data);
+
+/* cudaMemcpyAsync / cudaMemsetAsync call sites of the path
+ * (src/llm/layers/util/cached_attention_ops.cc:433-441,
+ *  src/llm/block_parameter.cc:56-66).  kind: 1 H2D, 2 D2H, 3 D2D. */
+int pluto_hip_memcpy_async(void* stream, void* dst, const void* src,
+                           size_t bytes, int kind);
+int pluto_hip_memset_async(void* stream, void* dst, int value, size_t bytes);
+int pluto_hip_stream_synchronize(void* stream);
+
+/* CastKernel of src/llm/layers/util.cc:14-40 (ToFloat / ToBFloat16). */
+int pluto_hip_cast_bf16_to_f32(void* stream, const void* src, float* dst,
+                               size_t count);
+int pluto_hip_cast_f32_to_bf16(void* stream, const float* src, void* dst,
+                               size_t count);
+
+/* ------------------------------------------------------------------------
+ * GPT-2 style causal multi-head attention over packed [rows, 3E] Q|K|V.
+ * --------------------------------------------------------------------- */
+
+/* AttentionLayer::fwd_impl + FlashAttentionForwardKernel
+ * (src/llm/layers/attention.cc:418-507, 98-170).
+ *   qkv          [rows, 3E], head h at columns h*D.. of each third
+ *   out          [rows, E]   (same storage type as qkv)
+ *   maxima       [rows/T * H, T] fp32, max of the scaled visible scores
+ *   normalizers  [rows/T * H, T] fp32, sum of exp(score - max)
+ * rows must be a positive multiple of context_length and E of num_heads. */
+int pluto_hip_mha_forward(void* stream, int dtype, const void* qkv, int rows,
+                          int context_length, int num_heads, int embedding_dim,
+                          void* out, float* maxima, float* normalizers);
+
+/* AttentionProbabilitiesKernel (src/llm/layers/attention.cc:176-230):
+ * fp32 probabilities [rows/T, H, T, T] rebuilt from the saved statistics,
+ * zeros above the diagonal. */
+int pluto_hip_mha_probabilities(void* stream, int dtype, const void* qkv,
+                                const float* maxima, const float* normalizers,
+                                int rows, int context_length, int num_heads,
+                                int embedding_dim, float* probabilities);
+
+/* AttentionLayer::bwd_impl + the two backward kernels
+ * (src/llm/layers/attention.cc:509-596, 235-396).
+ *   d_out   [rows, E] fp32 upstream gradient
+ *   d_qkv   [rows, 3E] fp32, every element written exactly once
+ * Deterministic: single-writer tiles, fixed reduction order, no atomics.
+ * The workspace replaces the `deltas` buffer the reference allocates
+ * (attention.cc:544) and holds the bf16 copy of d_out the MFMA path uses. */
+size_t pluto_hip_mha_backward_workspace_bytes(int dtype, int rows,
+                                              int context_length,
+                                              int num_heads,
+                                              int embedding_dim);
+int pluto_hip_mha_backward(void* stream, int dtype, const void* qkv,
+                           const void* out, const float* d_out,
+                           const float* maxima, const float* normalizers,
+                           int rows, int context_length, int num_heads,
+                           int embedding_dim, float* d_qkv, void* workspace,
+                           size_t workspace_bytes);
+
+/* ------------------------------------------------------------------------
+ * Qwen style grouped-query attention with a contiguous KV cache.
+ * --------------------------------------------------------------------- */
+
+/* FullAttentionParameters (src/llm/layers/util/cached_attention_ops.h:13-22);
+ * round_to_bfloat16 is an int here. */
+typedef struct {
+  int query_heads;
+  int key_value_heads;
+  int head_dim;
+  int rotary_dim;
+  int capacity;
+  float rms_norm_epsilon;
+  float rope_theta;
+  int round_to_bfloat16;
+} pluto_hip_attention_params;
+
+/* One sequence's K and V storage (KeyValueCache, src/llm/key_value_cache.h:
+ * 25-57).  Element (token t, kv head h, channel c) of either tensor lives at
+ * base[t * token_stride + h * head_stride + c].  The reference layout is FP32
+ * token-major (token_stride = kh*d, head_stride = d); the native layout of
+ * this library is BF16 head-major [kh, capacity, d] (token_stride = d,
+ * head_stride = capacity*d), which is lossless while round_to_bfloat16 is set
+ * because every stored value is then bf16 representable
+ * (cached_attention_ops.cc:64-67,75-77). */
+typedef struct {
+  void* keys;
+  void* values;
+  int dtype; /* PLUTO_HIP_F32 or PLUTO_HIP_BF16 */
+  long long token_stride;
+  long long head_stride;
+} pluto_hip_kv_cache_view;
+
+/* ValidateCachedAttention (cached_attention_ops.cc:283-306), parameter part:
+ * PLUTO_HIP_EINVAL for anything the reference rejects. */
+int pluto_hip_attention_params_validate(const pluto_hip_attention_params* p);
+
+/* Whole-sequence GQA ("prefill") with the semantics of
+ * QwenAttentionLayer::SequenceForward (src/llm/layers/qwen_attention.cc:
+ * 414-448: PrepareKernel :30-63, ForwardKernel :68-119) and the cache append
+ * of PrepareAttentionKernel (cached_attention_ops.cc:72-77): rows
+ * [start_position, start_position + length) of the cache are written, and
+ * row i attends to cache rows [0, start_position + i].
+ *   qg   bf16 [length, qh, 2, d]  (query at [..,0,:], gate logits at [..,1,:])
+ *   k,v  bf16 [length, kh, d]
+ *   q_norm, k_norm  fp32 [d], zero centred (multiplier 1 + w)
+ *   out  bf16 [length, qh, d] = bf16(bf16(core) * bf16(sigmoid(gate)))
+ *   lse  optional fp32 [length, qh]: max + log(normalizer) of each row
+ * The quadratic probability tensor of the reference is not produced. */
+size_t pluto_hip_gqa_prefill_workspace_bytes(const pluto_hip_attention_params* p,
+                                             int length);
+int pluto_hip_gqa_prefill(void* stream, const pluto_hip_attention_params* p,
+                          int length, int start_position, const void* qg,
+                          const void* k, const void* v, const float* q_norm,
+                          const float* k_norm,
+                          const pluto_hip_kv_cache_view* cache, void* out,
+                          float* lse, void* workspace, size_t workspace_bytes);
+
+/* Batched single-token decode: `batch` independent CachedAttentionStep calls
+ * (cached_attention_ops.cc:308-353: PrepareAttentionKernel :30-79,
+ * FullAttentionKernel :83-126) in one launch sequence.  Sequence b appends
+ * its token at row positions[b] of caches[b] and attends to rows
+ * [0, positions[b]].  The caller advances its position counters after a
+ * successful return (KeyValueCache::Advance).
+ *   io_dtype  storage of q_gate, k, v and out: PLUTO_HIP_F32 (the reference's
+ *             pointers) or PLUTO_HIP_BF16 (skips the four cast launches of
+ *             qwen_attention.cc:381-386,409-411)
+ *   q_gate [batch, qh, 2, d], k/v [batch, kh, d], out [batch, qh, d]
+ *   positions, caches: HOST arrays of length batch
+ *   probabilities: optional HOST array of `batch` device pointers (entries may
+ *             be NULL), each fp32 [qh, positions[b] + 1]
+ *             (AttentionProbabilitiesKernel, cached_attention_ops.cc:131-178)
+ *   split_tokens: tokens per split-K block (512 in the decode configuration;
+ *             0 selects the default)
+ * Returns PLUTO_HIP_ERANGE if any positions[b] >= capacity; nothing is
+ * queued in that case. */
+size_t pluto_hip_gqa_decode_workspace_bytes(const pluto_hip_attention_params* p,
+                                            int batch, const int* positions,
+                                            int split_tokens);
+int pluto_hip_gqa_decode(void* stream, const pluto_hip_attention_params* p,
+                         int batch, int io_dtype, const void* q_gate,
+                         const void* k, const void* v, const float* q_norm,
+                         const float* k_norm, const int* positions,
+                         const pluto_hip_kv_cache_view* caches, void* out,
+                         float* const* probabilities, int split_tokens,
+                         void* workspace, size_t workspace_bytes);
+
+/* ------------------------------------------------------------------------
+ * Gated delta-net.
+ * --------------------------------------------------------------------- */
+
+/* DeltaNetParameters (cached_attention_ops.h:49-57). */
+typedef struct {
+  int key_heads;
+  int value_heads;
+  int key_head_dim;
+  int value_head_dim;
+  int conv_kernel_dim;
+  float rms_norm_epsilon;
+  int round_to_bfloat16;
+} pluto_hip_delta_params;
+
+/* Chunked scan of the gated delta rule; semantics of RecurrenceForward
+ * (src/llm/layers/sequence_delta_net.cc:55-102) for `batch` independent
+ * sequences, without the per-token state snapshots:
+ *     S <- exp(g_t) S;  delta = (v_t - S^T k_t) beta_t;  S <- S + k_t delta^T
+ *     o_t = S^T (q_t * q_scale)
+ *   q, k        bf16 [batch, length, kh, kd]
+ *   v           bf16 [batch, length, vh, vd]
+ *   log_decay   fp32 [batch, length, vh]   (g_t <= 0)
+ *   beta        fp32 [batch, length, vh]
+ *   normalize_qk  when set, q and k are L2 normalised inside the kernel with
+ *               1e-6 added to the sum of squares (sequence_delta_net.cc:84-85)
+ *   state       fp32 [batch, vh, kd, vd], read as S_0, overwritten with S_T
+ *   out         bf16 [batch, length, vh, vd]
+ *   chunk       tokens per chunk (64); 0 selects the default. */
+size_t pluto_hip_gdn_scan_workspace_bytes(const pluto_hip_delta_params* p,
+                                          int batch, int length, int chunk);
+int pluto_hip_gdn_scan(void* stream, const pluto_hip_delta_params* p,
+                       int batch, int length, int chunk, const void* q,
+                       const void* k, const void* v, const float* log_decay,
+                       const float* beta, int normalize_qk, float q_scale,
+                       float* state, void* out, void* workspace,
+                       size_t workspace_bytes);
+
+/* Token-by-token form of the same recurrence (the reference's own loop
+ * structure); used for short sequences and as the device-side cross check
+ * of the chunked scan.  Same arguments; out_dtype selects fp32 or bf16 `out`. */
+int pluto_hip_gdn_recurrence(void* stream, const pluto_hip_delta_params* p,
+                             int batch, int length, const void* q,
+                             const void* k, const void* v,
+                             const float* log_decay, const float* beta,
+                             int normalize_qk, float q_scale, float* state,
+                             void* out, int out_dtype);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PLUTO_HIP_H_ */

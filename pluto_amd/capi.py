@@ -1,0 +1,200 @@
+"""ctypes binding of libpluto_hip.so (the C ABI declared in include/pluto_hip.h).
+
+torch is used for plumbing only: device memory (tensors) and the current HIP
+stream.  It is imported before the library is loaded so that both share one
+HIP runtime.  There is no fallback: if the library is missing or a call
+fails, an exception is raised.
+"""
+import ctypes
+import os
+
+import torch  # noqa: F401  (must precede loading the library, see above)
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libpluto_hip.so")
+
+F32 = 0
+BF16 = 1
+
+EINVAL, ERANGE, EUNSUPPORTED, EWORKSPACE = -1, -2, -3, -4
+
+
+class PlutoHipError(RuntimeError):
+    def __init__(self, code, name, text):
+        super().__init__("%s (%d): %s" % (name, code, text))
+        self.code = code
+
+
+class AttentionParams(ctypes.Structure):
+    _fields_ = [
+        ("query_heads", ctypes.c_int),
+        ("key_value_heads", ctypes.c_int),
+        ("head_dim", ctypes.c_int),
+        ("rotary_dim", ctypes.c_int),
+        ("capacity", ctypes.c_int),
+        ("rms_norm_epsilon", ctypes.c_float),
+        ("rope_theta", ctypes.c_float),
+        ("round_to_bfloat16", ctypes.c_int),
+    ]
+
+
+class KvCacheView(ctypes.Structure):
+    _fields_ = [
+        ("keys", ctypes.c_void_p),
+        ("values", ctypes.c_void_p),
+        ("dtype", ctypes.c_int),
+        ("token_stride", ctypes.c_longlong),
+        ("head_stride", ctypes.c_longlong),
+    ]
+
+
+class DeltaParams(ctypes.Structure):
+    _fields_ = [
+        ("key_heads", ctypes.c_int),
+        ("value_heads", ctypes.c_int),
+        ("key_head_dim", ctypes.c_int),
+        ("value_head_dim", ctypes.c_int),
+        ("conv_kernel_dim", ctypes.c_int),
+        ("rms_norm_epsilon", ctypes.c_float),
+        ("round_to_bfloat16", ctypes.c_int),
+    ]
+
+
+_VP = ctypes.c_void_p
+_I = ctypes.c_int
+_SZ = ctypes.c_size_t
+
+# name -> (restype, argtypes); every symbol declared in include/pluto_hip.h
+SIGNATURES = {
+    "pluto_hip_error_name": (ctypes.c_char_p, [_I]),
+    "pluto_hip_error_string": (ctypes.c_char_p, [_I]),
+    "pluto_hip_abi_version": (_I, []),
+    "pluto_hip_target_arch": (ctypes.c_char_p, []),
+    "pluto_hip_executor_create": (_I, [ctypes.POINTER(_VP)]),
+    "pluto_hip_executor_destroy": (_I, [_VP]),
+    "pluto_hip_executor_synchronize": (_I, [_VP]),
+    "pluto_hip_executor_stream": (_VP, [_VP]),
+    "pluto_hip_executor_immediate_stream": (_VP, [_VP]),
+    "pluto_hip_malloc_async": (_I, [_VP, _SZ, ctypes.POINTER(_VP)]),
+    "pluto_hip_free_async": (_I, [_VP, _VP]),
+    "pluto_hip_host_alloc": (_I, [_VP, _SZ, ctypes.POINTER(_VP)]),
+    "pluto_hip_host_free_async": (_I, [_VP, _VP]),
+    "pluto_hip_memcpy_async": (_I, [_VP, _VP, _VP, _SZ, _I]),
+    "pluto_hip_memset_async": (_I, [_VP, _VP, _I, _SZ]),
+    "pluto_hip_stream_synchronize": (_I, [_VP]),
+    "pluto_hip_cast_bf16_to_f32": (_I, [_VP, _VP, _VP, _SZ]),
+    "pluto_hip_cast_f32_to_bf16": (_I, [_VP, _VP, _VP, _SZ]),
+    "pluto_hip_mha_forward": (_I, [_VP, _I, _VP, _I, _I, _I, _I, _VP, _VP, _VP]),
+    "pluto_hip_mha_probabilities": (_I, [_VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _VP]),
+    "pluto_hip_mha_backward_workspace_bytes": (_SZ, [_I, _I, _I, _I, _I]),
+    "pluto_hip_mha_backward": (_I, [_VP, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I,
+                                    _VP, _VP, _SZ]),
+    "pluto_hip_attention_params_validate": (_I, [ctypes.POINTER(AttentionParams)]),
+    "pluto_hip_gqa_prefill_workspace_bytes": (_SZ, [ctypes.POINTER(AttentionParams), _I]),
+    "pluto_hip_gqa_prefill": (_I, [_VP, ctypes.POINTER(AttentionParams), _I, _I, _VP,
+                                   _VP, _VP, _VP, _VP, ctypes.POINTER(KvCacheView),
+                                   _VP, _VP, _VP, _SZ]),
+    "pluto_hip_gqa_decode_workspace_bytes": (_SZ, [ctypes.POINTER(AttentionParams), _I,
+                                                   ctypes.POINTER(_I), _I]),
+    "pluto_hip_gqa_decode": (_I, [_VP, ctypes.POINTER(AttentionParams), _I, _I, _VP,
+                                  _VP, _VP, _VP, _VP, ctypes.POINTER(_I),
+                                  ctypes.POINTER(KvCacheView), _VP,
+                                  ctypes.POINTER(_VP), _I, _VP, _SZ]),
+    "pluto_hip_gdn_scan_workspace_bytes": (_SZ, [ctypes.POINTER(DeltaParams), _I, _I, _I]),
+    "pluto_hip_gdn_scan": (_I, [_VP, ctypes.POINTER(DeltaParams), _I, _I, _I, _VP, _VP,
+                                _VP, _VP, _VP, _I, ctypes.c_float, _VP, _VP, _VP, _SZ]),
+    "pluto_hip_gdn_recurrence": (_I, [_VP, ctypes.POINTER(DeltaParams), _I, _I, _VP, _VP,
+                                      _VP, _VP, _VP, _I, ctypes.c_float, _VP, _VP, _I]),
+}
+
+_lib = None
+
+
+def lib():
+    """Loads libpluto_hip.so (built in-tree by pluto_amd.build) or raises."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                "%s is missing: run `python -m pluto_amd.build`" % LIB_PATH)
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (restype, argtypes) in SIGNATURES.items():
+            fn = getattr(handle, name)  # AttributeError: the build is stale
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _lib = handle
+    return _lib
+
+
+def check(code):
+    if code != 0:
+        l = lib()
+        raise PlutoHipError(code, l.pluto_hip_error_name(code).decode(),
+                            l.pluto_hip_error_string(code).decode())
+
+
+def current_stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def ptr(tensor):
+    return None if tensor is None else ctypes.c_void_p(tensor.data_ptr())
+
+
+def dtype_code(tensor):
+    if tensor.dtype == torch.bfloat16:
+        return BF16
+    if tensor.dtype == torch.float32:
+        return F32
+    raise TypeError("activations must be float32 or bfloat16")
+
+
+# ---- GPT-2 causal MHA ------------------------------------------------------
+
+def mha_forward(qkv, context_length, num_heads, stream=None):
+    """qkv [rows, 3E] (float32 or bfloat16, contiguous, on the GPU).
+    Returns (out [rows, E], maxima [rows/T*H, T], normalizers)."""
+    assert qkv.is_contiguous()
+    rows, packed = qkv.shape
+    E = packed // 3
+    out = torch.empty((rows, E), dtype=qkv.dtype, device=qkv.device)
+    stats = (max(rows // max(context_length, 1), 0) * num_heads, context_length)
+    maxima = torch.empty(stats, dtype=torch.float32, device=qkv.device)
+    normalizers = torch.empty(stats, dtype=torch.float32, device=qkv.device)
+    check(lib().pluto_hip_mha_forward(stream or current_stream(), dtype_code(qkv),
+                                      ptr(qkv), rows, context_length, num_heads, E,
+                                      ptr(out), ptr(maxima), ptr(normalizers)))
+    return out, maxima, normalizers
+
+
+def mha_probabilities(qkv, maxima, normalizers, context_length, num_heads, stream=None):
+    rows, packed = qkv.shape
+    E = packed // 3
+    probs = torch.empty((rows // context_length, num_heads, context_length, context_length),
+                        dtype=torch.float32, device=qkv.device)
+    check(lib().pluto_hip_mha_probabilities(stream or current_stream(), dtype_code(qkv),
+                                            ptr(qkv), ptr(maxima), ptr(normalizers), rows,
+                                            context_length, num_heads, E, ptr(probs)))
+    return probs
+
+
+def mha_backward_workspace(qkv, context_length, num_heads):
+    rows, packed = qkv.shape
+    size = lib().pluto_hip_mha_backward_workspace_bytes(
+        dtype_code(qkv), rows, context_length, num_heads, packed // 3)
+    return torch.empty(size, dtype=torch.uint8, device=qkv.device)
+
+
+def mha_backward(qkv, out, d_out, maxima, normalizers, context_length, num_heads,
+                 workspace=None, d_qkv=None, stream=None):
+    rows, packed = qkv.shape
+    E = packed // 3
+    if workspace is None:
+        workspace = mha_backward_workspace(qkv, context_length, num_heads)
+    if d_qkv is None:
+        d_qkv = torch.empty((rows, packed), dtype=torch.float32, device=qkv.device)
+    check(lib().pluto_hip_mha_backward(stream or current_stream(), dtype_code(qkv), ptr(qkv),
+                                       ptr(out), ptr(d_out), ptr(maxima), ptr(normalizers),
+                                       rows, context_length, num_heads, E, ptr(d_qkv),
+                                       ptr(workspace), workspace.numel()))
+    return d_qkv

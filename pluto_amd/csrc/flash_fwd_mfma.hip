@@ -1,0 +1,327 @@
+// Causal flash attention forward for bf16 activations on gfx950 matrix cores.
+//
+// One workgroup (4 wave64) owns 128 query rows of one (sequence, head); wave w
+// owns rows 32w..32w+31.  Key/value tiles of 64 rows are staged through LDS.
+// Both products are computed transposed with v_mfma_f32_32x32x16_bf16:
+//
+//   S^T[key, query] = K[key, :] . Q[query, :]      A = K (LDS), B = Q (regs)
+//   O^T[d,   query] = V^T[d, key] . P^T[key, query] A = V^T (LDS), B = P^T
+//
+// In the 32x32 accumulator layout lane l holds column (l % 32), i.e. ONE query,
+// so the softmax row statistics are per-lane scalars and need a single
+// cross-lane exchange (lane ^ 32) per tile, and the probabilities leave the
+// accumulator registers already laid out as the B operand of the second
+// product: no shuffle, no LDS round trip.  The contraction index of an MFMA
+// may be enumerated in any order as long as A and B agree, so V^T is written to
+// LDS with its keys permuted to the order in which the accumulator registers
+// hold them.
+//
+// Semantics follow FlashAttentionForwardKernel (src/llm/layers/attention.cc:
+// 98-170) and, with the gate epilogue, ForwardKernel
+// (src/llm/layers/qwen_attention.cc:68-119).  Deviation, within the stated
+// bf16 tolerance: probabilities are rounded to bf16 for the P.V product (the
+// reference keeps them FP32, attention.cc:151-156).
+#include "flash_fwd_mfma.h"
+
+#include "mfma_tile.h"
+
+namespace pluto_hip {
+namespace {
+
+constexpr int BM = 128;  // query rows per workgroup
+constexpr int BN = 64;   // keys per LDS tile
+constexpr int kThreads = 256;
+
+template <int D>
+struct Smem {
+  static constexpr int KCH = D / 8;  // 16-byte chunks per K row
+  // K tile, row major: chunk (key, ch) at key*KCH + (ch ^ (key & 7)).
+  uint4 k[BN * KCH];
+  // V^T tile: row d holds BN keys as 8 chunks of 8 keys in accumulator order;
+  // chunk c of row d at d*(BN/8) + (c ^ swizzle_d(d)).
+  uint4 vt[D * (BN / 8)];
+};
+
+template <int D>
+__global__ void __launch_bounds__(kThreads)
+flash_forward_kernel(FlashForwardArgs a) {
+  constexpr int KCH = D / 8;
+  constexpr int KS = D / 16;      // contraction steps of S^T
+  constexpr int DB = D / 32;      // 32-row blocks of O^T
+  constexpr int KB = BN / 32;     // 32-key blocks per tile
+  constexpr int OSTRIDE = D * 2 + 16;  // bytes per staged output row
+  static_assert(sizeof(Smem<D>) >= 0, "");
+  __shared__ __attribute__((aligned(16))) unsigned char raw[
+      sizeof(Smem<D>) > BM * OSTRIDE ? sizeof(Smem<D>) : BM * OSTRIDE];
+  Smem<D>& sm = *reinterpret_cast<Smem<D>*>(raw);
+
+  const int tid = threadIdx.x;
+  const int wave = tid / 64, lane = tid % 64;
+  const int h = lane / 32, n = lane % 32;
+  const int q_tiles = (a.q_rows + BM - 1) / BM;
+  // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.
+  // Renumber them so that the query tiles sharing one (sequence, kv head)
+  // K/V stream run on the same XCD.
+  const int logical = xcd_logical_block();
+  const int q_tile = q_tiles - 1 - logical % q_tiles;  // heaviest tiles first
+  const int q0 = q_tile * BM;
+  const int head = (logical / q_tiles) % a.query_heads;
+  const int seq = logical / (q_tiles * a.query_heads);
+  const int kv_head = head / a.group;
+  const int q_row = q0 + 32 * wave + n;
+
+  const uint16_t* q_base = a.q + seq * a.q_seq_stride + head * a.q_head_stride;
+  const uint16_t* k_base = a.k + seq * a.k_seq_stride + kv_head * a.k_head_stride;
+  const uint16_t* v_base = a.v + seq * a.v_seq_stride + kv_head * a.v_head_stride;
+
+  // Q fragments (B operand of S^T): row q_row, channels 16ks + 8h .. +7.
+  bf16x8 qf[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    uint4 bits = make_uint4(0, 0, 0, 0);
+    if (q_row < a.q_rows)
+      bits = *reinterpret_cast<const uint4*>(
+          q_base + static_cast<long long>(q_row) * a.q_row_stride + 16 * ks + 8 * h);
+    qf[ks] = as_bf16x8(bits);
+  }
+
+  floatx16 o_acc[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) o_acc[db][i] = 0.0f;
+  float m2 = kMasked;  // running maximum of score * scale * log2(e)
+  float l_part = 0.0f; // this lane-half's share of the normalizer
+
+  const int last_row = min(q0 + BM, a.q_rows) - 1;
+  const int visible = min(a.kv_rows, a.start_position + last_row + 1);
+  const int tiles = (visible + BN - 1) / BN;
+  const int wave_last_key = a.start_position + q0 + 32 * wave + 31;
+  const float scale2 = a.scale * kLog2e;
+
+  // Loader roles: waves 0-1 fetch K (row major), waves 2-3 fetch V and
+  // transpose it in registers.  Both move BN*D*2 bytes per tile with
+  // 16-byte loads.
+  constexpr int LOADS = BN * KCH / 128;  // 16-byte loads per loader thread
+  uint4 staged[LOADS];
+  const int ltid = tid % 128;
+  const bool loads_k = tid < 128;
+
+  auto fetch = [&](int tile) {
+    const int k0 = tile * BN;
+    if (loads_k) {
+#pragma unroll
+      for (int i = 0; i < LOADS; ++i) {
+        const int c = ltid + 128 * i;
+        const int key = c / KCH, ch = c % KCH;
+        uint4 bits = make_uint4(0, 0, 0, 0);
+        if (k0 + key < a.kv_rows)
+          bits = *reinterpret_cast<const uint4*>(
+              k_base + static_cast<long long>(k0 + key) * a.k_row_stride + 8 * ch);
+        staged[i] = bits;
+      }
+    } else {
+      // unit = (key quad, channel group); 4 loads (one per key) per unit.
+#pragma unroll
+      for (int u = 0; u < LOADS / 4; ++u) {
+        const int unit = ltid + 128 * u;
+        const int quad = unit / KCH, g = unit % KCH;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int key = k0 + 4 * quad + r;
+          uint4 bits = make_uint4(0, 0, 0, 0);
+          if (key < a.kv_rows)
+            bits = *reinterpret_cast<const uint4*>(
+                v_base + static_cast<long long>(key) * a.v_row_stride + 8 * g);
+          staged[4 * u + r] = bits;
+        }
+      }
+    }
+  };
+
+  auto commit = [&]() {
+    if (loads_k) {
+#pragma unroll
+      for (int i = 0; i < LOADS; ++i) {
+        const int c = ltid + 128 * i;
+        const int key = c / KCH, ch = c % KCH;
+        sm.k[row_major_index<KCH>(key, ch)] = staged[i];
+      }
+    } else {
+#pragma unroll
+      for (int u = 0; u < LOADS / 4; ++u) {
+        const int unit = ltid + 128 * u;
+        transposed_store<BN>(sm.vt, unit / KCH, unit % KCH, staged[4 * u + 0],
+                             staged[4 * u + 1], staged[4 * u + 2],
+                             staged[4 * u + 3]);
+      }
+    }
+  };
+
+  if (tiles > 0) fetch(0);
+  for (int tile = 0; tile < tiles; ++tile) {
+    const int k0 = tile * BN;
+    __syncthreads();  // everyone finished reading the previous tile
+    commit();
+    __syncthreads();
+    if (tile + 1 < tiles) fetch(tile + 1);
+    if (k0 > wave_last_key) continue;  // nothing visible to this wave's rows
+
+    // ---- S^T = K Q^T -------------------------------------------------
+    floatx16 s[KB];
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s[kb][i] = 0.0f;
+      if (k0 + 32 * kb > wave_last_key) continue;
+      const int key = 32 * kb + n;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const bf16x8 kf = as_bf16x8(sm.k[row_major_index<KCH>(key, 2 * ks + h)]);
+        s[kb] = mfma32(kf, qf[ks], s[kb]);
+      }
+    }
+    // ---- mask, row maximum --------------------------------------------
+    const bool needs_mask =
+        (k0 + BN - 1 > a.start_position + q0 + 32 * wave) || (k0 + BN > a.kv_rows);
+    float row_max = kMasked;
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        float t = s[kb][i] * scale2;
+        if (needs_mask) {
+          const int key = k0 + 32 * kb + 8 * (i / 4) + 4 * h + (i % 4);
+          if (key > a.start_position + q_row || key >= a.kv_rows) t = kMasked;
+        }
+        s[kb][i] = t;
+        row_max = fmaxf(row_max, t);
+      }
+    row_max = fmaxf(row_max, __shfl_xor(row_max, 32, 64));
+    const float m_new = fmaxf(m2, row_max);
+    const float alpha = __builtin_amdgcn_exp2f(m2 - m_new);
+    m2 = m_new;
+    float sum = 0.0f;
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float p = __builtin_amdgcn_exp2f(s[kb][i] - m_new);
+        s[kb][i] = p;
+        sum += p;
+      }
+    l_part = l_part * alpha + sum;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) o_acc[db][i] *= alpha;
+    // ---- O^T += V^T P^T -------------------------------------------------
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb) {
+      if (k0 + 32 * kb > wave_last_key) continue;
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {
+        const bf16x8 pf = accumulator_to_operand(s[kb], s2);
+        const int chunk = 4 * kb + 2 * s2 + h;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          const int d = 32 * db + n;
+          const bf16x8 vf = as_bf16x8(sm.vt[transposed_index<BN>(d, chunk)]);
+          o_acc[db] = mfma32(vf, pf, o_acc[db]);
+        }
+      }
+    }
+  }
+
+  // ---- epilogue ------------------------------------------------------------
+  const float l_total = l_part + __shfl_xor(l_part, 32, 64);
+  const float normalizer = l_total > 0.0f ? l_total : 1.0f;
+  const float inverse = 1.0f / normalizer;
+  __syncthreads();  // LDS is reused to transpose the output tile
+  {
+    unsigned char* row = raw + (32 * wave + n) * OSTRIDE;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int d = 32 * db + 8 * j + 4 * h;
+        bf16x4 packed;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          packed[r] = static_cast<__bf16>(o_acc[db][4 * j + r] * inverse);
+        *reinterpret_cast<bf16x4*>(row + 2 * d) = packed;
+      }
+  }
+  if (h == 0 && q_row < a.q_rows) {
+    const float maximum = m2 * (1.0f / kLog2e);
+    const long long stat =
+        (static_cast<long long>(seq) * a.query_heads + head) * a.q_rows + q_row;
+    if (a.maxima) a.maxima[stat] = maximum;
+    if (a.normalizers) a.normalizers[stat] = normalizer;
+    if (a.lse)
+      a.lse[(static_cast<long long>(seq) * a.q_rows + q_row) * a.query_heads + head] =
+          maximum + __logf(normalizer);
+  }
+  __syncthreads();
+  uint16_t* o_base = a.out + seq * a.o_seq_stride + head * a.o_head_stride;
+  const uint16_t* gate_base =
+      a.gate ? a.gate + seq * a.gate_seq_stride + head * a.gate_head_stride : nullptr;
+  for (int c = tid; c < BM * KCH; c += kThreads) {
+    const int r = c / KCH, ch = c % KCH;
+    const int row = q0 + r;
+    if (row >= a.q_rows) continue;
+    uint4 bits = *reinterpret_cast<const uint4*>(raw + r * OSTRIDE + 16 * ch);
+    if (gate_base) {
+      // out = bf16(bf16(core) * bf16(sigmoid(gate))): qwen_attention.cc:103-108
+      const uint4 gate_bits = *reinterpret_cast<const uint4*>(
+          gate_base + static_cast<long long>(row) * a.gate_row_stride + 8 * ch);
+      const uint16_t* core = reinterpret_cast<const uint16_t*>(&bits);
+      const uint16_t* gate = reinterpret_cast<const uint16_t*>(&gate_bits);
+      uint16_t result[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float sigmoid = 1.0f / (1.0f + expf(-bf16_bits_to_float(gate[e])));
+        result[e] = float_to_bf16_bits(bf16_bits_to_float(core[e]) *
+                                       round_to_bf16(sigmoid));
+      }
+      bits = *reinterpret_cast<const uint4*>(result);
+    }
+    *reinterpret_cast<uint4*>(o_base + static_cast<long long>(row) * a.o_row_stride +
+                              8 * ch) = bits;
+  }
+}
+
+}  // namespace
+
+bool flash_forward_supported(const FlashForwardArgs& a, int head_dim) {
+  if (head_dim != 64 && head_dim != 128) return false;
+  auto aligned = [](const void* p) {
+    return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+  };
+  auto mult8 = [](long long s) { return (s % 8) == 0; };
+  if (!aligned(a.q) || !aligned(a.k) || !aligned(a.v) || !aligned(a.out))
+    return false;
+  if (a.gate && !aligned(a.gate)) return false;
+  return mult8(a.q_seq_stride) && mult8(a.q_row_stride) && mult8(a.q_head_stride) &&
+         mult8(a.k_seq_stride) && mult8(a.k_row_stride) && mult8(a.k_head_stride) &&
+         mult8(a.v_seq_stride) && mult8(a.v_row_stride) && mult8(a.v_head_stride) &&
+         mult8(a.o_seq_stride) && mult8(a.o_row_stride) && mult8(a.o_head_stride) &&
+         mult8(a.gate_seq_stride) && mult8(a.gate_row_stride) &&
+         mult8(a.gate_head_stride);
+}
+
+int launch_flash_forward(hipStream_t stream, const FlashForwardArgs& a,
+                         int head_dim, int sequences) {
+  if (!flash_forward_supported(a, head_dim)) return PLUTO_HIP_EUNSUPPORTED;
+  const long long blocks =
+      static_cast<long long>((a.q_rows + BM - 1) / BM) * a.query_heads * sequences;
+  if (blocks <= 0 || blocks > 0x7fffffffLL) return PLUTO_HIP_EINVAL;
+  dim3 grid(static_cast<unsigned>(blocks));
+  if (head_dim == 64)
+    flash_forward_kernel<64><<<grid, kThreads, 0, stream>>>(a);
+  else
+    flash_forward_kernel<128><<<grid, kThreads, 0, stream>>>(a);
+  return launch_status();
+}
+
+}  // namespace pluto_hip

@@ -1,0 +1,235 @@
+"""GPU parity of GPT-2 style causal attention (forward, backward, statistics)
+against the CPU oracle, through the C ABI.  Shapes and invariants follow the
+reference's attention_reference_test.cc / attention_test.cc."""
+import math
+import os
+
+import numpy as np
+import pytest
+
+from tests.util import assert_close, from_bf16_bits, to_bf16_bits
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+FP32_REL = 1e-4   # stated tolerance for FP32 storage
+BF16_REL = 2e-2   # stated tolerance for bf16 storage
+
+
+@pytest.fixture(scope="module")
+def capi():
+    from pluto_amd import capi
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    capi.lib()
+    return capi
+
+
+def device_inputs(x, d_out, bf16):
+    xt = torch.from_numpy(x).cuda()
+    if bf16:
+        xt = xt.to(torch.bfloat16)
+    return xt, torch.from_numpy(d_out).cuda()
+
+
+def run_device(capi, x, d_out, T, H, bf16):
+    xt, gt = device_inputs(x, d_out, bf16)
+    out, maxima, normalizers = capi.mha_forward(xt, T, H)
+    d_qkv = capi.mha_backward(xt, out, gt, maxima, normalizers, T, H)
+    torch.cuda.synchronize()
+    return (out.float().cpu().numpy(), maxima.cpu().numpy(), normalizers.cpu().numpy(),
+            d_qkv.cpu().numpy())
+
+
+def run_oracle(oracle, x, d_out, T, H, bf16, seqs=None, heads=None):
+    if bf16:
+        bits = to_bf16_bits(oracle, x)
+        out_bits, maxima, normalizers = oracle.mha_fwd(bits, T, H, oracle.BF16, seqs, heads)
+        d_qkv = oracle.mha_bwd(bits, out_bits, d_out, T, H, oracle.BF16, seqs, heads)
+        return from_bf16_bits(oracle, out_bits), maxima, normalizers, d_qkv
+    out, maxima, normalizers = oracle.mha_fwd(x, T, H, oracle.F32, seqs, heads)
+    d_qkv = oracle.mha_bwd(x, out, d_out, T, H, oracle.F32, seqs, heads)
+    return out, maxima, normalizers, d_qkv
+
+
+def check(capi, oracle, T, H, E, B, bf16, seed, qk_scale=1.0):
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((B * T, 3 * E)).astype(np.float32)
+    x[:, :2 * E] *= qk_scale
+    d_out = rng.standard_normal((B * T, E)).astype(np.float32)
+    got = run_device(capi, x, d_out, T, H, bf16)
+    want = run_oracle(oracle, x, d_out, T, H, bf16)
+    rel = BF16_REL if bf16 else FP32_REL
+    if qk_scale > 1 and not bf16:
+        rel = 2e-3  # peaked scores: the reference's own tolerance (attention_reference_test.cc:56-73)
+    tag = "T%d H%d E%d B%d %s" % (T, H, E, B, "bf16" if bf16 else "fp32")
+    assert_close(got[0], want[0], rel, tag + " out")
+    lse_got = got[1] + np.log(got[2])
+    lse_want = want[1] + np.log(want[2])
+    assert_close(lse_got, lse_want, 1e-4 if not bf16 else 1e-3, tag + " lse")
+    assert_close(got[3], want[3], rel if not bf16 else BF16_REL, tag + " d_qkv")
+
+
+# attention_reference_test.cc:148-160
+SHAPES = [(1, 1, 16, 3), (4, 1, 16, 2), (4, 2, 32, 2), (8, 2, 32, 1), (33, 2, 64, 2),
+          (33, 2, 128, 2), (65, 2, 64, 2), (65, 2, 128, 2), (65, 2, 160, 2),
+          (65, 2, 192, 2), (65, 2, 256, 2)]
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("T,H,E,B", SHAPES)
+def test_matches_oracle_across_configurations(capi, oracle, T, H, E, B, bf16):
+    check(capi, oracle, T, H, E, B, bf16, seed=T * 7 + E)
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+def test_peaked_scores(capi, oracle, bf16):
+    check(capi, oracle, 65, 1, 64, 2, bf16, seed=5, qk_scale=20.0 if not bf16 else 4.0)
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("width", [1, 3, 7, 8, 15, 24, 33])
+def test_sub_tile_head_widths(capi, oracle, width, bf16):
+    check(capi, oracle, 33, 1, width, 2, bf16, seed=width)
+
+
+def test_three_odd_heads(capi, oracle):
+    check(capi, oracle, 65, 3, 21, 2, False, seed=1)
+    check(capi, oracle, 65, 3, 96, 2, True, seed=2, qk_scale=2.0)
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+def test_production_context_one_head(capi, oracle, bf16):
+    # attention_reference_test.cc:171-176: T=1024, one 64-wide head
+    check(capi, oracle, 1024, 1, 64, 1, bf16, seed=9)
+
+
+def test_mfma_heads_of_128(capi, oracle):
+    check(capi, oracle, 300, 2, 256, 2, True, seed=12)
+
+
+def test_closed_form_two_tokens(capi):
+    # attention_test.cc:282-360
+    T, H, E, rows = 4, 2, 32, 32
+    x = np.zeros((rows, 3 * E), np.float32)
+    x[0, 0] = 1; x[0, E] = 1; x[0, 2 * E] = 1
+    x[1, 0] = 2; x[1, E] = 2; x[1, 2 * E] = 2
+    x[2, 2 * E] = 4
+    d_out = np.zeros((rows, E), np.float32)
+    d_out[0, 0] = 1
+    out, _, _, g = run_device(capi, x, d_out, T, H, False)
+    scale = 1 / math.sqrt(E // H)
+    w1, w2 = math.exp(2 * scale), math.exp(4 * scale)
+    assert abs(out[0, 0] - 1.0) <= 1e-6
+    assert abs(out[1, 0] - (w1 + 2 * w2) / (w1 + w2)) <= 1e-5
+    assert abs(g[0, 0]) <= 1e-6 and abs(g[0, E]) <= 1e-6
+    assert abs(g[0, 2 * E] - 1.0) <= 1e-6
+    assert abs(g[1, 0]) <= 1e-6
+
+
+@pytest.mark.parametrize("bf16,T,E,H", [(False, 65, 128, 2), (True, 65, 128, 2), (True, 300, 128, 2)])
+def test_future_tokens_and_other_sequences_cannot_matter(capi, bf16, T, E, H):
+    # attention_reference_test.cc:207-308: exact equality
+    B = 2
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal((B * T, 3 * E)).astype(np.float32)
+    d_out = rng.standard_normal((B * T, E)).astype(np.float32)
+    cut = T * 2 // 3
+    d_out[cut:] = 0
+    y = x.copy()
+    y[cut:T] = rng.standard_normal((T - cut, 3 * E))
+    y[T:] = rng.standard_normal((T, 3 * E))
+    a = run_device(capi, x, d_out, T, H, bf16)
+    b = run_device(capi, y, d_out, T, H, bf16)
+    np.testing.assert_array_equal(a[0][:cut], b[0][:cut])
+    np.testing.assert_array_equal(a[3][:cut], b[3][:cut])
+    assert np.all(b[3][T:] == 0)
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+def test_bitwise_repeatable(capi, bf16):
+    # attention_test.cc:362-475
+    T, H, E, B = 200, 3, 192, 2
+    rng = np.random.default_rng(21)
+    x = rng.standard_normal((B * T, 3 * E)).astype(np.float32)
+    d_out = rng.standard_normal((B * T, E)).astype(np.float32)
+    first = run_device(capi, x, d_out, T, H, bf16)
+    for _ in range(4):
+        again = run_device(capi, x, d_out, T, H, bf16)
+        for a, b in zip(first, again):
+            np.testing.assert_array_equal(a, b)
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+def test_probabilities_pass(capi, bf16):
+    # attention_test.cc:41-146: rows sum to one, zeros above the diagonal, P.V = out
+    T, H, E, B = 70, 2, 64, 2
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((B * T, 3 * E)).astype(np.float32)
+    xt, _ = device_inputs(x, np.zeros((B * T, E), np.float32), bf16)
+    out, maxima, normalizers = capi.mha_forward(xt, T, H)
+    probs = capi.mha_probabilities(xt, maxima, normalizers, T, H).cpu().numpy()
+    assert np.all(np.triu(probs, 1) == 0)
+    np.testing.assert_allclose(probs.sum(-1), 1.0, atol=3e-5 if not bf16 else 2e-3)
+    xv = xt.float().cpu().numpy().reshape(B, T, 3, H, E // H)
+    pv = np.einsum("bhts,bshd->bthd", probs, xv[:, :, 2]).reshape(B * T, E)
+    np.testing.assert_allclose(out.float().cpu().numpy(), pv, atol=5e-3 if bf16 else 3e-5)
+
+
+def test_config1_gpt2_small_forward_fp32(capi, oracle):
+    # B=4, T=256, H=12, D=64, fp32 storage, N(0,1), seed 0
+    T, H, E, B = 256, 12, 768, 4
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((B * T, 3 * E)).astype(np.float32)
+    xt = torch.from_numpy(x).cuda()
+    out, maxima, normalizers = capi.mha_forward(xt, T, H)
+    want, wm, wn = oracle.mha_fwd(x, T, H)
+    assert_close(out.cpu().numpy(), want, FP32_REL, "config 1 out")
+    assert_close((maxima + normalizers.log()).cpu().numpy(), wm + np.log(wn), 1e-4, "config 1 lse")
+
+
+def test_config2_gpt2_small_forward_backward_bf16(capi, oracle):
+    # B=16, T=1024, H=12, D=64, bf16 storage, N(0,1), seed 1.  The oracle is run
+    # on whole (sequence, head) units (they are independent); the rest of the
+    # tensor is checked against the any-shape FP32-arithmetic kernels.
+    T, H, E, B = 1024, 12, 768, 16
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((B * T, 3 * E)).astype(np.float32)
+    d_out = rng.standard_normal((B * T, E)).astype(np.float32)
+    xt, gt = device_inputs(x, d_out, True)
+    out, maxima, normalizers = capi.mha_forward(xt, T, H)
+    d_qkv = capi.mha_backward(xt, out, gt, maxima, normalizers, T, H)
+    D = E // H
+    units = [(0, 0), (7, 5), (15, 11)]
+    bits = to_bf16_bits(oracle, x)
+    for seq, head in units:
+        o_bits, wm, wn = oracle.mha_fwd(bits, T, H, oracle.BF16, (seq, seq + 1), (head, head + 1))
+        want_g = oracle.mha_bwd(bits, o_bits, d_out, T, H, oracle.BF16, (seq, seq + 1), (head, head + 1))
+        rows = slice(seq * T, (seq + 1) * T)
+        cols = slice(head * D, (head + 1) * D)
+        tag = "config 2 seq %d head %d " % (seq, head)
+        assert_close(out[rows, cols].float().cpu().numpy(), from_bf16_bits(oracle, o_bits)[rows, cols], BF16_REL, tag + "out")
+        stat = seq * H + head
+        assert_close((maxima[stat] + normalizers[stat].log()).cpu().numpy(), wm[stat] + np.log(wn[stat]), 1e-3, tag + "lse")
+        g = d_qkv[rows].cpu().numpy()
+        for part, name in ((0, "dQ"), (1, "dK"), (2, "dV")):
+            c = slice(part * E + head * D, part * E + (head + 1) * D)
+            assert_close(g[:, c], want_g[rows, c], BF16_REL, tag + name)
+    os.environ["PLUTO_HIP_FORCE_GENERIC"] = "1"
+    try:
+        out2, m2, n2 = capi.mha_forward(xt, T, H)
+        d2 = capi.mha_backward(xt, out2, gt, m2, n2, T, H)
+        torch.cuda.synchronize()
+    finally:
+        del os.environ["PLUTO_HIP_FORCE_GENERIC"]
+    assert_close(out.float().cpu().numpy(), out2.float().cpu().numpy(), BF16_REL, "config 2 out vs fp32-arithmetic kernel")
+    assert_close(d_qkv.cpu().numpy(), d2.cpu().numpy(), BF16_REL, "config 2 d_qkv vs fp32-arithmetic kernel")
+
+
+def test_rejects_bad_arguments_before_any_work(capi):
+    # attention_test.cc:549-626
+    x = torch.zeros((6, 12), device="cuda")
+    for T, H in ((4, 2), (3, 3), (0, 2), (3, 0)):
+        with pytest.raises(capi.PlutoHipError) as info:
+            capi.mha_forward(x, T, H)
+        assert info.value.code == capi.EINVAL
