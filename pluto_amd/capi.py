@@ -198,3 +198,99 @@ def mha_backward(qkv, out, d_out, maxima, normalizers, context_length, num_heads
                                        rows, context_length, num_heads, E, ptr(d_qkv),
                                        ptr(workspace), workspace.numel()))
     return d_qkv
+
+
+# ---- Qwen grouped-query attention -------------------------------------------
+
+def attention_params(query_heads=24, key_value_heads=4, head_dim=256, rotary_dim=64,
+                     capacity=4096, rms_norm_epsilon=1e-6, rope_theta=10000000.0,
+                     round_to_bfloat16=True):
+    return AttentionParams(query_heads, key_value_heads, head_dim, rotary_dim, capacity,
+                           rms_norm_epsilon, rope_theta, int(bool(round_to_bfloat16)))
+
+
+class KvCache:
+    """One sequence's K and V storage plus the view handed to the C ABI.
+
+    layout "head_major": [kv_heads, capacity, head_dim] (native, bf16 by default);
+    layout "token_major": [capacity, kv_heads, head_dim] (the reference's layout)."""
+
+    def __init__(self, capacity, kv_heads, head_dim, dtype=torch.bfloat16,
+                 layout="head_major", device="cuda", fill=None):
+        shape = ((kv_heads, capacity, head_dim) if layout == "head_major"
+                 else (capacity, kv_heads, head_dim))
+        self.keys = torch.empty(shape, dtype=dtype, device=device)
+        self.values = torch.empty(shape, dtype=dtype, device=device)
+        if fill is not None:
+            self.keys.fill_(fill)
+            self.values.fill_(fill)
+        self.layout = layout
+        self.capacity, self.kv_heads, self.head_dim = capacity, kv_heads, head_dim
+        self.position = 0
+
+    def view(self):
+        if self.layout == "head_major":
+            token_stride, head_stride = self.head_dim, self.capacity * self.head_dim
+        else:
+            token_stride, head_stride = self.kv_heads * self.head_dim, self.head_dim
+        return KvCacheView(self.keys.data_ptr(), self.values.data_ptr(),
+                           dtype_code(self.keys), token_stride, head_stride)
+
+    def token_major(self, tensor):
+        """[capacity, kv_heads, head_dim] float32 copy on the host."""
+        t = tensor.float().cpu()
+        return (t.permute(1, 0, 2) if self.layout == "head_major" else t).contiguous().numpy()
+
+
+def gqa_prefill(p, qg, k, v, q_norm, k_norm, cache, start_position=0, want_lse=False,
+                stream=None):
+    """qg bf16 [T, qh, 2, d]; k, v bf16 [T, kh, d]; norms fp32 [d]."""
+    T = qg.shape[0]
+    out = torch.empty((T, p.query_heads, p.head_dim), dtype=torch.bfloat16, device=qg.device)
+    lse = (torch.empty((T, p.query_heads), dtype=torch.float32, device=qg.device)
+           if want_lse else None)
+    size = lib().pluto_hip_gqa_prefill_workspace_bytes(ctypes.byref(p), T)
+    workspace = torch.empty(max(size, 1), dtype=torch.uint8, device=qg.device)
+    view = cache.view()
+    check(lib().pluto_hip_gqa_prefill(stream or current_stream(), ctypes.byref(p), T,
+                                      start_position, ptr(qg), ptr(k), ptr(v), ptr(q_norm),
+                                      ptr(k_norm), ctypes.byref(view), ptr(out), ptr(lse),
+                                      ptr(workspace), size))
+    cache.position = start_position + T
+    return (out, lse) if want_lse else out
+
+
+def gqa_decode_workspace(p, positions, split_tokens=0, device="cuda"):
+    batch = len(positions)
+    pos = (ctypes.c_int * batch)(*positions)
+    size = lib().pluto_hip_gqa_decode_workspace_bytes(ctypes.byref(p), batch, pos, split_tokens)
+    return torch.empty(max(size, 1), dtype=torch.uint8, device=device)
+
+
+def gqa_decode(p, q_gate, k, v, q_norm, k_norm, caches, positions=None, split_tokens=0,
+               probabilities=None, workspace=None, out=None, advance=True, stream=None):
+    """q_gate [batch, qh, 2, d]; k, v [batch, kh, d] (float32 or bfloat16);
+    caches: list of KvCache.  positions default to the caches' own counters,
+    which are advanced after a successful call."""
+    batch = q_gate.shape[0]
+    if positions is None:
+        positions = [c.position for c in caches]
+    pos = (ctypes.c_int * batch)(*positions)
+    views = (KvCacheView * batch)(*[c.view() for c in caches])
+    if workspace is None:
+        workspace = gqa_decode_workspace(p, positions, split_tokens, q_gate.device)
+    if out is None:
+        out = torch.empty((batch, p.query_heads, p.head_dim), dtype=q_gate.dtype,
+                          device=q_gate.device)
+    probs = None
+    if probabilities is not None:
+        probs = (ctypes.c_void_p * batch)(*[None if t is None else t.data_ptr()
+                                             for t in probabilities])
+    check(lib().pluto_hip_gqa_decode(stream or current_stream(), ctypes.byref(p), batch,
+                                     dtype_code(q_gate), ptr(q_gate), ptr(k), ptr(v),
+                                     ptr(q_norm), ptr(k_norm), pos, views, ptr(out), probs,
+                                     split_tokens, ptr(workspace), workspace.numel()))
+    if advance:
+        for c in caches:
+            c.position += 1
+    return out

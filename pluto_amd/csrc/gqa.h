@@ -1,0 +1,105 @@
+// Argument blocks and launchers of the Qwen grouped-query attention kernels.
+#pragma once
+
+#include "common.h"
+
+namespace pluto_hip {
+
+constexpr int kDecodeBatchMax = 64;  // sequences per decode launch
+
+struct CacheView {
+  void* keys = nullptr;
+  void* values = nullptr;
+  int dtype = PLUTO_HIP_BF16;
+  long long token_stride = 0;
+  long long head_stride = 0;
+};
+
+struct PrefillPrepareArgs {
+  const void* qg = nullptr;  // bf16 [T, qh, 2, d]
+  const void* k = nullptr;   // bf16 [T, kh, d]
+  const void* v = nullptr;   // bf16 [T, kh, d]
+  const float* q_norm = nullptr;
+  const float* k_norm = nullptr;
+  const float* cosines = nullptr;  // [T, rotary/2]
+  const float* sines = nullptr;
+  void* q_out = nullptr;  // [T, qh, d], bf16 when rounding, else fp32
+  int q_out_dtype = PLUTO_HIP_BF16;
+  CacheView cache;
+  int length = 0, start_position = 0;
+  int query_heads = 0, key_value_heads = 0, head_dim = 0, rotary_dim = 0;
+  float epsilon = 1e-6f;
+  bool round = true;
+};
+
+// Per-launch slice of a decode batch, passed by value as a kernel argument.
+struct DecodeBatch {
+  int first = 0;  // index of the slice's first sequence in the full batch
+  int count = 0;
+  int positions[kDecodeBatchMax];
+  void* keys[kDecodeBatchMax];
+  void* values[kDecodeBatchMax];
+  int block_start[kDecodeBatchMax + 1];  // prefix sum of split-K blocks
+};
+
+struct DecodePrepareArgs {
+  const void* q_gate = nullptr;  // [batch, qh, 2, d]
+  const void* k = nullptr;       // [batch, kh, d]
+  const void* v = nullptr;
+  int io_dtype = PLUTO_HIP_F32;
+  const float* q_norm = nullptr;
+  const float* k_norm = nullptr;
+  void* q_out = nullptr;  // [batch, qh, d]
+  int q_out_dtype = PLUTO_HIP_BF16;
+  int cache_dtype = PLUTO_HIP_BF16;
+  long long token_stride = 0, head_stride = 0;
+  int query_heads = 0, key_value_heads = 0, head_dim = 0, rotary_dim = 0;
+  float epsilon = 1e-6f, theta = 1e7f;
+  bool round = true;
+};
+
+struct DecodeArgs {
+  const uint16_t* q = nullptr;  // prepared queries, bf16 [batch, qh, d]
+  long long token_stride = 0, head_stride = 0;
+  int query_heads = 0, key_value_heads = 0, head_dim = 0;
+  int split_tokens = 512;
+  float scale = 1.0f;
+  // partial results of split-K block i (global index block_start[b] + j,
+  // kv head g): o [block, kh, group, d], m and l [block, kh, group]
+  float* part_o = nullptr;
+  float* part_m = nullptr;
+  float* part_l = nullptr;
+  long long block_base = 0;  // global index of this launch's first block
+};
+
+struct DecodeCombineArgs {
+  const float* part_o = nullptr;
+  const float* part_m = nullptr;
+  const float* part_l = nullptr;
+  long long block_base = 0;
+  const void* q_gate = nullptr;  // gate logits at [batch, qh, 1, :]
+  void* out = nullptr;           // [batch, qh, d]
+  int io_dtype = PLUTO_HIP_F32;
+  int query_heads = 0, key_value_heads = 0, head_dim = 0;
+  bool round = true;
+};
+
+int launch_rope_table(hipStream_t stream, int start_position, int length,
+                      int rotary_dim, float theta, bool round, float* cosines,
+                      float* sines);
+int launch_prefill_prepare(hipStream_t stream, const PrefillPrepareArgs& args);
+int launch_decode_prepare(hipStream_t stream, const DecodePrepareArgs& args,
+                          const DecodeBatch& batch);
+bool decode_fast_supported(int head_dim, int group);
+int launch_decode_fast(hipStream_t stream, const DecodeArgs& args,
+                       const DecodeBatch& batch);
+int launch_decode_combine(hipStream_t stream, const DecodeCombineArgs& args,
+                          const DecodeBatch& batch);
+// Two-pass probability row of one sequence (any dtype, any shape):
+// AttentionProbabilitiesKernel, cached_attention_ops.cc:131-178.
+int launch_decode_probabilities(hipStream_t stream, const void* q, int q_dtype,
+                                const CacheView& cache, int query_heads,
+                                int key_value_heads, int head_dim, int length,
+                                float scale, float* probabilities);
+
+}  // namespace pluto_hip

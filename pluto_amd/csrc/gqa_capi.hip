@@ -1,0 +1,353 @@
+// C ABI of Qwen grouped-query attention: validation, workspace carving and
+// kernel selection for whole-sequence prefill and batched single-token decode.
+#include <cmath>
+#include <limits>
+
+#include "attn_generic.h"
+#include "flash_fwd_mfma.h"
+#include "gqa.h"
+
+namespace pluto_hip {
+bool force_generic();  // mha_capi.hip
+namespace {
+
+// ValidateCachedAttention, parameter part (cached_attention_ops.cc:286-297).
+int validate_params(const pluto_hip_attention_params* p) {
+  if (!p) return PLUTO_HIP_EINVAL;
+  const int int_max = std::numeric_limits<int>::max();
+  if (p->query_heads <= 0 || p->key_value_heads <= 0 ||
+      p->query_heads % p->key_value_heads != 0 || p->head_dim <= 0 ||
+      p->head_dim > 256 || p->rotary_dim <= 0 || p->rotary_dim > p->head_dim ||
+      p->rotary_dim % 2 != 0 || p->capacity <= 0 || p->capacity > int_max - 32 ||
+      !std::isfinite(p->rope_theta) || p->rope_theta <= 0.0f ||
+      !std::isfinite(p->rms_norm_epsilon) || p->rms_norm_epsilon <= 0.0f ||
+      p->query_heads > int_max / (2 * p->head_dim) ||
+      p->query_heads > int_max - p->key_value_heads)
+    return PLUTO_HIP_EINVAL;
+  return 0;
+}
+
+int validate_cache(const pluto_hip_kv_cache_view* c, const pluto_hip_attention_params* p) {
+  if (!c || !c->keys || !c->values) return PLUTO_HIP_EINVAL;
+  if (c->dtype != PLUTO_HIP_F32 && c->dtype != PLUTO_HIP_BF16) return PLUTO_HIP_EINVAL;
+  if (c->token_stride < p->head_dim && c->head_stride < p->head_dim) return PLUTO_HIP_EINVAL;
+  if (c->token_stride <= 0 || c->head_stride <= 0) return PLUTO_HIP_EINVAL;
+  return 0;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+size_t element_bytes(int dtype) { return dtype == PLUTO_HIP_BF16 ? 2 : 4; }
+
+struct PrefillLayout {
+  size_t cosines, sines, queries, total;
+};
+
+PrefillLayout prefill_layout(const pluto_hip_attention_params* p, int length) {
+  PrefillLayout l{};
+  const size_t table = align_up(static_cast<size_t>(length) * (p->rotary_dim / 2) * 4, 256);
+  l.cosines = 0;
+  l.sines = table;
+  l.queries = 2 * table;
+  l.total = l.queries + align_up(static_cast<size_t>(length) * p->query_heads * p->head_dim *
+                                     (p->round_to_bfloat16 ? 2 : 4),
+                                 256);
+  return l;
+}
+
+int split_or_default(int split_tokens) { return split_tokens == 0 ? 512 : split_tokens; }
+
+long long decode_blocks(int batch, const int* positions, int split) {
+  long long blocks = 0;
+  for (int b = 0; b < batch; ++b) blocks += (static_cast<long long>(positions[b]) + split) / split;
+  return blocks;
+}
+
+}  // namespace
+}  // namespace pluto_hip
+
+using namespace pluto_hip;
+
+extern "C" {
+
+int pluto_hip_attention_params_validate(const pluto_hip_attention_params* p) {
+  return validate_params(p);
+}
+
+size_t pluto_hip_gqa_prefill_workspace_bytes(const pluto_hip_attention_params* p, int length) {
+  if (validate_params(p) != 0 || length <= 0) return 0;
+  return prefill_layout(p, length).total;
+}
+
+int pluto_hip_gqa_prefill(void* stream, const pluto_hip_attention_params* p, int length,
+                          int start_position, const void* qg, const void* k, const void* v,
+                          const float* q_norm, const float* k_norm,
+                          const pluto_hip_kv_cache_view* cache, void* out, float* lse,
+                          void* workspace, size_t workspace_bytes) {
+  int status = validate_params(p);
+  if (status != 0) return status;
+  if (length <= 0 || start_position < 0) return PLUTO_HIP_EINVAL;
+  if (!qg || !k || !v || !q_norm || !k_norm || !out) return PLUTO_HIP_EINVAL;
+  status = validate_cache(cache, p);
+  if (status != 0) return status;
+  // cached_attention_ops.cc:318-320: appending beyond capacity fails first.
+  if (static_cast<long long>(start_position) + length > p->capacity) return PLUTO_HIP_ERANGE;
+  const PrefillLayout layout = prefill_layout(p, length);
+  if (!workspace || workspace_bytes < layout.total) return PLUTO_HIP_EWORKSPACE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  char* scratch = static_cast<char*>(workspace);
+  float* cosines = reinterpret_cast<float*>(scratch + layout.cosines);
+  float* sines = reinterpret_cast<float*>(scratch + layout.sines);
+  void* queries = scratch + layout.queries;
+  const bool round = p->round_to_bfloat16 != 0;
+  const int qh = p->query_heads, kh = p->key_value_heads, d = p->head_dim;
+
+  status = launch_rope_table(s, start_position, length, p->rotary_dim, p->rope_theta, round,
+                             cosines, sines);
+  if (status != 0) return status;
+  PrefillPrepareArgs prep;
+  prep.qg = qg;
+  prep.k = k;
+  prep.v = v;
+  prep.q_norm = q_norm;
+  prep.k_norm = k_norm;
+  prep.cosines = cosines;
+  prep.sines = sines;
+  prep.q_out = queries;
+  prep.q_out_dtype = round ? PLUTO_HIP_BF16 : PLUTO_HIP_F32;
+  prep.cache = {cache->keys, cache->values, cache->dtype, cache->token_stride,
+                cache->head_stride};
+  prep.length = length;
+  prep.start_position = start_position;
+  prep.query_heads = qh;
+  prep.key_value_heads = kh;
+  prep.head_dim = d;
+  prep.rotary_dim = p->rotary_dim;
+  prep.epsilon = p->rms_norm_epsilon;
+  prep.round = round;
+  status = launch_prefill_prepare(s, prep);
+  if (status != 0) return status;
+
+  const float scale = 1.0f / std::sqrt(static_cast<float>(d));
+  const uint16_t* gate = static_cast<const uint16_t*>(qg) + d;
+  if (round && cache->dtype == PLUTO_HIP_BF16 && !force_generic()) {
+    FlashForwardArgs f;
+    f.q = static_cast<const uint16_t*>(queries);
+    f.q_row_stride = 1LL * qh * d;
+    f.q_head_stride = d;
+    f.k = static_cast<const uint16_t*>(cache->keys);
+    f.v = static_cast<const uint16_t*>(cache->values);
+    f.k_row_stride = f.v_row_stride = cache->token_stride;
+    f.k_head_stride = f.v_head_stride = cache->head_stride;
+    f.out = static_cast<uint16_t*>(out);
+    f.o_row_stride = 1LL * qh * d;
+    f.o_head_stride = d;
+    f.gate = gate;
+    f.gate_row_stride = 2LL * qh * d;
+    f.gate_head_stride = 2LL * d;
+    f.lse = lse;
+    f.q_rows = length;
+    f.kv_rows = start_position + length;
+    f.start_position = start_position;
+    f.query_heads = qh;
+    f.group = qh / kh;
+    f.scale = scale;
+    if (flash_forward_supported(f, d)) return launch_flash_forward(s, f, d, 1);
+  }
+  GenericForwardArgs a;
+  a.q = {queries, 0, 1LL * qh * d, d, prep.q_out_dtype};
+  a.k = {cache->keys, 0, cache->token_stride, cache->head_stride, cache->dtype};
+  a.v = {cache->values, 0, cache->token_stride, cache->head_stride, cache->dtype};
+  a.gate = {gate, 0, 2LL * qh * d, 2LL * d, PLUTO_HIP_BF16};
+  a.out = out;
+  a.o_row_stride = 1LL * qh * d;
+  a.o_head_stride = d;
+  a.o_dtype = PLUTO_HIP_BF16;
+  a.lse = lse;
+  a.q_rows = length;
+  a.kv_rows = start_position + length;
+  a.start_position = start_position;
+  a.query_heads = qh;
+  a.group = qh / kh;
+  a.head_dim = d;
+  a.scale = scale;
+  a.round_to_bf16 = round;
+  return launch_generic_forward(s, a, 1);
+}
+
+size_t pluto_hip_gqa_decode_workspace_bytes(const pluto_hip_attention_params* p, int batch,
+                                            const int* positions, int split_tokens) {
+  if (validate_params(p) != 0 || batch <= 0 || !positions) return 0;
+  const int split = split_or_default(split_tokens);
+  if (split < 64 || split > 512 || split % 64 != 0) return 0;
+  for (int b = 0; b < batch; ++b)
+    if (positions[b] < 0) return 0;
+  const long long blocks = decode_blocks(batch, positions, split);
+  const size_t heads = static_cast<size_t>(p->query_heads);
+  size_t bytes = align_up(static_cast<size_t>(batch) * heads * p->head_dim * 4, 256);
+  bytes += align_up(static_cast<size_t>(blocks) * heads * p->head_dim * 4, 256);
+  bytes += 2 * align_up(static_cast<size_t>(blocks) * heads * 4, 256);
+  return bytes;
+}
+
+int pluto_hip_gqa_decode(void* stream, const pluto_hip_attention_params* p, int batch,
+                         int io_dtype, const void* q_gate, const void* k, const void* v,
+                         const float* q_norm, const float* k_norm, const int* positions,
+                         const pluto_hip_kv_cache_view* caches, void* out,
+                         float* const* probabilities, int split_tokens, void* workspace,
+                         size_t workspace_bytes) {
+  int status = validate_params(p);
+  if (status != 0) return status;
+  if (batch <= 0 || (io_dtype != PLUTO_HIP_F32 && io_dtype != PLUTO_HIP_BF16))
+    return PLUTO_HIP_EINVAL;
+  // cached_attention_ops.cc:314-317: null pointers are rejected before any work.
+  if (!q_gate || !k || !v || !q_norm || !k_norm || !out || !positions || !caches)
+    return PLUTO_HIP_EINVAL;
+  const int split = split_or_default(split_tokens);
+  if (split < 64 || split > 512 || split % 64 != 0) return PLUTO_HIP_EINVAL;
+  for (int b = 0; b < batch; ++b) {
+    status = validate_cache(&caches[b], p);
+    if (status != 0) return status;
+    if (caches[b].dtype != caches[0].dtype || caches[b].token_stride != caches[0].token_stride ||
+        caches[b].head_stride != caches[0].head_stride)
+      return PLUTO_HIP_EINVAL;
+    if (positions[b] < 0) return PLUTO_HIP_EINVAL;
+  }
+  for (int b = 0; b < batch; ++b)  // cached_attention_ops.cc:318-320
+    if (positions[b] >= p->capacity) return PLUTO_HIP_ERANGE;
+  const size_t needed = pluto_hip_gqa_decode_workspace_bytes(p, batch, positions, split);
+  if (!workspace || workspace_bytes < needed) return PLUTO_HIP_EWORKSPACE;
+
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int qh = p->query_heads, kh = p->key_value_heads, d = p->head_dim;
+  const int group = qh / kh;
+  const bool round = p->round_to_bfloat16 != 0;
+  const long long blocks = decode_blocks(batch, positions, split);
+  char* scratch = static_cast<char*>(workspace);
+  void* queries = scratch;
+  size_t offset = align_up(static_cast<size_t>(batch) * qh * d * 4, 256);
+  float* part_o = reinterpret_cast<float*>(scratch + offset);
+  offset += align_up(static_cast<size_t>(blocks) * qh * d * 4, 256);
+  float* part_m = reinterpret_cast<float*>(scratch + offset);
+  offset += align_up(static_cast<size_t>(blocks) * qh * 4, 256);
+  float* part_l = reinterpret_cast<float*>(scratch + offset);
+
+  const pluto_hip_kv_cache_view& c0 = caches[0];
+  bool fast = round && c0.dtype == PLUTO_HIP_BF16 && decode_fast_supported(d, group) &&
+              !force_generic() && c0.token_stride % 8 == 0 && c0.head_stride % 8 == 0;
+  for (int b = 0; b < batch && fast; ++b)
+    fast = aligned16(caches[b].keys) && aligned16(caches[b].values);
+  const int q_dtype = round ? PLUTO_HIP_BF16 : PLUTO_HIP_F32;
+  const float scale = 1.0f / std::sqrt(static_cast<float>(d));
+  const size_t io_bytes = element_bytes(io_dtype);
+
+  long long block_base = 0;
+  for (int first = 0; first < batch; first += kDecodeBatchMax) {
+    DecodeBatch slice;
+    slice.first = first;
+    slice.count = batch - first < kDecodeBatchMax ? batch - first : kDecodeBatchMax;
+    slice.block_start[0] = 0;
+    for (int i = 0; i < slice.count; ++i) {
+      slice.positions[i] = positions[first + i];
+      slice.keys[i] = caches[first + i].keys;
+      slice.values[i] = caches[first + i].values;
+      slice.block_start[i + 1] = slice.block_start[i] + (positions[first + i] + split) / split;
+    }
+    DecodePrepareArgs prep;
+    prep.q_gate = q_gate;
+    prep.k = k;
+    prep.v = v;
+    prep.io_dtype = io_dtype;
+    prep.q_norm = q_norm;
+    prep.k_norm = k_norm;
+    prep.q_out = queries;
+    prep.q_out_dtype = q_dtype;
+    prep.cache_dtype = c0.dtype;
+    prep.token_stride = c0.token_stride;
+    prep.head_stride = c0.head_stride;
+    prep.query_heads = qh;
+    prep.key_value_heads = kh;
+    prep.head_dim = d;
+    prep.rotary_dim = p->rotary_dim;
+    prep.epsilon = p->rms_norm_epsilon;
+    prep.theta = p->rope_theta;
+    prep.round = round;
+    status = launch_decode_prepare(s, prep, slice);
+    if (status != 0) return status;
+    if (fast) {
+      DecodeArgs a;
+      a.q = static_cast<const uint16_t*>(queries);
+      a.token_stride = c0.token_stride;
+      a.head_stride = c0.head_stride;
+      a.query_heads = qh;
+      a.key_value_heads = kh;
+      a.head_dim = d;
+      a.split_tokens = split;
+      a.scale = scale;
+      a.part_o = part_o;
+      a.part_m = part_m;
+      a.part_l = part_l;
+      a.block_base = block_base;
+      status = launch_decode_fast(s, a, slice);
+      if (status != 0) return status;
+      DecodeCombineArgs c;
+      c.part_o = part_o;
+      c.part_m = part_m;
+      c.part_l = part_l;
+      c.block_base = block_base;
+      c.q_gate = q_gate;
+      c.out = out;
+      c.io_dtype = io_dtype;
+      c.query_heads = qh;
+      c.key_value_heads = kh;
+      c.head_dim = d;
+      c.round = round;
+      status = launch_decode_combine(s, c, slice);
+      if (status != 0) return status;
+    } else {
+      for (int i = 0; i < slice.count; ++i) {
+        const int b = first + i;
+        GenericForwardArgs a;
+        const char* qbase = static_cast<const char*>(queries) +
+                            static_cast<size_t>(b) * qh * d * element_bytes(q_dtype);
+        a.q = {qbase, 0, 1LL * qh * d, d, q_dtype};
+        a.k = {caches[b].keys, 0, c0.token_stride, c0.head_stride, c0.dtype};
+        a.v = {caches[b].values, 0, c0.token_stride, c0.head_stride, c0.dtype};
+        const char* gbase = static_cast<const char*>(q_gate) +
+                            (static_cast<size_t>(b) * qh * 2 * d + d) * io_bytes;
+        a.gate = {gbase, 0, 2LL * qh * d, 2LL * d, io_dtype};
+        a.out = static_cast<char*>(out) + static_cast<size_t>(b) * qh * d * io_bytes;
+        a.o_row_stride = 1LL * qh * d;
+        a.o_head_stride = d;
+        a.o_dtype = io_dtype;
+        a.q_rows = 1;
+        a.kv_rows = positions[b] + 1;
+        a.start_position = positions[b];
+        a.query_heads = qh;
+        a.group = group;
+        a.head_dim = d;
+        a.scale = scale;
+        a.round_to_bf16 = round;
+        status = launch_generic_forward(s, a, 1);
+        if (status != 0) return status;
+      }
+    }
+    if (probabilities) {
+      for (int i = 0; i < slice.count; ++i) {
+        const int b = first + i;
+        if (!probabilities[b]) continue;
+        const char* qbase = static_cast<const char*>(queries) +
+                            static_cast<size_t>(b) * qh * d * element_bytes(q_dtype);
+        const CacheView view{caches[b].keys, caches[b].values, c0.dtype, c0.token_stride,
+                             c0.head_stride};
+        status = launch_decode_probabilities(s, qbase, q_dtype, view, qh, kh, d,
+                                             positions[b] + 1, scale, probabilities[b]);
+        if (status != 0) return status;
+      }
+    }
+    block_base += slice.block_start[slice.count];
+  }
+  return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,327 @@
+// Batched single-token GQA decode against a bf16 KV cache: split-K over blocks
+// of the sequence, tuned as an HBM streaming kernel.
+//
+// Semantics: FullAttentionKernel (src/llm/layers/util/cached_attention_ops.cc:
+// 83-126) for every sequence of the batch.  One workgroup owns one
+// (sequence, kv head, block of `split_tokens` cache rows) and serves ALL query
+// heads of the group, so every K and V byte is read from HBM exactly once (the
+// reference launches one program per query head and streams the cache once per
+// head of the group).
+//
+//   scores  S^T[token, head] = K[token, :] . q[head, :] with
+//           v_mfma_f32_16x16x32_bf16: the A operand (16 tokens x 32 channels) is
+//           loaded straight from global memory, 64 contiguous bytes per lane;
+//           the group's heads are the (zero padded) 16 columns.
+//   values  O[head, :] += p[head, token] * V[token, :] on the vector ALU: 16
+//           bytes of V per lane, probabilities broadcast from LDS.  The kernel
+//           is bound by HBM, not by this arithmetic.
+// Partial (o, m, l) triples are written per block; a second kernel combines a
+// sequence's blocks in ascending order (fixed order: bitwise repeatable) and
+// applies bf16(bf16(core) * bf16(sigmoid(gate))).
+#include "gqa.h"
+
+namespace pluto_hip {
+namespace {
+
+constexpr int kMaxSplit = 512;
+constexpr int kThreads = 256;
+
+__device__ inline bf16x8 load_bf16x8(const uint16_t* p) {
+  return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p));
+}
+
+__device__ inline int find_sequence(const DecodeBatch& batch, int block) {
+  int lo = 0, hi = batch.count - 1;
+  while (lo < hi) {  // last b with block_start[b] <= block
+    const int mid = (lo + hi + 1) / 2;
+    if (batch.block_start[mid] <= block) lo = mid; else hi = mid - 1;
+  }
+  return lo;
+}
+
+template <int D, int GROUP>
+__global__ void __launch_bounds__(kThreads)
+decode_split_kernel(DecodeArgs a, DecodeBatch batch) {
+  constexpr int KSTEPS = D / 32;
+  constexpr int QUARTER = D / 4;           // channels per lane quarter in phase 1
+  constexpr int LANES_PER_ROW = D / 8;     // phase 2: 16-byte pieces per V row
+  constexpr int ROWS_PER_PASS = 64 / LANES_PER_ROW;
+  __shared__ __attribute__((aligned(16))) float p_lds[kMaxSplit][8];
+  __shared__ __attribute__((aligned(16))) float o_lds[4][GROUP][D];
+  __shared__ float wave_max[4][16];
+  __shared__ float wave_sum_lds[4][16];
+
+  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+  const int kh = a.key_value_heads;
+  const int g = blockIdx.x % kh;
+  const int block = blockIdx.x / kh;
+  const int b = find_sequence(batch, block);
+  const int seq = batch.first + b;
+  const int length = batch.positions[b] + 1;
+  const int split = a.split_tokens;
+  const int t0 = (block - batch.block_start[b]) * split;
+  const int per_wave = split / 4;
+  const uint16_t* keys = static_cast<const uint16_t*>(batch.keys[b]) + g * a.head_stride;
+  const uint16_t* values = static_cast<const uint16_t*>(batch.values[b]) + g * a.head_stride;
+  const float scale2 = a.scale * kLog2e;
+
+  // ---- phase 1: scores -------------------------------------------------
+  const int hq = lane / 16, n = lane % 16;
+  bf16x8 qf[KSTEPS];
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ++ks) {
+    uint4 bits = make_uint4(0, 0, 0, 0);
+    if (n < GROUP)
+      bits = *reinterpret_cast<const uint4*>(
+          a.q + (static_cast<long long>(seq) * a.query_heads + g * GROUP + n) * D +
+          QUARTER * hq + 8 * ks);
+    qf[ks] = __builtin_bit_cast(bf16x8, bits);
+  }
+  const int groups = per_wave / 16;  // 16-token groups per wave (<= 8)
+  floatx4 s[kMaxSplit / 64];
+  float local_max = kMasked;
+#pragma unroll
+  for (int grp = 0; grp < kMaxSplit / 64; ++grp) {
+    if (grp < groups) {
+      const int token_local = wave * per_wave + 16 * grp;
+      int token = t0 + token_local + n;  // A operand row = lane % 16
+      token = min(token, length - 1);    // stay inside the valid prefix
+      const uint16_t* row = keys + static_cast<long long>(token) * a.token_stride + QUARTER * hq;
+      floatx4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks)
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(load_bf16x8(row + 8 * ks), qf[ks], acc,
+                                                      0, 0, 0);
+      // accumulator register r = (token 4*hq + r of the group, head n)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int t = t0 + token_local + 4 * hq + r;
+        const float v = t < length ? acc[r] * scale2 : kMasked;
+        acc[r] = v;
+        local_max = fmaxf(local_max, v);
+      }
+      s[grp] = acc;
+    }
+  }
+  local_max = fmaxf(local_max, __shfl_xor(local_max, 16, 64));
+  local_max = fmaxf(local_max, __shfl_xor(local_max, 32, 64));
+  if (hq == 0) wave_max[wave][n] = local_max;
+  __syncthreads();
+  const float block_max = fmaxf(fmaxf(wave_max[0][n], wave_max[1][n]),
+                                fmaxf(wave_max[2][n], wave_max[3][n]));
+  float local_sum = 0.0f;
+#pragma unroll
+  for (int grp = 0; grp < kMaxSplit / 64; ++grp) {
+    if (grp < groups) {
+      const int token_local = wave * per_wave + 16 * grp + 4 * hq;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float p = __builtin_amdgcn_exp2f(s[grp][r] - block_max);
+        local_sum += p;
+        if (n < 8) p_lds[token_local + r][n] = p;
+      }
+    }
+  }
+  local_sum += __shfl_xor(local_sum, 16, 64);
+  local_sum += __shfl_xor(local_sum, 32, 64);
+  if (hq == 0) wave_sum_lds[wave][n] = local_sum;
+  __syncthreads();
+
+  // ---- phase 2: O += p V ------------------------------------------------
+  const int sub = lane / LANES_PER_ROW, piece = lane % LANES_PER_ROW;
+  float acc[GROUP][8];
+#pragma unroll
+  for (int hh = 0; hh < GROUP; ++hh)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[hh][e] = 0.0f;
+  const int passes = per_wave / ROWS_PER_PASS;
+#pragma unroll 8
+  for (int pass = 0; pass < passes; ++pass) {
+    const int token_local = wave * per_wave + pass * ROWS_PER_PASS + sub;
+    const int token = min(t0 + token_local, length - 1);
+    const uint4 bits = *reinterpret_cast<const uint4*>(
+        values + static_cast<long long>(token) * a.token_stride + 8 * piece);
+    const float4 p0 = *reinterpret_cast<const float4*>(&p_lds[token_local][0]);
+    const float4 p1 = *reinterpret_cast<const float4*>(&p_lds[token_local][4]);
+    const float p[8] = {p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w};
+    const uint32_t w[4] = {bits.x, bits.y, bits.z, bits.w};
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[2 * i] = __uint_as_float(w[i] << 16);
+      v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+#pragma unroll
+    for (int hh = 0; hh < GROUP; ++hh)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[hh][e] += p[hh] * v[e];
+  }
+#pragma unroll
+  for (int hh = 0; hh < GROUP; ++hh)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      float x = acc[hh][e];
+#pragma unroll
+      for (int offset = LANES_PER_ROW; offset < 64; offset <<= 1)
+        x += __shfl_xor(x, offset, 64);
+      acc[hh][e] = x;
+    }
+  if (sub == 0) {
+#pragma unroll
+    for (int hh = 0; hh < GROUP; ++hh) {
+      float4 lo = make_float4(acc[hh][0], acc[hh][1], acc[hh][2], acc[hh][3]);
+      float4 hi = make_float4(acc[hh][4], acc[hh][5], acc[hh][6], acc[hh][7]);
+      *reinterpret_cast<float4*>(&o_lds[wave][hh][8 * piece]) = lo;
+      *reinterpret_cast<float4*>(&o_lds[wave][hh][8 * piece + 4]) = hi;
+    }
+  }
+  __syncthreads();
+  const long long slot = (a.block_base + block) * kh + g;
+  for (int i = tid; i < GROUP * D; i += kThreads) {
+    const int hh = i / D, c = i % D;
+    a.part_o[(slot * GROUP + hh) * D + c] =
+        (o_lds[0][hh][c] + o_lds[1][hh][c]) + (o_lds[2][hh][c] + o_lds[3][hh][c]);
+  }
+  if (tid < GROUP) {
+    a.part_m[slot * GROUP + tid] =
+        fmaxf(fmaxf(wave_max[0][tid], wave_max[1][tid]), fmaxf(wave_max[2][tid], wave_max[3][tid]));
+    a.part_l[slot * GROUP + tid] = (wave_sum_lds[0][tid] + wave_sum_lds[1][tid]) +
+                                   (wave_sum_lds[2][tid] + wave_sum_lds[3][tid]);
+  }
+}
+
+// One workgroup per (sequence, query head): combines the blocks in ascending
+// order and applies the sigmoid gate (cached_attention_ops.cc:119-125).
+__global__ void __launch_bounds__(64)
+decode_combine_kernel(DecodeCombineArgs a, DecodeBatch batch) {
+  const int b = blockIdx.x / a.query_heads, head = blockIdx.x % a.query_heads;
+  const int seq = batch.first + b;
+  const int group = a.query_heads / a.key_value_heads;
+  const int g = head / group, hh = head % group;
+  const int D = a.head_dim;
+  const int first = batch.block_start[b], blocks = batch.block_start[b + 1] - first;
+  float maximum = kMasked;
+  for (int j = 0; j < blocks; ++j) {
+    const long long slot = ((a.block_base + first + j) * a.key_value_heads + g) * group + hh;
+    maximum = fmaxf(maximum, a.part_m[slot]);
+  }
+  float normalizer = 0.0f;
+  float o[4] = {0.0f, 0.0f, 0.0f, 0.0f};  // head_dim <= 256 = 4 channels per lane
+  for (int j = 0; j < blocks; ++j) {
+    const long long slot = ((a.block_base + first + j) * a.key_value_heads + g) * group + hh;
+    const float w = __builtin_amdgcn_exp2f(a.part_m[slot] - maximum);
+    normalizer += a.part_l[slot] * w;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c = threadIdx.x + 64 * i;
+      if (c < D) o[i] += a.part_o[slot * D + c] * w;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int c = threadIdx.x + 64 * i;
+    if (c >= D) continue;
+    const float core = o[i] / normalizer;
+    const long long at = static_cast<long long>(seq) * a.query_heads + head;
+    const float logit = load_element(a.q_gate, (at * 2 + 1) * D + c, a.io_dtype);
+    const float sigmoid = 1.0f / (1.0f + expf(-logit));
+    const float value = a.round ? round_to_bf16(round_to_bf16(core) * round_to_bf16(sigmoid))
+                                : core * sigmoid;
+    store_element(a.out, at * D + c, a.io_dtype, value);
+  }
+}
+
+// Two-pass probability row for inspection: one workgroup per query head.
+__global__ void __launch_bounds__(256)
+decode_probabilities_kernel(const void* q, int q_dtype, CacheView cache, int query_heads,
+                            int key_value_heads, int head_dim, int length, float scale,
+                            float* probabilities) {
+  __shared__ float query[256];
+  __shared__ float reduce[4];
+  const int head = blockIdx.x;
+  const int kv = head / (query_heads / key_value_heads);
+  float* row = probabilities + static_cast<long long>(head) * length;
+  for (int c = threadIdx.x; c < head_dim; c += 256)
+    query[c] = load_element(q, static_cast<long long>(head) * head_dim + c, q_dtype);
+  __syncthreads();
+  float maximum = kMasked;
+  for (int t = threadIdx.x; t < length; t += 256) {
+    const long long base = t * cache.token_stride + kv * cache.head_stride;
+    float score = 0.0f;
+    for (int c = 0; c < head_dim; ++c)
+      score += load_element(cache.keys, base + c, cache.dtype) * query[c];
+    score *= scale;
+    row[t] = score;
+    maximum = fmaxf(maximum, score);
+  }
+  maximum = wave_max(maximum);
+  if (threadIdx.x % 64 == 0) reduce[threadIdx.x / 64] = maximum;
+  __syncthreads();
+  maximum = fmaxf(fmaxf(reduce[0], reduce[1]), fmaxf(reduce[2], reduce[3]));
+  __syncthreads();
+  float sum = 0.0f;
+  for (int t = threadIdx.x; t < length; t += 256) {
+    const float p = expf(row[t] - maximum);
+    row[t] = p;
+    sum += p;
+  }
+  sum = wave_sum(sum);
+  if (threadIdx.x % 64 == 0) reduce[threadIdx.x / 64] = sum;
+  __syncthreads();
+  sum = (reduce[0] + reduce[1]) + (reduce[2] + reduce[3]);
+  for (int t = threadIdx.x; t < length; t += 256) row[t] = row[t] / sum;
+}
+
+template <int D>
+int launch_for_group(hipStream_t stream, const DecodeArgs& a, const DecodeBatch& batch,
+                     int group, unsigned blocks) {
+  switch (group) {
+    case 1: decode_split_kernel<D, 1><<<blocks, kThreads, 0, stream>>>(a, batch); break;
+    case 2: decode_split_kernel<D, 2><<<blocks, kThreads, 0, stream>>>(a, batch); break;
+    case 4: decode_split_kernel<D, 4><<<blocks, kThreads, 0, stream>>>(a, batch); break;
+    case 6: decode_split_kernel<D, 6><<<blocks, kThreads, 0, stream>>>(a, batch); break;
+    case 8: decode_split_kernel<D, 8><<<blocks, kThreads, 0, stream>>>(a, batch); break;
+    default: return PLUTO_HIP_EUNSUPPORTED;
+  }
+  return launch_status();
+}
+
+}  // namespace
+
+bool decode_fast_supported(int head_dim, int group) {
+  const bool dim_ok = head_dim == 64 || head_dim == 128 || head_dim == 256;
+  const bool group_ok = group == 1 || group == 2 || group == 4 || group == 6 || group == 8;
+  return dim_ok && group_ok;
+}
+
+int launch_decode_fast(hipStream_t stream, const DecodeArgs& a, const DecodeBatch& batch) {
+  const int group = a.query_heads / a.key_value_heads;
+  const long long blocks =
+      static_cast<long long>(batch.block_start[batch.count]) * a.key_value_heads;
+  if (blocks <= 0 || blocks > 0x7fffffffLL) return PLUTO_HIP_EINVAL;
+  if (a.split_tokens < 64 || a.split_tokens > kMaxSplit || a.split_tokens % 64 != 0)
+    return PLUTO_HIP_EINVAL;
+  switch (a.head_dim) {
+    case 64: return launch_for_group<64>(stream, a, batch, group, static_cast<unsigned>(blocks));
+    case 128: return launch_for_group<128>(stream, a, batch, group, static_cast<unsigned>(blocks));
+    case 256: return launch_for_group<256>(stream, a, batch, group, static_cast<unsigned>(blocks));
+    default: return PLUTO_HIP_EUNSUPPORTED;
+  }
+}
+
+int launch_decode_combine(hipStream_t stream, const DecodeCombineArgs& a,
+                          const DecodeBatch& batch) {
+  decode_combine_kernel<<<batch.count * a.query_heads, 64, 0, stream>>>(a, batch);
+  return launch_status();
+}
+
+int launch_decode_probabilities(hipStream_t stream, const void* q, int q_dtype,
+                                const CacheView& cache, int query_heads,
+                                int key_value_heads, int head_dim, int length,
+                                float scale, float* probabilities) {
+  decode_probabilities_kernel<<<query_heads, 256, 0, stream>>>(
+      q, q_dtype, cache, query_heads, key_value_heads, head_dim, length, scale, probabilities);
+  return launch_status();
+}
+
+}  // namespace pluto_hip

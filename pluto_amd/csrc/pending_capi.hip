@@ -16,27 +16,4 @@ int pluto_hip_gdn_recurrence(void*, const pluto_hip_delta_params*, int, int,
                              const float*, int, float, float*, void*, int) {
   return PLUTO_HIP_EUNSUPPORTED;
 }
-int pluto_hip_attention_params_validate(const pluto_hip_attention_params*) {
-  return PLUTO_HIP_EUNSUPPORTED;
-}
-size_t pluto_hip_gqa_prefill_workspace_bytes(const pluto_hip_attention_params*, int) {
-  return 0;
-}
-int pluto_hip_gqa_prefill(void*, const pluto_hip_attention_params*, int, int,
-                          const void*, const void*, const void*, const float*,
-                          const float*, const pluto_hip_kv_cache_view*, void*,
-                          float*, void*, size_t) {
-  return PLUTO_HIP_EUNSUPPORTED;
-}
-size_t pluto_hip_gqa_decode_workspace_bytes(const pluto_hip_attention_params*, int,
-                                            const int*, int) {
-  return 0;
-}
-int pluto_hip_gqa_decode(void*, const pluto_hip_attention_params*, int, int,
-                         const void*, const void*, const void*, const float*,
-                         const float*, const int*, const pluto_hip_kv_cache_view*,
-                         void*, float* const*, int, void*, size_t) {
-  return PLUTO_HIP_EUNSUPPORTED;
-}
-
 }  // extern "C"
