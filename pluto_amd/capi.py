@@ -294,3 +294,43 @@ def gqa_decode(p, q_gate, k, v, q_norm, k_norm, caches, positions=None, split_to
         for c in caches:
             c.position += 1
     return out
+
+
+# ---- gated delta-net -----------------------------------------------------------
+
+def delta_params(key_heads=16, value_heads=48, key_head_dim=128, value_head_dim=128,
+                 conv_kernel_dim=4, rms_norm_epsilon=1e-6, round_to_bfloat16=True):
+    return DeltaParams(key_heads, value_heads, key_head_dim, value_head_dim, conv_kernel_dim,
+                       rms_norm_epsilon, int(bool(round_to_bfloat16)))
+
+
+def gdn_scan_workspace(p, batch, length, chunk=0, device="cuda"):
+    size = lib().pluto_hip_gdn_scan_workspace_bytes(ctypes.byref(p), batch, length, chunk)
+    return torch.empty(max(size, 16), dtype=torch.uint8, device=device)
+
+
+def gdn_scan(p, q, k, v, log_decay, beta, state, normalize_qk=False, q_scale=1.0, chunk=0,
+             workspace=None, out=None, stream=None):
+    """q, k bf16 [B, T, kh, kd]; v bf16 [B, T, vh, vd]; log_decay, beta fp32 [B, T, vh];
+    state fp32 [B, vh, kd, vd] (updated in place).  Returns out bf16 [B, T, vh, vd]."""
+    batch, length = q.shape[0], q.shape[1]
+    if workspace is None:
+        workspace = gdn_scan_workspace(p, batch, length, chunk, q.device)
+    if out is None:
+        out = torch.empty(v.shape, dtype=torch.bfloat16, device=q.device)
+    check(lib().pluto_hip_gdn_scan(stream or current_stream(), ctypes.byref(p), batch, length,
+                                   chunk, ptr(q), ptr(k), ptr(v), ptr(log_decay), ptr(beta),
+                                   int(bool(normalize_qk)), float(q_scale), ptr(state), ptr(out),
+                                   ptr(workspace), workspace.numel()))
+    return out
+
+
+def gdn_recurrence(p, q, k, v, log_decay, beta, state, normalize_qk=False, q_scale=1.0,
+                   out_dtype=None, stream=None):
+    batch, length = q.shape[0], q.shape[1]
+    out = torch.empty(v.shape, dtype=out_dtype or torch.bfloat16, device=q.device)
+    check(lib().pluto_hip_gdn_recurrence(stream or current_stream(), ctypes.byref(p), batch,
+                                         length, ptr(q), ptr(k), ptr(v), ptr(log_decay),
+                                         ptr(beta), int(bool(normalize_qk)), float(q_scale),
+                                         ptr(state), ptr(out), dtype_code(out)))
+    return out

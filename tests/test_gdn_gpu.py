@@ -1,0 +1,181 @@
+"""GPU parity of the gated delta-net scan (chunked matrix-core path and the
+token-by-token recurrence) with the CPU oracle, through the C ABI.  Cases follow
+sequence_delta_net_test.cc and cached_attention_ops_test.cc of the reference."""
+import math
+import os
+
+import numpy as np
+import pytest
+
+from tests.util import assert_close, assert_close_bf16
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+
+@pytest.fixture(scope="module")
+def capi():
+    from pluto_amd import capi
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    capi.lib()
+    return capi
+
+
+def dev(x, dtype=None):
+    t = torch.from_numpy(np.ascontiguousarray(x)).cuda()
+    return t.to(dtype) if dtype is not None else t
+
+
+def make_inputs(oracle, rng, B, T, kh, vh, kd, vd, normalized):
+    q = rng.standard_normal((B, T, kh, kd)).astype(np.float32)
+    k = rng.standard_normal((B, T, kh, kd)).astype(np.float32)
+    if normalized:  # L2-normalised per head, as the scan configuration states
+        q /= np.linalg.norm(q, axis=-1, keepdims=True)
+        k /= np.linalg.norm(k, axis=-1, keepdims=True)
+    q, k = oracle.bf16_round(q), oracle.bf16_round(k)
+    v = oracle.bf16_round(rng.standard_normal((B, T, vh, vd)).astype(np.float32))
+    beta = (1 / (1 + np.exp(-rng.standard_normal((B, T, vh))))).astype(np.float32)
+    g = (-np.log1p(np.exp(rng.standard_normal((B, T, vh))))).astype(np.float32)
+    return q, k, v, g, beta
+
+
+def run_device(capi, fn, p, q, k, v, g, beta, state0, normalize, scale):
+    bf = torch.bfloat16
+    state = dev(state0.astype(np.float32))
+    out = fn(p, dev(q, bf), dev(k, bf), dev(v, bf), dev(g), dev(beta), state,
+             normalize_qk=normalize, q_scale=scale)
+    torch.cuda.synchronize()
+    return out.float().cpu().numpy(), state.cpu().numpy()
+
+
+def run_oracle(oracle, po, q, k, v, g, beta, state0, normalize, scale, heads=None):
+    outs, states = [], []
+    for b in range(q.shape[0]):
+        core, state = oracle.gdn_scan(po, q[b], k[b], v[b], g[b], beta[b], normalize, scale,
+                                      state0[b], heads)
+        outs.append(core)
+        states.append(state)
+    return np.stack(outs), np.stack(states)
+
+
+@pytest.mark.parametrize("kh,vh,kd,vd", [(1, 2, 3, 5), (2, 4, 5, 35), (2, 6, 128, 128), (1, 1, 64, 256)])
+@pytest.mark.parametrize("normalize", [False, True])
+def test_recurrence_matches_oracle(capi, oracle, kh, vh, kd, vd, normalize):
+    B, T = 2, 37
+    p = capi.delta_params(kh, vh, kd, vd)
+    po = oracle.delta_params(kh, vh, kd, vd)
+    rng = np.random.default_rng(kd + vd)
+    q, k, v, g, beta = make_inputs(oracle, rng, B, T, kh, vh, kd, vd, not normalize)
+    state0 = 0.1 * rng.standard_normal((B, vh, kd, vd))
+    scale = 1 / math.sqrt(kd)
+    got, got_state = run_device(capi, capi.gdn_recurrence, p, q, k, v, g, beta, state0, normalize, scale)
+    want, want_state = run_oracle(oracle, po, q, k, v, g, beta, state0, normalize, scale)
+    # fp32 state and sums, output rounded to bf16: sequence_delta_net_test.cc:253-255
+    assert np.all(np.abs(got - want) <= 1.5e-4 + 1.5e-2 * np.abs(want))
+    assert_close(got_state, want_state, 1e-4, "recurrence state")
+
+
+@pytest.mark.parametrize("T", [64, 65, 200, 1024])
+@pytest.mark.parametrize("normalize", [False, True])
+def test_chunked_scan_matches_oracle(capi, oracle, T, normalize):
+    B, kh, vh, kd, vd = 2, 2, 4, 128, 128
+    p = capi.delta_params(kh, vh, kd, vd)
+    po = oracle.delta_params(kh, vh, kd, vd)
+    rng = np.random.default_rng(T)
+    q, k, v, g, beta = make_inputs(oracle, rng, B, T, kh, vh, kd, vd, not normalize)
+    state0 = 0.1 * rng.standard_normal((B, vh, kd, vd))
+    scale = 1 / math.sqrt(kd)
+    got, got_state = run_device(capi, capi.gdn_scan, p, q, k, v, g, beta, state0, normalize, scale)
+    want, want_state = run_oracle(oracle, po, q, k, v, g, beta, state0, normalize, scale)
+    assert_close_bf16(got, want, "chunked scan T%d out" % T)
+    assert_close_bf16(got_state, want_state, "chunked scan T%d state" % T)
+
+
+def test_textbook_special_cases(capi, oracle):
+    # beta = 0: pure decay of the initial state; g = 0, beta = 1 with orthonormal
+    # keys: the state becomes sum k v^T and reading with a key returns its value.
+    kd = vd = 128
+    T = 128
+    p = capi.delta_params(1, 1, kd, vd)
+    rng = np.random.default_rng(0)
+    basis, _ = np.linalg.qr(rng.standard_normal((kd, kd)))
+    k = oracle.bf16_round(basis.T.reshape(1, T, 1, kd).astype(np.float32))
+    v = oracle.bf16_round(rng.standard_normal((1, T, 1, vd)).astype(np.float32))
+    zeros = np.zeros((1, T, 1), np.float32)
+    state0 = np.zeros((1, 1, kd, vd))
+    got, state = run_device(capi, capi.gdn_scan, p, k, k, v, zeros, zeros + 1, state0, False, 1.0)
+    # bf16 keys are orthonormal only to 2^-9: compare with that slack
+    np.testing.assert_allclose(got[0, :, 0], v[0, :, 0], atol=0.05)
+    np.testing.assert_allclose(state[0, 0], k[0, :, 0].astype(np.float64).T @ v[0, :, 0], atol=0.05)
+    s0 = rng.standard_normal((1, 1, kd, vd))
+    g = -rng.random((1, T, 1)).astype(np.float32)
+    got, state = run_device(capi, capi.gdn_scan, p, k, k, v, g, zeros, s0, False, 1.0)
+    total = math.exp(float(g.astype(np.float64).sum()))
+    np.testing.assert_allclose(state[0, 0], total * s0[0, 0], rtol=2e-2, atol=1e-30)
+
+
+def test_state_carries_across_calls(capi, oracle):
+    B, kh, vh, kd, vd = 1, 1, 2, 128, 128
+    p = capi.delta_params(kh, vh, kd, vd)
+    rng = np.random.default_rng(6)
+    q, k, v, g, beta = make_inputs(oracle, rng, B, 320, kh, vh, kd, vd, True)
+    state0 = np.zeros((B, vh, kd, vd))
+    whole, whole_state = run_device(capi, capi.gdn_scan, p, q, k, v, g, beta, state0, False, 0.1)
+    first, mid = run_device(capi, capi.gdn_scan, p, q[:, :128], k[:, :128], v[:, :128], g[:, :128],
+                            beta[:, :128], state0, False, 0.1)
+    second, end = run_device(capi, capi.gdn_scan, p, q[:, 128:], k[:, 128:], v[:, 128:], g[:, 128:],
+                             beta[:, 128:], mid, False, 0.1)
+    # the split falls on a chunk boundary: identical arithmetic, identical bits
+    np.testing.assert_array_equal(np.concatenate([first, second], 1), whole)
+    np.testing.assert_array_equal(end, whole_state)
+
+
+def test_config5_chunked_scan(capi, oracle):
+    # B=2, T=16384, 16 heads, d_k=d_v=128, chunk 64, bf16 inputs, fp32 state;
+    # q,k ~ N(0,1) L2-normalised, beta = sigmoid(N(0,1)), g = -softplus(N(0,1)), seed 4.
+    B, T, H, kd, vd = 2, 16384, 16, 128, 128
+    p = capi.delta_params(H, H, kd, vd)
+    po = oracle.delta_params(H, H, kd, vd)
+    rng = np.random.default_rng(4)
+    q, k, v, g, beta = make_inputs(oracle, rng, B, T, H, H, kd, vd, True)
+    state0 = np.zeros((B, H, kd, vd))
+    scale = 1 / math.sqrt(kd)
+    bf = torch.bfloat16
+    dq, dk, dv, dg, db = dev(q, bf), dev(k, bf), dev(v, bf), dev(g), dev(beta)
+    state = dev(state0.astype(np.float32))
+    out = capi.gdn_scan(p, dq, dk, dv, dg, db, state, q_scale=scale, chunk=64)
+    torch.cuda.synchronize()
+    got, got_state = out.float().cpu().numpy(), state.cpu().numpy()
+    # CPU recurrence on whole (sequence, head) chains (they are independent)
+    for b, h in ((0, 3), (1, 12)):
+        core, want_state = oracle.gdn_scan(po, q[b], k[b], v[b], g[b], beta[b], False, scale,
+                                           state0[b], (h, h + 1))
+        assert_close_bf16(got[b, :, h], core[:, h], "config 5 seq %d head %d out" % (b, h))
+        assert_close_bf16(got_state[b, h], want_state[h], "config 5 seq %d head %d state" % (b, h))
+    # every chain: against the token-by-token kernel
+    state2 = dev(state0.astype(np.float32))
+    out2 = capi.gdn_recurrence(p, dq, dk, dv, dg, db, state2, q_scale=scale)
+    torch.cuda.synchronize()
+    assert_close_bf16(got, out2.float().cpu().numpy(), "config 5 vs recurrence kernel out")
+    assert_close_bf16(got_state, state2.cpu().numpy(), "config 5 vs recurrence kernel state")
+    # bitwise repeatable
+    state3 = dev(state0.astype(np.float32))
+    out3 = capi.gdn_scan(p, dq, dk, dv, dg, db, state3, q_scale=scale, chunk=64)
+    assert torch.equal(out, out3) and torch.equal(state, state3)
+
+
+def test_rejects_bad_arguments(capi):
+    # cached_attention_ops_test.cc:622-636
+    t = torch.zeros(64, device="cuda")
+    for kw in (dict(key_head_dim=129), dict(key_heads=0), dict(key_heads=2, value_heads=3),
+               dict(value_head_dim=257), dict(conv_kernel_dim=33), dict(rms_norm_epsilon=0.0)):
+        p = capi.delta_params(**{**dict(key_heads=1, value_heads=1, key_head_dim=4, value_head_dim=4), **kw})
+        code = capi.lib().pluto_hip_gdn_recurrence(capi.current_stream(), p, 1, 1, capi.ptr(t),
+                                                   capi.ptr(t), capi.ptr(t), capi.ptr(t), capi.ptr(t),
+                                                   0, 1.0, capi.ptr(t), capi.ptr(t), capi.F32)
+        assert code == capi.EINVAL
+    p = capi.delta_params(1, 1, 4, 4)
+    code = capi.lib().pluto_hip_gdn_recurrence(capi.current_stream(), p, 1, 1, None, None, None,
+                                               None, None, 0, 1.0, None, None, capi.F32)
+    assert code == capi.EINVAL
