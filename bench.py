@@ -1,15 +1,23 @@
 #!/usr/bin/env python3
 """Benchmark of the attention hot path on one MI355X.
 
-`python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]`
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
 
 A step is one pass of the hot path over one batch of synthetic input that is
-already resident in HBM.  The default workload is the configuration the
-headline metric is quoted on: GPT-2-small causal attention forward+backward,
-bf16 storage, B=16, T=1024, H=12, D=64.  One JSON line is printed.
+already resident in HBM when the timed region starts.  The default workload is
+the configuration the headline metric is quoted on: GPT-2-small causal
+attention forward+backward, bf16 storage with fp32 accumulation, B=16, T=1024,
+H=12, D=64.  The other configurations of the path can be selected with
+--workload; --workload all appends their figures under "workloads".
+
+Exactly one JSON line is printed.  `roofline` describes the dominant kernel
+group of the step (its own average duration is measured with HIP events on
+the launch stream); `cpu_baseline` is the scalar CPU oracle timed on this
+host on a bounded sample of the same workload (a reported baseline only).
 """
 import argparse
 import json
+import math
 import os
 import sys
 import time
@@ -18,8 +26,11 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
-PEAK_HBM_GBS = 8000.0       # MI355X HBM3E, published
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA (published)
+PEAK_FP32_TFLOPS = 157.3    # MI355X fp32 matrix (published)
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E (published)
+
+NAMES = ["mha_train_bf16", "mha_fwd_fp32", "gqa_prefill", "gqa_decode", "gdn_scan"]
 
 
 def parse_args():
@@ -27,9 +38,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="mha_train_bf16",
-                    choices=["mha_train_bf16", "mha_fwd_fp32", "gqa_prefill",
-                             "gqa_decode", "gdn_scan"])
+    ap.add_argument("--workload", default="mha_train_bf16", choices=NAMES + ["all"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     return ap.parse_args()
 
@@ -38,26 +47,19 @@ def causal_pairs(T):
     return T * (T + 1) // 2
 
 
-class EventTimer:
-    """HIP events on the stream the kernels are launched on."""
-
-    def __init__(self, torch, stream):
-        self.torch, self.stream = torch, stream
-        self.pairs = []
-
-    def time(self, fn):
-        start = self.torch.cuda.Event(enable_timing=True)
-        end = self.torch.cuda.Event(enable_timing=True)
-        start.record(self.stream)
-        fn()
-        end.record(self.stream)
-        self.pairs.append((start, end))
-
-    def mean_ms(self):
-        return sum(s.elapsed_time(e) for s, e in self.pairs) / max(len(self.pairs), 1)
+def values(np, count, phase, scale):
+    i = np.arange(count, dtype=np.float32)
+    return (np.float32(scale) * np.sin(np.float32(phase) + i * np.float32(0.29))).astype(np.float32)
 
 
-def mha_train_bf16(args, torch, capi):
+# --------------------------------------------------------------------------
+# Workloads.  Each returns a dict:
+#   step        callable running the whole hot path once
+#   parts       [(name, callable, algorithmic work of that part)]
+#   work        algorithmic FLOPs (bound mfma) or bytes (bound hbm) per step
+# --------------------------------------------------------------------------
+
+def mha_train_bf16(torch, capi):
     B, T, H, D = 16, 1024, 12, 64
     E = H * D
     gen = torch.Generator(device="cuda").manual_seed(1)
@@ -78,98 +80,228 @@ def mha_train_bf16(args, torch, capi):
         forward()
         backward()
 
-    fwd_flops = 4.0 * B * H * D * causal_pairs(T)
-    bwd_flops = 10.0 * B * H * D * causal_pairs(T)
-    return dict(
-        step=step, parts=[("forward", forward, fwd_flops), ("backward", backward, bwd_flops)],
-        flops=fwd_flops + bwd_flops, metric="attention_fwd_bwd_tflops", unit="TFLOP/s",
-        dtype="bf16", bound="mfma", peak=PEAK_BF16_TFLOPS,
-        config={"workload": "gpt2_small_causal_mha_fwd_bwd", "batch": B, "seq_len": T,
-                "heads": H, "head_dim": D, "storage": "bf16", "accumulate": "fp32"},
-        cpu=("mha", dict(B=B, T=T, H=H, D=D, bf16=True)))
+    fwd = 4.0 * B * H * D * causal_pairs(T)
+    bwd = 10.0 * B * H * D * causal_pairs(T)
+    return dict(step=step, parts=[("forward", forward, fwd), ("backward", backward, bwd)],
+                work=fwd + bwd, metric="attention_fwd_bwd_tflops", unit="TFLOP/s", dtype="bf16",
+                bound="mfma", peak=PEAK_BF16_TFLOPS,
+                config={"workload": "gpt2_small_causal_mha_fwd_bwd", "batch": B, "seq_len": T,
+                        "heads": H, "head_dim": D, "storage": "bf16", "accumulate": "fp32"},
+                cpu=("mha", dict(B=B, T=T, H=H, D=D, bf16=True, backward=True)))
 
 
-WORKLOADS = {"mha_train_bf16": mha_train_bf16}
+def mha_fwd_fp32(torch, capi):
+    B, T, H, D = 4, 256, 12, 64
+    E = H * D
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    qkv = torch.randn((B * T, 3 * E), generator=gen, device="cuda")
+
+    def forward():
+        capi.mha_forward(qkv, T, H)
+
+    work = 4.0 * B * H * D * causal_pairs(T)
+    return dict(step=forward, parts=[("forward", forward, work)], work=work,
+                metric="attention_fwd_tflops", unit="TFLOP/s", dtype="f32", bound="mfma",
+                peak=PEAK_FP32_TFLOPS,
+                config={"workload": "gpt2_small_causal_mha_fwd_fp32", "batch": B, "seq_len": T,
+                        "heads": H, "head_dim": D, "storage": "fp32"},
+                cpu=("mha", dict(B=B, T=T, H=H, D=D, bf16=False, backward=False)))
 
 
-def cpu_baseline_mha(spec, budget_units=1):
-    """Times the scalar CPU oracle (one thread) on whole (sequence, head) units of
-    the same workload and scales to the full size."""
+def gqa_prefill(torch, capi):
+    import numpy as np
+    T, qh, kh, d = 8192, 24, 4, 128
+    p = capi.attention_params(qh, kh, d, 32, capacity=T)
+    gen = torch.Generator(device="cuda").manual_seed(2)
+    bf = torch.bfloat16
+    qg = (0.5 * torch.randn((T, qh, 2, d), generator=gen, device="cuda")).to(bf)
+    k = (0.5 * torch.randn((T, kh, d), generator=gen, device="cuda")).to(bf)
+    v = (0.5 * torch.randn((T, kh, d), generator=gen, device="cuda")).to(bf)
+    qw = torch.from_numpy(values(np, d, 0.2, 0.3)).cuda()
+    kw = torch.from_numpy(values(np, d, 0.8, 0.4)).cuda()
+    cache = capi.KvCache(T, kh, d)
+
+    def step():
+        capi.gqa_prefill(p, qg, k, v, qw, kw, cache)
+
+    work = 4.0 * qh * d * causal_pairs(T)
+    return dict(step=step, parts=[("prefill", step, work)], work=work,
+                metric="gqa_prefill_tflops", unit="TFLOP/s", dtype="bf16", bound="mfma",
+                peak=PEAK_BF16_TFLOPS,
+                config={"workload": "qwen_gqa_prefill", "batch": 1, "seq_len": T, "query_heads": qh,
+                        "kv_heads": kh, "head_dim": d, "kv_cache": "bf16 [1,4,8192,128], written by the call"},
+                cpu=None)
+
+
+def gqa_decode(torch, capi):
+    import numpy as np
+    batch, qh, kh, d, capacity = 32, 24, 4, 128, 32768
+    p = capi.attention_params(qh, kh, d, 32, capacity=capacity)
+    rng = np.random.default_rng(3)
+    lengths = (1024 + np.floor(rng.random(batch) * 31745)).astype(int)
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    bf = torch.bfloat16
+    caches = []
+    for L in lengths:
+        c = capi.KvCache(capacity, kh, d)
+        c.keys[:, :L] = torch.randn((kh, L, d), generator=gen, device="cuda").to(bf)
+        c.values[:, :L] = torch.randn((kh, L, d), generator=gen, device="cuda").to(bf)
+        c.position = int(L - 1)
+        caches.append(c)
+    q_gate = torch.randn((batch, qh, 2, d), generator=gen, device="cuda").to(bf)
+    k = torch.randn((batch, kh, d), generator=gen, device="cuda").to(bf)
+    v = torch.randn((batch, kh, d), generator=gen, device="cuda").to(bf)
+    qw = torch.from_numpy(values(np, d, 0.2, 0.3)).cuda()
+    kw = torch.from_numpy(values(np, d, 0.8, 0.4)).cuda()
+    positions = [int(L - 1) for L in lengths]
+    workspace = capi.gqa_decode_workspace(p, positions, 512)
+    out = torch.empty((batch, qh, d), dtype=bf, device="cuda")
+
+    def step():
+        capi.gqa_decode(p, q_gate, k, v, qw, kw, caches, positions=positions, split_tokens=512,
+                        workspace=workspace, out=out, advance=False)
+
+    work = 2.0 * kh * d * 2 * float(lengths.sum())   # K and V bytes of the valid prefix
+    return dict(step=step, parts=[("decode", step, work)], work=work,
+                metric="gqa_decode_hbm_gbs", unit="GB/s", dtype="bf16", bound="hbm",
+                peak=PEAK_HBM_GBS,
+                config={"workload": "qwen_gqa_decode", "batch": batch, "sum_context": int(lengths.sum()),
+                        "query_heads": qh, "kv_heads": kh, "head_dim": d, "split_tokens": 512,
+                        "kv_cache": "bf16 head-major"},
+                cpu=None)
+
+
+def gdn_scan(torch, capi):
+    B, T, H, dk, dv = 2, 16384, 16, 128, 128
+    p = capi.delta_params(H, H, dk, dv)
+    gen = torch.Generator(device="cuda").manual_seed(4)
+    bf = torch.bfloat16
+    q = torch.nn.functional.normalize(torch.randn((B, T, H, dk), generator=gen, device="cuda"), dim=-1).to(bf)
+    k = torch.nn.functional.normalize(torch.randn((B, T, H, dk), generator=gen, device="cuda"), dim=-1).to(bf)
+    v = torch.randn((B, T, H, dv), generator=gen, device="cuda").to(bf)
+    beta = torch.sigmoid(torch.randn((B, T, H), generator=gen, device="cuda"))
+    g = -torch.nn.functional.softplus(torch.randn((B, T, H), generator=gen, device="cuda"))
+    state = torch.zeros((B, H, dk, dv), device="cuda")
+    workspace = capi.gdn_scan_workspace(p, B, T, 64)
+    out = torch.empty((B, T, H, dv), dtype=bf, device="cuda")
+    scale = 1.0 / math.sqrt(dk)
+
+    def step():
+        state.zero_()
+        capi.gdn_scan(p, q, k, v, g, beta, state, q_scale=scale, chunk=64, workspace=workspace,
+                      out=out)
+
+    work = B * T * H * (2 * dk + 2 * dv) * 2.0 + 2.0 * B * T * H * 4 + B * H * dk * dv * 4.0
+    return dict(step=step, parts=[("scan", step, work)], work=work,
+                metric="gated_delta_scan_hbm_gbs", unit="GB/s", dtype="bf16", bound="hbm",
+                peak=PEAK_HBM_GBS,
+                config={"workload": "gated_delta_net_chunked_scan", "batch": B, "seq_len": T,
+                        "heads": H, "d_k": dk, "d_v": dv, "chunk": 64, "state": "fp32"},
+                cpu=None)
+
+
+WORKLOADS = {"mha_train_bf16": mha_train_bf16, "mha_fwd_fp32": mha_fwd_fp32,
+             "gqa_prefill": gqa_prefill, "gqa_decode": gqa_decode, "gdn_scan": gdn_scan}
+
+
+def cpu_baseline_mha(spec):
+    """Scalar CPU oracle (one thread) on whole (sequence, head) units of the same
+    workload; the rate is per unit of algorithmic work, so it needs no scaling."""
     import numpy as np
     from oracle import pyoracle as oracle
     B, T, H, D = spec["B"], spec["T"], spec["H"], spec["D"]
     E = H * D
     rng = np.random.default_rng(1)
-    x = rng.standard_normal((T, 3 * E)).astype(np.float32)   # one sequence is enough
+    x = rng.standard_normal((T, 3 * E)).astype(np.float32)
     d_out = rng.standard_normal((T, E)).astype(np.float32)
-    bits = oracle.f32_to_bf16_bits(x).reshape(x.shape)
+    dtype = oracle.BF16 if spec["bf16"] else oracle.F32
+    data = oracle.f32_to_bf16_bits(x).reshape(x.shape) if spec["bf16"] else x
+    units, seconds = 0, 0.0
+    while seconds < 10.0 and units < H:
+        t0 = time.perf_counter()
+        out, _, _ = oracle.mha_fwd(data, T, H, dtype, (0, 1), (units, units + 1))
+        if spec["backward"]:
+            oracle.mha_bwd(data, out, d_out, T, H, dtype, (0, 1), (units, units + 1))
+        seconds += time.perf_counter() - t0
+        units += 1
+    flops = (14.0 if spec["backward"] else 4.0) * D * causal_pairs(T) * units
+    return dict(value=round(flops / seconds / 1e12, 6), unit="TFLOP/s", cores=1, kind="port",
+                sample="%d of %d (sequence, head) units of the workload, %s, %.1f s of CPU time" % (
+                    units, B * H, "forward+backward" if spec["backward"] else "forward", seconds))
+
+
+def measure(torch, w, steps, warmup):
+    stream = torch.cuda.current_stream()
+    for _ in range(warmup):
+        w["step"]()
+    torch.cuda.synchronize()
     t0 = time.perf_counter()
-    out, _, _ = oracle.mha_fwd(bits, T, H, oracle.BF16, (0, 1), (0, budget_units))
-    oracle.mha_bwd(bits, out, d_out, T, H, oracle.BF16, (0, 1), (0, budget_units))
-    seconds = time.perf_counter() - t0
-    flops = 14.0 * D * causal_pairs(T) * budget_units
-    return dict(value=flops / seconds / 1e12, unit="TFLOP/s", cores=1, kind="port",
-                sample="%d of %d (sequence, head) units, forward+backward, %.1f s" % (
-                    budget_units, B * H, seconds))
+    for _ in range(steps):
+        w["step"]()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / steps
+    parts = {}
+    for name, fn, work in w["parts"]:
+        pairs = []
+        for _ in range(steps):
+            start = torch.cuda.Event(enable_timing=True)
+            end = torch.cuda.Event(enable_timing=True)
+            start.record(stream)
+            fn()
+            end.record(stream)
+            pairs.append((start, end))
+        torch.cuda.synchronize()
+        parts[name] = (sum(s.elapsed_time(e) for s, e in pairs) / len(pairs), work)
+    dominant = max(parts, key=lambda k: parts[k][0])
+    dom_ms, dom_work = parts[dominant]
+    divisor = 1e12 if w["bound"] == "mfma" else 1e9
+    value = w["work"] / (ms_per_step * 1e-3) / divisor
+    achieved = dom_work / (dom_ms * 1e-3) / divisor
+    return dict(ms_per_step=ms_per_step, value=value, parts=parts, dominant=dominant,
+                achieved=achieved, kernel_ms=dom_ms)
 
 
 def main():
     args = parse_args()
     if args.gpus != 1:
-        print("bench.py measures one GPU: this build has no multi-GPU path "
-              "(run with --gpus 1)", file=sys.stderr)
+        print("bench.py measures one GPU: this build has no multi-GPU path (use --gpus 1)",
+              file=sys.stderr)
         sys.exit(2)
     import torch
     from pluto_amd import capi
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
     capi.lib()
-    if args.workload not in WORKLOADS:
-        print("workload %s is not built yet" % args.workload, file=sys.stderr)
-        sys.exit(2)
-    w = WORKLOADS[args.workload](args, torch, capi)
-    stream = torch.cuda.current_stream()
-    for _ in range(args.warmup):
-        w["step"]()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        w["step"]()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    ms_per_step = wall * 1e3 / args.steps
-    # Per-part device time with HIP events on the launch stream.
-    parts = {}
-    for name, fn, work in w["parts"]:
-        timer = EventTimer(torch, stream)
-        for _ in range(args.steps):
-            timer.time(fn)
-        torch.cuda.synchronize()
-        parts[name] = (timer.mean_ms(), work)
-    dominant = max(parts, key=lambda k: parts[k][0])
-    dom_ms, dom_work = parts[dominant]
-    if w["bound"] == "mfma":
-        value = w["flops"] / (ms_per_step * 1e-3) / 1e12
-        achieved = dom_work / (dom_ms * 1e-3) / 1e12
-        roof_unit = "TFLOP/s"
-    else:
-        value = w["bytes"] / (ms_per_step * 1e-3) / 1e9
-        achieved = dom_work / (dom_ms * 1e-3) / 1e9
-        roof_unit = "GB/s"
+    head = "mha_train_bf16" if args.workload == "all" else args.workload
+    w = WORKLOADS[head](torch, capi)
+    m = measure(torch, w, args.steps, args.warmup)
     result = {
-        "metric": w["metric"], "value": round(value, 3), "unit": w["unit"], "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "metric": w["metric"], "value": round(m["value"], 3), "unit": w["unit"], "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(m["ms_per_step"], 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": w["dtype"], "data": "synthetic", "config": w["config"],
-        "roofline": {"bound": w["bound"], "kernel": dominant, "achieved": round(achieved, 3),
-                     "peak": w["peak"], "unit": roof_unit,
-                     "frac": round(achieved / w["peak"], 4), "traffic": None,
-                     "kernel_ms": round(dom_ms, 4)},
-        "parts_ms": {k: round(v[0], 4) for k, v in parts.items()},
+        "roofline": {"bound": w["bound"], "kernel": m["dominant"],
+                     "achieved": round(m["achieved"], 3), "peak": w["peak"],
+                     "unit": "TFLOP/s" if w["bound"] == "mfma" else "GB/s",
+                     "frac": round(m["achieved"] / w["peak"], 4), "traffic": None,
+                     "kernel_ms": round(m["kernel_ms"], 4)},
+        "parts_ms": {k: round(v[0], 4) for k, v in m["parts"].items()},
     }
-    if not args.no_cpu_baseline:
-        kind, spec = w["cpu"]
-        result["cpu_baseline"] = cpu_baseline_mha(spec) if kind == "mha" else None
+    if not args.no_cpu_baseline and w["cpu"] is not None:
+        result["cpu_baseline"] = cpu_baseline_mha(w["cpu"][1])
+    if args.workload == "all":
+        others = {}
+        for name in NAMES:
+            if name == head:
+                continue
+            del w
+            torch.cuda.empty_cache()
+            w = WORKLOADS[name](torch, capi)
+            mm = measure(torch, w, max(args.steps // 2, 5), max(args.warmup // 2, 2))
+            others[name] = {"metric": w["metric"], "value": round(mm["value"], 3), "unit": w["unit"],
+                            "ms_per_step": round(mm["ms_per_step"], 4), "bound": w["bound"],
+                            "frac_of_peak": round(mm["value"] / w["peak"], 4), "config": w["config"]}
+        result["workloads"] = others
     print(json.dumps(result))
 
 

@@ -54,6 +54,7 @@ struct ChunkSmem {
   float beta[C];
   float inv_k[C];           // 1/|k| (or 1)
   float q_factor[C];        // q_scale / |q| (or q_scale)
+  float rhs_factor[2][C];   // [0]: beta (U columns), [1]: beta exp(c) / |k| (W columns)
 };
 
 __global__ void __launch_bounds__(256)
@@ -114,8 +115,11 @@ gdn_chunk_prepare(GdnArgs a) {
     qq += __shfl_xor(qq, 2, 64);
     if (part == 0) {
       // sequence_delta_net.cc:84-85: x * rsqrt(sum(x^2) + 1e-6)
-      sm.inv_k[row] = a.normalize_qk ? rsqrtf(kk + 1e-6f) : 1.0f;
+      const float inv_k = a.normalize_qk ? rsqrtf(kk + 1e-6f) : 1.0f;
+      sm.inv_k[row] = inv_k;
       sm.q_factor[row] = a.normalize_qk ? a.q_scale * rsqrtf(qq + 1e-6f) : a.q_scale;
+      sm.rhs_factor[0][row] = sm.beta[row];
+      sm.rhs_factor[1][row] = sm.beta[row] * __expf(sm.cum[row]) * inv_k;
     }
   }
   __syncthreads();
@@ -166,23 +170,27 @@ gdn_chunk_prepare(GdnArgs a) {
   {
     const bool is_u = tid < DV;
     const int c = is_u ? tid : tid - DV;
+    const uint16_t* column = is_u ? &sm.vw[0][c] : &sm.k[0][c];  // same row stride
+    const float* factor = sm.rhs_factor[is_u ? 0 : 1];
 #pragma unroll
     for (int i = 0; i < C; ++i) {
-      float rhs;
-      if (is_u)
-        rhs = sm.beta[i] * bf16_bits_to_float(sm.vw[i][c]);
-      else
-        rhs = sm.beta[i] * __expf(sm.cum[i]) * sm.inv_k[i] * bf16_bits_to_float(sm.k[i][c]);
-      float acc = rhs;
+      const float rhs = factor[i] * bf16_bits_to_float(column[i * (DK + 8)]);
+      // four partial sums shorten the dependent chain of a row
+      float acc0 = rhs, acc1 = 0.0f, acc2 = 0.0f, acc3 = 0.0f;
 #pragma unroll
       for (int j4 = 0; j4 < (i + 3) / 4; ++j4) {
         const float4 row = *reinterpret_cast<const float4*>(&sm.a[i][4 * j4]);
         // entries at or beyond the diagonal are zero
-        acc -= row.x * x[4 * j4];
-        if (4 * j4 + 1 < i) acc -= row.y * x[4 * j4 + 1];
-        if (4 * j4 + 2 < i) acc -= row.z * x[4 * j4 + 2];
-        if (4 * j4 + 3 < i) acc -= row.w * x[4 * j4 + 3];
+        acc0 -= row.x * x[4 * j4];
+        if (4 * j4 + 1 < i) acc1 -= row.y * x[4 * j4 + 1];
+        if (4 * j4 + 2 < i) acc2 -= row.z * x[4 * j4 + 2];
+        if (4 * j4 + 3 < i) acc3 -= row.w * x[4 * j4 + 3];
       }
+      const float acc = (acc0 + acc1) + (acc2 + acc3);
+      // keep the scheduler from hoisting later rows' LDS reads over this row:
+      // that only lengthens live ranges until registers spill
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_sched_barrier(0);
       x[i] = acc;
     }
   }
@@ -291,41 +299,67 @@ gdn_chunk_scan(GdnArgs a) {
     for (int r = 0; r < 4; ++r)
       s[t][r] = state[(16 * t + 4 * hq + r) * DV + 16 * slice + m];
 
-  for (int chunk = 0; chunk < chunks; ++chunk) {
-    const char* in = a.workspace + (static_cast<size_t>(bh) * chunks + chunk) * kGdnChunkBytes;
+  // Operands are fetched half an iteration ahead: the first-phase operands
+  // (U, -W, cQ) of chunk c+1 are requested before the second phase of chunk c
+  // runs, and the second-phase operands (A2, Kt) of chunk c before its first
+  // phase, so the dependent matrix-core chain does not wait on memory.
+  floatx4 u_reg[4];
+  uint4 w_reg[16], q_reg[16], a2_reg[8], kt_reg[16];
+  float decay = 1.0f;
+  const char* base = a.workspace + static_cast<size_t>(bh) * chunks * kGdnChunkBytes;
+  auto load_first = [&](int chunk) {
+    const char* in = base + static_cast<size_t>(chunk) * kGdnChunkBytes;
     const floatx4* u_in = reinterpret_cast<const floatx4*>(in + kGdnOffsetU);
     const uint4* neg_w = reinterpret_cast<const uint4*>(in + kGdnOffsetW);
     const uint4* q_in = reinterpret_cast<const uint4*>(in + kGdnOffsetQ);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) u_reg[i] = u_in[(i * SLICES + slice) * 64 + lane];
+#pragma unroll
+    for (int f = 0; f < 16; ++f) {
+      w_reg[f] = neg_w[f * 64 + lane];
+      q_reg[f] = q_in[f * 64 + lane];
+    }
+  };
+  auto load_second = [&](int chunk) {
+    const char* in = base + static_cast<size_t>(chunk) * kGdnChunkBytes;
     const uint4* a2_in = reinterpret_cast<const uint4*>(in + kGdnOffsetA2);
     const uint4* kt_in = reinterpret_cast<const uint4*>(in + kGdnOffsetKt);
-    const float decay = *reinterpret_cast<const float*>(in + kGdnOffsetDecay);
-
+#pragma unroll
+    for (int f = 0; f < 8; ++f) a2_reg[f] = a2_in[f * 64 + lane];
+#pragma unroll
+    for (int f = 0; f < 16; ++f) kt_reg[f] = kt_in[f * 64 + lane];
+    decay = *reinterpret_cast<const float*>(in + kGdnOffsetDecay);
+  };
+  load_first(0);
+  for (int chunk = 0; chunk < chunks; ++chunk) {
+    load_second(chunk);
     bf16x8 sb[4];
 #pragma unroll
     for (int kb = 0; kb < 4; ++kb) sb[kb] = tiles_to_operand(s[2 * kb], s[2 * kb + 1]);
-    // D = U - W S0
-    floatx4 d[4];
+    // D = U - W S0 and the S0 part of O = exp(c) Q S0 + (M o Q K^T) D
+    floatx4 d[4], o[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      floatx4 acc = u_in[(i * SLICES + slice) * 64 + lane];
+      floatx4 acc = u_reg[i];
+      floatx4 out_acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-      for (int kb = 0; kb < 4; ++kb)
-        acc = mfma16(bits_to_bf16x8(neg_w[(4 * i + kb) * 64 + lane]), sb[kb], acc);
+      for (int kb = 0; kb < 4; ++kb) {
+        acc = mfma16(bits_to_bf16x8(w_reg[4 * i + kb]), sb[kb], acc);
+        out_acc = mfma16(bits_to_bf16x8(q_reg[4 * i + kb]), sb[kb], out_acc);
+      }
       d[i] = acc;
+      o[i] = out_acc;
     }
+    if (chunk + 1 < chunks) load_first(chunk + 1);
     bf16x8 db[2];
     db[0] = tiles_to_operand(d[0], d[1]);
     db[1] = tiles_to_operand(d[2], d[3]);
-    // O = exp(c) Q S0 + (M o Q K^T) D
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      floatx4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-      for (int kb = 0; kb < 4; ++kb)
-        acc = mfma16(bits_to_bf16x8(q_in[(4 * i + kb) * 64 + lane]), sb[kb], acc);
+      floatx4 acc = o[i];
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb)
-        acc = mfma16(bits_to_bf16x8(a2_in[(2 * i + kb) * 64 + lane]), db[kb], acc);
+        acc = mfma16(bits_to_bf16x8(a2_reg[2 * i + kb]), db[kb], acc);
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int token = chunk * C + 16 * i + 4 * hq + r;
@@ -340,7 +374,7 @@ gdn_chunk_scan(GdnArgs a) {
       floatx4 acc = s[t] * decay;
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb)
-        acc = mfma16(bits_to_bf16x8(kt_in[(2 * t + kb) * 64 + lane]), db[kb], acc);
+        acc = mfma16(bits_to_bf16x8(kt_reg[2 * t + kb]), db[kb], acc);
       s[t] = acc;
     }
   }
