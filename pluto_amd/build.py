@@ -25,6 +25,9 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 DEVICE_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++20", "-fPIC", "-fno-exceptions",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # keep matrix-core accumulators in ordinary VGPRs: the softmax works on them
+    # directly, and AGPR accumulators cost a copy per element per tile
+    "-mllvm", "-amdgpu-mfma-vgpr-form",
     "-Wno-unused-command-line-argument",
     "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
 ]

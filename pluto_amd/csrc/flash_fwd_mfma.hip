@@ -90,8 +90,22 @@ flash_forward_kernel(FlashForwardArgs a) {
   for (int db = 0; db < DB; ++db)
 #pragma unroll
     for (int i = 0; i < 16; ++i) o_acc[db][i] = 0.0f;
-  float m2 = kMasked;  // running maximum of score * scale * log2(e)
-  float l_part = 0.0f; // this lane-half's share of the normalizer
+  // Online softmax in the log2 domain with a lazily updated reference point:
+  // probabilities are 2^(s*scale2 - m_used); m_used follows the running row
+  // maximum only when that has grown by more than kLazy, so the accumulator
+  // rescale is rare.  The true maximum is tracked separately and the saved
+  // statistics are converted to it at the end.
+  constexpr float kLazy = 8.0f;
+  float m_used = kMasked;   // reference point, score * scale * log2(e) units
+  float m_true = kMasked;   // running maximum of the raw scores
+  // Row sums come out of the matrix cores: an all-ones A operand makes every
+  // row of this accumulator the sum over keys of the bf16 probabilities.
+  floatx16 l_acc;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) l_acc[i] = 0.0f;
+  bf16x8 ones;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) ones[e] = static_cast<__bf16>(1.0f);
 
   const int last_row = min(q0 + BM, a.q_rows) - 1;
   const int visible = min(a.kv_rows, a.start_position + last_row + 1);
@@ -114,11 +128,11 @@ flash_forward_kernel(FlashForwardArgs a) {
       for (int i = 0; i < LOADS; ++i) {
         const int c = ltid + 128 * i;
         const int key = c / KCH, ch = c % KCH;
-        uint4 bits = make_uint4(0, 0, 0, 0);
-        if (k0 + key < a.kv_rows)
-          bits = *reinterpret_cast<const uint4*>(
-              k_base + static_cast<long long>(k0 + key) * a.k_row_stride + 8 * ch);
-        staged[i] = bits;
+        // rows beyond the valid prefix are clamped to its last row: their
+        // scores are masked, and a finite row keeps 0 * V finite
+        const int row = min(k0 + key, a.kv_rows - 1);
+        staged[i] = *reinterpret_cast<const uint4*>(
+            k_base + static_cast<long long>(row) * a.k_row_stride + 8 * ch);
       }
     } else {
       // unit = (key quad, channel group); 4 loads (one per key) per unit.
@@ -128,12 +142,9 @@ flash_forward_kernel(FlashForwardArgs a) {
         const int quad = unit / KCH, g = unit % KCH;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          const int key = k0 + 4 * quad + r;
-          uint4 bits = make_uint4(0, 0, 0, 0);
-          if (key < a.kv_rows)
-            bits = *reinterpret_cast<const uint4*>(
-                v_base + static_cast<long long>(key) * a.v_row_stride + 8 * g);
-          staged[4 * u + r] = bits;
+          const int row = min(k0 + 4 * quad + r, a.kv_rows - 1);
+          staged[4 * u + r] = *reinterpret_cast<const uint4*>(
+              v_base + static_cast<long long>(row) * a.v_row_stride + 8 * g);
         }
       }
     }
@@ -181,48 +192,54 @@ flash_forward_kernel(FlashForwardArgs a) {
         s[kb] = mfma32(kf, qf[ks], s[kb]);
       }
     }
-    // ---- mask, row maximum --------------------------------------------
+    // ---- mask (diagonal and tail tiles only), row maximum ----------------
     const bool needs_mask =
         (k0 + BN - 1 > a.start_position + q0 + 32 * wave) || (k0 + BN > a.kv_rows);
+    if (needs_mask) {
+      // keys up to `limit` are visible to this lane's query
+      const int limit = min(a.start_position + q_row, a.kv_rows - 1) - k0 - 4 * h;
+#pragma unroll
+      for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+          s[kb][i] = (32 * kb + 8 * (i / 4) + (i % 4) > limit) ? kMasked : s[kb][i];
+    }
     float row_max = kMasked;
 #pragma unroll
     for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        float t = s[kb][i] * scale2;
-        if (needs_mask) {
-          const int key = k0 + 32 * kb + 8 * (i / 4) + 4 * h + (i % 4);
-          if (key > a.start_position + q_row || key >= a.kv_rows) t = kMasked;
-        }
-        s[kb][i] = t;
-        row_max = fmaxf(row_max, t);
-      }
+      for (int i = 0; i < 16; i += 2) row_max = fmaxf(row_max, fmaxf(s[kb][i], s[kb][i + 1]));
     row_max = fmaxf(row_max, __shfl_xor(row_max, 32, 64));
-    const float m_new = fmaxf(m2, row_max);
-    const float alpha = __builtin_amdgcn_exp2f(m2 - m_new);
-    m2 = m_new;
-    float sum = 0.0f;
+    m_true = fmaxf(m_true, row_max);
+    const float candidate = m_true * scale2;
+    const bool grow = candidate > m_used + kLazy;
+    if (__any(grow)) {
+      const float m_new = grow ? candidate : m_used;
+      const float alpha = __builtin_amdgcn_exp2f(m_used - m_new);
+      m_used = m_new;
+      l_acc[0] *= alpha;
 #pragma unroll
-    for (int kb = 0; kb < KB; ++kb)
+      for (int db = 0; db < DB; ++db)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const float p = __builtin_amdgcn_exp2f(s[kb][i] - m_new);
-        s[kb][i] = p;
-        sum += p;
-      }
-    l_part = l_part * alpha + sum;
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) o_acc[db][i] *= alpha;
-    // ---- O^T += V^T P^T -------------------------------------------------
+        for (int i = 0; i < 16; ++i) o_acc[db][i] *= alpha;
+    }
+    // ---- P^T = 2^(S^T scale2 - m_used);  O^T += V^T P^T;  l += 1^T P^T ---
 #pragma unroll
     for (int kb = 0; kb < KB; ++kb) {
       if (k0 + 32 * kb > wave_last_key) continue;
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2) {
-        const bf16x8 pf = accumulator_to_operand(s[kb], s2);
+        uint32_t packed[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          floatx2 pair;
+          pair[0] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kb][8 * s2 + 2 * e], scale2, -m_used));
+          pair[1] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kb][8 * s2 + 2 * e + 1], scale2, -m_used));
+          packed[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, bf16x2));
+        }
+        const bf16x8 pf = __builtin_bit_cast(bf16x8, make_uint4(packed[0], packed[1], packed[2], packed[3]));
         const int chunk = 4 * kb + 2 * s2 + h;
+        l_acc = mfma32(ones, pf, l_acc);
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
           const int d = 32 * db + n;
@@ -234,9 +251,12 @@ flash_forward_kernel(FlashForwardArgs a) {
   }
 
   // ---- epilogue ------------------------------------------------------------
-  const float l_total = l_part + __shfl_xor(l_part, 32, 64);
-  const float normalizer = l_total > 0.0f ? l_total : 1.0f;
-  const float inverse = 1.0f / normalizer;
+  // l_acc already holds the sum over all keys (both lane halves contract
+  // into the same accumulator column).
+  const float l_used = l_acc[0] > 0.0f ? l_acc[0] : 1.0f;
+  const float inverse = 1.0f / l_used;
+  // statistics relative to the true maximum: attention.cc:161-168
+  const float normalizer = l_used * __builtin_amdgcn_exp2f(m_used - m_true * scale2);
   __syncthreads();  // LDS is reused to transpose the output tile
   {
     unsigned char* row = raw + (32 * wave + n) * OSTRIDE;
@@ -253,7 +273,7 @@ flash_forward_kernel(FlashForwardArgs a) {
       }
   }
   if (h == 0 && q_row < a.q_rows) {
-    const float maximum = m2 * (1.0f / kLog2e);
+    const float maximum = m_true * a.scale;
     const long long stat =
         (static_cast<long long>(seq) * a.query_heads + head) * a.q_rows + q_row;
     if (a.maxima) a.maxima[stat] = maximum;
