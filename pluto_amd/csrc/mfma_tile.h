@@ -65,12 +65,19 @@ __device__ inline void transposed_store(uint4* tile, int quad, int g, uint4 r0,
   }
 }
 
+// Two floats to packed bf16 (one v_cvt_pk_bf16_f32).
+__device__ inline uint32_t pack_bf16(float lo, float hi) {
+  floatx2 two = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(two, bf16x2));
+}
+
 // Accumulator registers 8*s2 .. 8*s2+7 as a bf16 B operand.
 __device__ inline bf16x8 accumulator_to_operand(const floatx16& acc, int s2) {
-  bf16x8 out;
-#pragma unroll
-  for (int e = 0; e < 8; ++e) out[e] = static_cast<__bf16>(acc[8 * s2 + e]);
-  return out;
+  return __builtin_bit_cast(
+      bf16x8, make_uint4(pack_bf16(acc[8 * s2 + 0], acc[8 * s2 + 1]),
+                         pack_bf16(acc[8 * s2 + 2], acc[8 * s2 + 3]),
+                         pack_bf16(acc[8 * s2 + 4], acc[8 * s2 + 5]),
+                         pack_bf16(acc[8 * s2 + 6], acc[8 * s2 + 7])));
 }
 
 __device__ inline floatx16 mfma32(bf16x8 a, bf16x8 b, floatx16 c) {
