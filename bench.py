@@ -30,7 +30,19 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA (published)
 PEAK_FP32_TFLOPS = 157.3    # MI355X fp32 matrix (published)
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E (published)
 
+# HBM bytes per step of a kernel group, from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE runs of this file (FETCH_SIZE x 2.0 KiB and WRITE_SIZE x 1.0 KiB,
+# the factors a 1 GiB device copy gives: `--workload copy`).  The summaries are
+# kept as profiles/*_hbm_traffic.md.  None = not measured.
+MEASURED_TRAFFIC_BYTES = {
+    ("mha_train_bf16", "forward"): 146.7e6,
+    ("mha_train_bf16", "backward"): 566.3e6,
+}
+
 NAMES = ["mha_train_bf16", "mha_fwd_fp32", "gqa_prefill", "gqa_decode", "gdn_scan"]
+# "copy" is a plain device copy of known size: the calibration case for the
+# FETCH_SIZE / WRITE_SIZE counters that `roofline.traffic` is derived from.
+EXTRA = ["copy"]
 
 
 def parse_args():
@@ -38,7 +50,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="mha_train_bf16", choices=NAMES + ["all"])
+    ap.add_argument("--workload", default="mha_train_bf16", choices=NAMES + EXTRA + ["all"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     return ap.parse_args()
 
@@ -200,7 +212,22 @@ def gdn_scan(torch, capi):
                 cpu=None)
 
 
-WORKLOADS = {"mha_train_bf16": mha_train_bf16, "mha_fwd_fp32": mha_fwd_fp32,
+def copy(torch, capi):
+    n = 256 * 2 ** 20   # 1 GiB read + 1 GiB written per step
+    src = torch.ones(n, dtype=torch.float32, device="cuda")
+    dst = torch.empty_like(src)
+
+    def step():
+        dst.copy_(src)
+
+    work = 2.0 * n * 4
+    return dict(step=step, parts=[("copy", step, work)], work=work, metric="device_copy_gbs",
+                unit="GB/s", dtype="f32", bound="hbm", peak=PEAK_HBM_GBS,
+                config={"workload": "device_copy_calibration", "bytes_read": n * 4,
+                        "bytes_written": n * 4}, cpu=None)
+
+
+WORKLOADS = {"copy": copy, "mha_train_bf16": mha_train_bf16, "mha_fwd_fp32": mha_fwd_fp32,
              "gqa_prefill": gqa_prefill, "gqa_decode": gqa_decode, "gdn_scan": gdn_scan}
 
 
@@ -283,7 +310,8 @@ def main():
         "roofline": {"bound": w["bound"], "kernel": m["dominant"],
                      "achieved": round(m["achieved"], 3), "peak": w["peak"],
                      "unit": "TFLOP/s" if w["bound"] == "mfma" else "GB/s",
-                     "frac": round(m["achieved"] / w["peak"], 4), "traffic": None,
+                     "frac": round(m["achieved"] / w["peak"], 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get((head, m["dominant"])),
                      "kernel_ms": round(m["kernel_ms"], 4)},
         "parts_ms": {k: round(v[0], 4) for k, v in m["parts"].items()},
     }
