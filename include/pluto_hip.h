@@ -275,6 +275,42 @@ int pluto_hip_gdn_recurrence(void* stream, const pluto_hip_delta_params* p,
                              int normalize_qk, float q_scale, float* state,
                              void* out, int out_dtype);
 
+/* Whole gated delta-net layer over sequences; semantics of
+ * SequenceDeltaNetLayer::fwd_impl (src/llm/layers/sequence_delta_net.cc:435-480:
+ * ConvForward :31-51, RecurrenceForward :55-102, OutputForward :104-121) for
+ * `batch` independent sequences, each starting from an empty convolution history.
+ *   qkv  bf16 [batch, length, 2*kh*kd + vh*vd], packed [all Q | all K | all V]
+ *   z    bf16 [batch, length, vh*vd];  a, b  bf16 [batch, length, vh]
+ *   conv_weight fp32 [channels, kernel]; a_log, dt_bias fp32 [vh]; norm fp32 [vd]
+ *   state fp32 [batch, vh, kd, vd], read as the initial recurrent state (zeros for
+ *        the reference's behaviour) and overwritten with the final one
+ *   out  bf16 [batch, length, vh*vd]
+ * The per-token state snapshots the reference saves for its backward pass are
+ * not produced. */
+size_t pluto_hip_gdn_layer_workspace_bytes(const pluto_hip_delta_params* p,
+                                           int batch, int length);
+int pluto_hip_gdn_layer_forward(void* stream, const pluto_hip_delta_params* p,
+                                int batch, int length, const void* qkv,
+                                const void* z, const void* a, const void* b,
+                                const float* conv_weight, const float* a_log,
+                                const float* dt_bias, const float* norm,
+                                float* state, void* out, void* workspace,
+                                size_t workspace_bytes);
+
+/* DeltaNetState::Step (src/llm/layers/util/cached_attention_ops.cc:401-431:
+ * ConvolutionKernel :180-203, DeltaRecurrenceKernel :205-251, DeltaOutputKernel
+ * :253-272): one token, contiguous FP32 device arrays as in the reference.
+ *   conv_state fp32 [channels, kernel] and recurrent_state fp32 [vh, kd, vd]
+ *   are updated in place (DeltaNetState::Reset = zero both). */
+size_t pluto_hip_gdn_step_workspace_bytes(const pluto_hip_delta_params* p);
+int pluto_hip_gdn_step(void* stream, const pluto_hip_delta_params* p,
+                       float* conv_state, float* recurrent_state,
+                       const float* qkv, const float* z, const float* a,
+                       const float* b, const float* conv_weight,
+                       const float* a_log, const float* dt_bias,
+                       const float* norm, float* output, void* workspace,
+                       size_t workspace_bytes);
+
 #ifdef __cplusplus
 }
 #endif

@@ -103,6 +103,11 @@ SIGNATURES = {
     "pluto_hip_gdn_scan_workspace_bytes": (_SZ, [ctypes.POINTER(DeltaParams), _I, _I, _I]),
     "pluto_hip_gdn_scan": (_I, [_VP, ctypes.POINTER(DeltaParams), _I, _I, _I, _VP, _VP,
                                 _VP, _VP, _VP, _I, ctypes.c_float, _VP, _VP, _VP, _SZ]),
+    "pluto_hip_gdn_layer_workspace_bytes": (_SZ, [ctypes.POINTER(DeltaParams), _I, _I]),
+    "pluto_hip_gdn_layer_forward": (_I, [_VP, ctypes.POINTER(DeltaParams), _I, _I] + [_VP] * 10 +
+                                    [_VP, _SZ]),
+    "pluto_hip_gdn_step_workspace_bytes": (_SZ, [ctypes.POINTER(DeltaParams)]),
+    "pluto_hip_gdn_step": (_I, [_VP, ctypes.POINTER(DeltaParams)] + [_VP] * 11 + [_VP, _SZ]),
     "pluto_hip_gdn_recurrence": (_I, [_VP, ctypes.POINTER(DeltaParams), _I, _I, _VP, _VP,
                                       _VP, _VP, _VP, _I, ctypes.c_float, _VP, _VP, _I]),
 }
@@ -334,3 +339,42 @@ def gdn_recurrence(p, q, k, v, log_decay, beta, state, normalize_qk=False, q_sca
                                          ptr(beta), int(bool(normalize_qk)), float(q_scale),
                                          ptr(state), ptr(out), dtype_code(out)))
     return out
+
+
+def gdn_layer_forward(p, qkv, z, a, b, conv_weight, a_log, dt_bias, norm, state, stream=None):
+    """Whole delta-net layer: qkv bf16 [B, T, channels], z bf16 [B, T, vh*vd], a/b bf16
+    [B, T, vh]; state fp32 [B, vh, kd, vd] updated in place.  Returns out bf16 [B, T, vh*vd]."""
+    batch, length = qkv.shape[0], qkv.shape[1]
+    size = lib().pluto_hip_gdn_layer_workspace_bytes(ctypes.byref(p), batch, length)
+    workspace = torch.empty(max(size, 16), dtype=torch.uint8, device=qkv.device)
+    out = torch.empty(z.shape, dtype=torch.bfloat16, device=qkv.device)
+    check(lib().pluto_hip_gdn_layer_forward(stream or current_stream(), ctypes.byref(p), batch,
+                                            length, ptr(qkv), ptr(z), ptr(a), ptr(b),
+                                            ptr(conv_weight), ptr(a_log), ptr(dt_bias), ptr(norm),
+                                            ptr(state), ptr(out), ptr(workspace), workspace.numel()))
+    return out
+
+
+class DeltaNetStep:
+    """Single-token delta-net state (DeltaNetState of the reference): fp32 arrays."""
+
+    def __init__(self, p, device="cuda"):
+        self.p = p
+        channels = 2 * p.key_heads * p.key_head_dim + p.value_heads * p.value_head_dim
+        self.conv = torch.zeros((channels, p.conv_kernel_dim), device=device)
+        self.state = torch.zeros((p.value_heads, p.key_head_dim, p.value_head_dim), device=device)
+        size = lib().pluto_hip_gdn_step_workspace_bytes(ctypes.byref(p))
+        self.workspace = torch.empty(max(size, 16), dtype=torch.uint8, device=device)
+
+    def reset(self):
+        self.conv.zero_()
+        self.state.zero_()
+
+    def step(self, qkv, z, a, b, conv_weight, a_log, dt_bias, norm, stream=None):
+        p = self.p
+        out = torch.empty(p.value_heads * p.value_head_dim, device=qkv.device)
+        check(lib().pluto_hip_gdn_step(stream or current_stream(), ctypes.byref(p), ptr(self.conv),
+                                       ptr(self.state), ptr(qkv), ptr(z), ptr(a), ptr(b),
+                                       ptr(conv_weight), ptr(a_log), ptr(dt_bias), ptr(norm),
+                                       ptr(out), ptr(self.workspace), self.workspace.numel()))
+        return out

@@ -23,9 +23,14 @@ constexpr size_t kGdnOffsetDecay = 90112;
 constexpr size_t kGdnChunkBytes = 90368;
 
 struct GdnArgs {
-  const uint16_t* q = nullptr;  // bf16 [batch, T, kh, kd]
+  // Row `token` (= sequence * T + t) of q starts at q + token * q_token_stride
+  // elements, head h at + h * kd; likewise k and v (head h at + h * vd).
+  // bf16 for the chunked scan; the recurrence kernel also reads fp32.
+  const uint16_t* q = nullptr;
   const uint16_t* k = nullptr;
-  const uint16_t* v = nullptr;  // bf16 [batch, T, vh, vd]
+  const uint16_t* v = nullptr;
+  long long q_token_stride = 0, k_token_stride = 0, v_token_stride = 0;
+  int in_dtype = PLUTO_HIP_BF16;
   const float* log_decay = nullptr;  // [batch, T, vh]
   const float* beta = nullptr;
   float* state = nullptr;   // fp32 [batch, vh, kd, vd]
@@ -42,5 +47,25 @@ struct GdnArgs {
 bool gdn_chunked_supported(const GdnArgs& args, int chunk);
 int launch_gdn_chunked(hipStream_t stream, const GdnArgs& args);
 int launch_gdn_recurrence(hipStream_t stream, const GdnArgs& args, int out_dtype);
+
+// Layer-level pieces around the scan (gdn_layer.hip).
+// Causal depthwise convolution + SiLU over whole sequences with zero history:
+// ConvForward, src/llm/layers/sequence_delta_net.cc:31-51.
+int launch_gdn_conv_sequence(hipStream_t stream, const void* input, int in_dtype,
+                             const float* weight, int batch, int length, int channels,
+                             int kernel, bool round, void* post, int post_dtype);
+// One token against a [channels, kernel] shift register: ConvolutionKernel,
+// src/llm/layers/util/cached_attention_ops.cc:180-203.
+int launch_gdn_conv_step(hipStream_t stream, const float* input, const float* weight,
+                         int channels, int kernel, bool round, float* state, float* output);
+// g = -exp(A_log) softplus(a + dt_bias), beta = round(sigmoid(b)):
+// sequence_delta_net.cc:88-96.
+int launch_gdn_gates(hipStream_t stream, const void* a, const void* b, int in_dtype,
+                     const float* a_log, const float* dt_bias, long long rows, int heads,
+                     bool round, float* log_decay, float* beta);
+// RMSNorm (plain weight) x SiLU(z): OutputForward, sequence_delta_net.cc:104-121.
+int launch_gdn_output(hipStream_t stream, const void* core, int core_dtype, const void* z,
+                      int z_dtype, const float* norm, long long rows, int value_dim,
+                      float epsilon, bool round, void* out, int out_dtype);
 
 }  // namespace pluto_hip

@@ -26,6 +26,8 @@ GdnArgs make_args(const pluto_hip_delta_params* p, int batch, int length, const 
   a.q = static_cast<const uint16_t*>(q);
   a.k = static_cast<const uint16_t*>(k);
   a.v = static_cast<const uint16_t*>(v);
+  a.q_token_stride = a.k_token_stride = 1LL * p->key_heads * p->key_head_dim;
+  a.v_token_stride = 1LL * p->value_heads * p->value_head_dim;
   a.log_decay = log_decay;
   a.beta = beta;
   a.state = state;
@@ -39,6 +41,31 @@ GdnArgs make_args(const pluto_hip_delta_params* p, int batch, int length, const 
   a.round_output = p->round_to_bfloat16;
   a.q_scale = q_scale;
   return a;
+}
+
+struct LayerLayout {
+  size_t post, log_decay, beta, core, scan, total;
+};
+
+size_t chunk_scratch_bytes(const pluto_hip_delta_params* p, int batch, int length) {
+  if (p->key_head_dim != 128 || p->value_head_dim != 128) return 0;
+  const size_t chunks = (static_cast<size_t>(length) + 63) / 64;
+  return static_cast<size_t>(batch) * p->value_heads * chunks * kGdnChunkBytes;
+}
+
+LayerLayout layer_layout(const pluto_hip_delta_params* p, int batch, int length) {
+  const size_t tokens = static_cast<size_t>(batch) * length;
+  const size_t channels = 2 * static_cast<size_t>(p->key_heads) * p->key_head_dim +
+                          static_cast<size_t>(p->value_heads) * p->value_head_dim;
+  const size_t element = p->round_to_bfloat16 ? 2 : 4;
+  LayerLayout l{};
+  l.post = 0;
+  l.log_decay = align_up(tokens * channels * element, 256);
+  l.beta = l.log_decay + align_up(tokens * p->value_heads * 4, 256);
+  l.core = l.beta + align_up(tokens * p->value_heads * 4, 256);
+  l.scan = l.core + align_up(tokens * p->value_heads * p->value_head_dim * element, 256);
+  l.total = l.scan + (p->round_to_bfloat16 ? chunk_scratch_bytes(p, batch, length) : 0) + 256;
+  return l;
 }
 
 }  // namespace
@@ -92,6 +119,135 @@ int pluto_hip_gdn_recurrence(void* stream, const pluto_hip_delta_params* p, int 
   GdnArgs a = make_args(p, batch, length, q, k, v, log_decay, beta, normalize_qk, q_scale, state);
   a.out_any = out;
   return launch_gdn_recurrence(static_cast<hipStream_t>(stream), a, out_dtype);
+}
+
+size_t pluto_hip_gdn_layer_workspace_bytes(const pluto_hip_delta_params* p, int batch,
+                                           int length) {
+  if (validate_delta(p) != 0 || batch <= 0 || length <= 0) return 0;
+  return layer_layout(p, batch, length).total;
+}
+
+int pluto_hip_gdn_layer_forward(void* stream, const pluto_hip_delta_params* p, int batch,
+                                int length, const void* qkv, const void* z, const void* a,
+                                const void* b, const float* conv_weight, const float* a_log,
+                                const float* dt_bias, const float* norm, float* state,
+                                void* out, void* workspace, size_t workspace_bytes) {
+  int status = validate_delta(p);
+  if (status != 0) return status;
+  if (batch <= 0 || length <= 0) return PLUTO_HIP_EINVAL;
+  if (!qkv || !z || !a || !b || !conv_weight || !a_log || !dt_bias || !norm || !state || !out)
+    return PLUTO_HIP_EINVAL;
+  const LayerLayout layout = layer_layout(p, batch, length);
+  if (!workspace || workspace_bytes < layout.total) return PLUTO_HIP_EWORKSPACE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  char* scratch = static_cast<char*>(workspace);
+  const bool round = p->round_to_bfloat16 != 0;
+  const int mid_dtype = round ? PLUTO_HIP_BF16 : PLUTO_HIP_F32;
+  const int kh = p->key_heads, vh = p->value_heads, kd = p->key_head_dim, vd = p->value_head_dim;
+  const int channels = 2 * kh * kd + vh * vd;
+  const long long tokens = static_cast<long long>(batch) * length;
+  void* post = scratch + layout.post;
+  float* log_decay = reinterpret_cast<float*>(scratch + layout.log_decay);
+  float* beta = reinterpret_cast<float*>(scratch + layout.beta);
+  void* core = scratch + layout.core;
+  status = launch_gdn_conv_sequence(s, qkv, PLUTO_HIP_BF16, conv_weight, batch, length, channels,
+                                    p->conv_kernel_dim, round, post, mid_dtype);
+  if (status != 0) return status;
+  status = launch_gdn_gates(s, a, b, PLUTO_HIP_BF16, a_log, dt_bias, tokens, vh, round,
+                            log_decay, beta);
+  if (status != 0) return status;
+  const size_t element = round ? 2 : 4;
+  GdnArgs g;
+  g.q = static_cast<const uint16_t*>(post);
+  g.k = reinterpret_cast<const uint16_t*>(static_cast<char*>(post) + element * kh * kd);
+  g.v = reinterpret_cast<const uint16_t*>(static_cast<char*>(post) + element * 2 * kh * kd);
+  g.q_token_stride = g.k_token_stride = g.v_token_stride = channels;
+  g.in_dtype = mid_dtype;
+  g.log_decay = log_decay;
+  g.beta = beta;
+  g.state = state;
+  g.out = static_cast<uint16_t*>(core);
+  g.out_any = core;
+  g.workspace = scratch + layout.scan;
+  g.batch = batch;
+  g.length = length;
+  g.key_heads = kh;
+  g.value_heads = vh;
+  g.key_dim = kd;
+  g.value_dim = vd;
+  g.normalize_qk = 1;  // sequence_delta_net.cc:84-85
+  g.round_output = round;
+  g.q_scale = 1.0f / std::sqrt(static_cast<float>(kd));
+  if (round && !force_generic() && gdn_chunked_supported(g, 64))
+    status = launch_gdn_chunked(s, g);
+  else
+    status = launch_gdn_recurrence(s, g, mid_dtype);
+  if (status != 0) return status;
+  return launch_gdn_output(s, core, mid_dtype, z, PLUTO_HIP_BF16, norm, tokens * vh, vd,
+                           p->rms_norm_epsilon, round, out, PLUTO_HIP_BF16);
+}
+
+size_t pluto_hip_gdn_step_workspace_bytes(const pluto_hip_delta_params* p) {
+  if (validate_delta(p) != 0) return 0;
+  const size_t channels = 2 * static_cast<size_t>(p->key_heads) * p->key_head_dim +
+                          static_cast<size_t>(p->value_heads) * p->value_head_dim;
+  return align_up(channels * 4, 256) + 2 * align_up(static_cast<size_t>(p->value_heads) * 4, 256) +
+         align_up(static_cast<size_t>(p->value_heads) * p->value_head_dim * 4, 256);
+}
+
+int pluto_hip_gdn_step(void* stream, const pluto_hip_delta_params* p, float* conv_state,
+                       float* recurrent_state, const float* qkv, const float* z,
+                       const float* a, const float* b, const float* conv_weight,
+                       const float* a_log, const float* dt_bias, const float* norm,
+                       float* output, void* workspace, size_t workspace_bytes) {
+  int status = validate_delta(p);
+  if (status != 0) return status;
+  // cached_attention_ops.cc:405-408
+  if (!conv_state || !recurrent_state || !qkv || !z || !a || !b || !conv_weight || !a_log ||
+      !dt_bias || !norm || !output)
+    return PLUTO_HIP_EINVAL;
+  if (!workspace || workspace_bytes < pluto_hip_gdn_step_workspace_bytes(p))
+    return PLUTO_HIP_EWORKSPACE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool round = p->round_to_bfloat16 != 0;
+  const int kh = p->key_heads, vh = p->value_heads, kd = p->key_head_dim, vd = p->value_head_dim;
+  const int channels = 2 * kh * kd + vh * vd;
+  char* scratch = static_cast<char*>(workspace);
+  float* convolved = reinterpret_cast<float*>(scratch);
+  size_t offset = align_up(static_cast<size_t>(channels) * 4, 256);
+  float* log_decay = reinterpret_cast<float*>(scratch + offset);
+  offset += align_up(static_cast<size_t>(vh) * 4, 256);
+  float* beta = reinterpret_cast<float*>(scratch + offset);
+  offset += align_up(static_cast<size_t>(vh) * 4, 256);
+  float* core = reinterpret_cast<float*>(scratch + offset);
+  status = launch_gdn_conv_step(s, qkv, conv_weight, channels, p->conv_kernel_dim, round,
+                                conv_state, convolved);
+  if (status != 0) return status;
+  status = launch_gdn_gates(s, a, b, PLUTO_HIP_F32, a_log, dt_bias, 1, vh, round, log_decay, beta);
+  if (status != 0) return status;
+  GdnArgs g;
+  g.q = reinterpret_cast<const uint16_t*>(convolved);
+  g.k = reinterpret_cast<const uint16_t*>(convolved + kh * kd);
+  g.v = reinterpret_cast<const uint16_t*>(convolved + 2 * kh * kd);
+  g.q_token_stride = g.k_token_stride = g.v_token_stride = channels;
+  g.in_dtype = PLUTO_HIP_F32;
+  g.log_decay = log_decay;
+  g.beta = beta;
+  g.state = recurrent_state;
+  g.out_any = core;
+  g.batch = 1;
+  g.length = 1;
+  g.key_heads = kh;
+  g.value_heads = vh;
+  g.key_dim = kd;
+  g.value_dim = vd;
+  g.normalize_qk = 1;  // cached_attention_ops.cc:224-228
+  g.round_output = round;
+  g.q_scale = 1.0f / std::sqrt(static_cast<float>(kd));
+  status = launch_gdn_recurrence(s, g, PLUTO_HIP_F32);
+  if (status != 0) return status;
+  return launch_gdn_output(s, core, PLUTO_HIP_F32, z, PLUTO_HIP_F32, norm, vh, vd,
+                           p->rms_norm_epsilon, round, output, PLUTO_HIP_F32);
 }
 
 }  // extern "C"

@@ -75,9 +75,9 @@ gdn_chunk_prepare(GdnArgs a) {
     uint4 kb = make_uint4(0, 0, 0, 0), qb = kb, vb = kb;
     if (row < valid) {
       const long long token = static_cast<long long>(seq) * a.length + t0 + row;
-      kb = *reinterpret_cast<const uint4*>(a.k + (token * a.key_heads + key_head) * DK + 8 * c8);
-      qb = *reinterpret_cast<const uint4*>(a.q + (token * a.key_heads + key_head) * DK + 8 * c8);
-      vb = *reinterpret_cast<const uint4*>(a.v + (token * a.value_heads + head) * DV + 8 * c8);
+      kb = *reinterpret_cast<const uint4*>(a.k + token * a.k_token_stride + key_head * DK + 8 * c8);
+      qb = *reinterpret_cast<const uint4*>(a.q + token * a.q_token_stride + key_head * DK + 8 * c8);
+      vb = *reinterpret_cast<const uint4*>(a.v + token * a.v_token_stride + head * DV + 8 * c8);
     }
     *reinterpret_cast<uint4*>(&sm.k[row][8 * c8]) = kb;
     *reinterpret_cast<uint4*>(&sm.q[row][8 * c8]) = qb;
@@ -409,8 +409,8 @@ gdn_recurrence_kernel(GdnArgs a, int out_dtype) {
     __syncthreads();
     if (threadIdx.x < 128) {
       const int d = threadIdx.x;
-      ks[d] = d < kd ? bf16_bits_to_float(a.k[(token * a.key_heads + key_head) * kd + d]) : 0.0f;
-      qs[d] = d < kd ? bf16_bits_to_float(a.q[(token * a.key_heads + key_head) * kd + d]) : 0.0f;
+      ks[d] = d < kd ? load_element(a.k, token * a.k_token_stride + key_head * kd + d, a.in_dtype) : 0.0f;
+      qs[d] = d < kd ? load_element(a.q, token * a.q_token_stride + key_head * kd + d, a.in_dtype) : 0.0f;
     }
     __syncthreads();
     float k_factor = 1.0f, q_factor = a.q_scale;
@@ -427,7 +427,7 @@ gdn_recurrence_kernel(GdnArgs a, int out_dtype) {
     const float decay = __expf(a.log_decay[scalar]);
     const float beta = a.beta[scalar];
     float value = 0.0f;
-    if (active) value = bf16_bits_to_float(a.v[(token * a.value_heads + head) * vd + column]);
+    if (active) value = load_element(a.v, token * a.v_token_stride + head * vd + column, a.in_dtype);
     float prediction = 0.0f;
 #pragma unroll
     for (int d = 0; d < 128; ++d) {
@@ -462,8 +462,9 @@ gdn_recurrence_kernel(GdnArgs a, int out_dtype) {
 
 bool gdn_chunked_supported(const GdnArgs& a, int chunk) {
   auto aligned = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
-  return chunk == C && a.key_dim == DK && a.value_dim == DV && aligned(a.q) && aligned(a.k) &&
-         aligned(a.v) && aligned(a.workspace);
+  return chunk == C && a.key_dim == DK && a.value_dim == DV && a.in_dtype == PLUTO_HIP_BF16 &&
+         a.q_token_stride % 8 == 0 && a.k_token_stride % 8 == 0 && a.v_token_stride % 8 == 0 &&
+         aligned(a.q) && aligned(a.k) && aligned(a.v) && aligned(a.workspace);
 }
 
 int launch_gdn_chunked(hipStream_t stream, const GdnArgs& a) {

@@ -179,3 +179,83 @@ def test_rejects_bad_arguments(capi):
     code = capi.lib().pluto_hip_gdn_recurrence(capi.current_stream(), p, 1, 1, None, None, None,
                                                None, None, 0, 1.0, None, None, capi.F32)
     assert code == capi.EINVAL
+
+
+def values(count, phase, scale=1.0):
+    i = np.arange(count, dtype=np.float32)
+    return (np.float32(scale) * np.sin(np.float32(phase) + i * np.float32(0.29))).astype(np.float32)
+
+
+def layer_weights(kh, vh, kd, vd, kernel):
+    channels = 2 * kh * kd + vh * vd
+    return (values(channels * kernel, 0.73, 0.6).reshape(channels, kernel), values(vh, 0.18, 0.5),
+            values(vh, -0.7, 0.3), values(vd, 0.5, 0.6))
+
+
+@pytest.mark.parametrize("round_flag", [False, True])
+@pytest.mark.parametrize("dim", [5, 128])
+def test_single_token_step_matches_scalar_specification(capi, oracle, dim, round_flag):
+    # cached_attention_ops_test.cc:400-470
+    kh, vh, kd, vd = 2, 6, dim, (7 if dim == 5 else 128)
+    p = capi.delta_params(kh, vh, kd, vd, round_to_bfloat16=round_flag)
+    po = oracle.delta_params(kh, vh, kd, vd, round_to_bfloat16=round_flag)
+    channels = 2 * kh * kd + vh * vd
+    w, a_log, dt, norm = layer_weights(kh, vh, kd, vd, 4)
+    dw, dal, ddt, dn = dev(w), dev(a_log), dev(dt), dev(norm)
+    state = capi.DeltaNetStep(p)
+    reference = oracle.DeltaNetStep(po)
+    first = None
+    for step in range(7):
+        t = 0 if step == 6 else step
+        if step == 6:
+            state.reset()
+        qkv = values(channels, 0.3 + t * 0.71)
+        z = values(vh * vd, -0.6 + t * 0.27)
+        a = values(vh, 0.1 + t * 0.1)
+        b = values(vh, -0.7 + t * 0.3)
+        a[0], a[1] = 100.0, -100.0   # softplus at both extremes
+        got = state.step(dev(qkv), dev(z), dev(a), dev(b), dw, dal, ddt, dn).cpu().numpy()
+        assert np.all(np.isfinite(got))
+        if step < 6:
+            want = reference.step(qkv, z, a, b, w, a_log, dt, norm)
+            bound = (2e-4 + 8e-3 * np.abs(want)) if round_flag else (3e-5 + 1e-4 * np.abs(want))
+            loose = 2e-4 + 1.6e-2 * np.abs(want)
+            diff = np.abs(got - want)
+            assert np.all(diff <= (loose if round_flag else bound)), diff.max()
+            assert np.mean(diff > bound) <= 5e-3
+        if step == 0:
+            first = got.copy()
+        if step == 6:
+            np.testing.assert_array_equal(got, first)   # Reset replays bit-equal
+
+
+@pytest.mark.parametrize("kh,vh,kd,vd,T,round_flag", [(2, 6, 5, 7, 9, False), (2, 6, 5, 7, 9, True),
+                                                     (2, 4, 128, 128, 7, True), (2, 4, 128, 128, 200, True),
+                                                     (1, 2, 128, 128, 70, False)])
+def test_layer_forward_matches_scalar_specification(capi, oracle, kh, vh, kd, vd, T, round_flag):
+    # sequence_delta_net_test.cc:213-255
+    B = 2
+    p = capi.delta_params(kh, vh, kd, vd, round_to_bfloat16=round_flag)
+    po = oracle.delta_params(kh, vh, kd, vd, round_to_bfloat16=round_flag)
+    channels = 2 * kh * kd + vh * vd
+    w, a_log, dt, norm = layer_weights(kh, vh, kd, vd, 4)
+    rng = np.random.default_rng(T + kd)
+    qkv = oracle.bf16_round(rng.standard_normal((B, T, channels)).astype(np.float32))
+    z = oracle.bf16_round(rng.standard_normal((B, T, vh * vd)).astype(np.float32))
+    a = oracle.bf16_round(rng.standard_normal((B, T, vh)).astype(np.float32))
+    b = oracle.bf16_round(rng.standard_normal((B, T, vh)).astype(np.float32))
+    bf = torch.bfloat16
+    state = torch.zeros((B, vh, kd, vd), device="cuda")
+    out = capi.gdn_layer_forward(p, dev(qkv, bf), dev(z, bf), dev(a, bf), dev(b, bf), dev(w),
+                                 dev(a_log), dev(dt), dev(norm), state)
+    torch.cuda.synchronize()
+    got = out.float().cpu().numpy()
+    for i in range(B):
+        want = oracle.gdn_sequence(po, qkv[i], z[i], a[i], b[i], w, a_log, dt, norm)
+        if kd == 128 and round_flag:
+            assert_close_bf16(got[i], want["out"], "delta-net layer T%d" % T)
+            assert_close_bf16(state[i].cpu().numpy(), want["state"], "delta-net layer state")
+        else:
+            # sequence_delta_net_test.cc:253-255
+            assert np.all(np.abs(got[i] - want["out"]) <= 1.5e-4 + 1.5e-2 * np.abs(want["out"]))
+            assert_close(state[i].cpu().numpy(), want["state"], 2e-3, "delta-net layer state")
