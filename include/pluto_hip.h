@@ -198,6 +198,21 @@ int pluto_hip_gqa_prefill(void* stream, const pluto_hip_attention_params* p,
                           const pluto_hip_kv_cache_view* cache, void* out,
                           float* lse, void* workspace, size_t workspace_bytes);
 
+/* The FP32 probabilities tensor of the same ForwardKernel
+ * (qwen_attention.cc:68-119, reported to attention_probabilities_hook at
+ * :441-444), produced on request by a separate two-pass kernel:
+ * probabilities [qh, length, start_position + length], zeros after each row's
+ * visible prefix.  Must follow pluto_hip_gqa_prefill on the same stream with
+ * the same parameters, cache and workspace: it reads the normalised, rotated
+ * queries that call left in the workspace and the keys it appended. */
+int pluto_hip_gqa_prefill_probabilities(void* stream,
+                                        const pluto_hip_attention_params* p,
+                                        int length, int start_position,
+                                        const pluto_hip_kv_cache_view* cache,
+                                        const void* workspace,
+                                        size_t workspace_bytes,
+                                        float* probabilities);
+
 /* Batched single-token decode: `batch` independent CachedAttentionStep calls
  * (cached_attention_ops.cc:308-353: PrepareAttentionKernel :30-79,
  * FullAttentionKernel :83-126) in one launch sequence.  Sequence b appends

@@ -1,5 +1,6 @@
-"""Builds pluto_amd/libpluto_hip.so (the C ABI + gfx950 kernels) and, for the
-host-side C++ mirror of the reference API, pluto_amd/libpluto_llm.so.
+"""Builds pluto_amd/libpluto_hip.so (the C ABI + gfx950 kernels, hipcc) and
+pluto_amd/libpluto_llm.so (the host-side C++ mirror of the reference's layer
+API above that C ABI, g++).
 
 Usage: python -m pluto_amd.build [--force]
 Sources are compiled with hipcc for gfx950 only; objects go to build/ (git
@@ -56,7 +57,15 @@ def _compile(src, flags):
     return obj
 
 
-def build(force=False, verbose=True):
+CXX = os.environ.get("CXX", "g++")
+# The host mirror is plain C++ above the C ABI: no HIP headers, no device code.
+HOST_FLAGS = ["-O2", "-g", "-std=c++20", "-fPIC", "-fno-exceptions", "-Wall", "-Wextra",
+              "-I" + os.path.join(ROOT, "include"), "-I" + ROOT]
+HOST_TEST = os.path.join(ROOT, "build", "bin", "host_tests")
+HOST_TEST_SOURCES = os.path.join(ROOT, "tests", "cpp")
+
+
+def build_device(force=False, verbose=True):
     os.makedirs(OBJ, exist_ok=True)
     headers = glob.glob(os.path.join(CSRC, "*.h")) + glob.glob(
         os.path.join(ROOT, "include", "*.h"))
@@ -68,20 +77,51 @@ def build(force=False, verbose=True):
              objects)
         if verbose:
             print("built", LIB)
-    host_sources = sorted(glob.glob(os.path.join(HOST, "*.cc")))
-    host_headers = glob.glob(os.path.join(HOST, "*.h")) + headers
-    if host_sources and (force or not _newer(HOST_LIB, host_sources + host_headers + [LIB])):
-        flags = ["-O2", "-std=c++20", "-fPIC", "-fno-exceptions", "-x", "hip",
-                 "--offload-arch=gfx950",
-                 "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-                 "-Wno-unused-command-line-argument",
-                 "-I" + os.path.join(ROOT, "include"), "-I" + ROOT]
+    return LIB
+
+
+def _compile_host(src):
+    obj = os.path.join(OBJ, "host_" + os.path.basename(src) + ".o")
+    _run([CXX] + HOST_FLAGS + ["-c", src, "-o", obj])
+    return obj
+
+
+def build_host(force=False, verbose=True):
+    """libpluto_llm.so (the reference's layer API over the C ABI) and the C++
+    test runner build/bin/host_tests that tests/test_host_cpp.py drives."""
+    os.makedirs(OBJ, exist_ok=True)
+    os.makedirs(os.path.dirname(HOST_TEST), exist_ok=True)
+    headers = glob.glob(os.path.join(HOST, "*.h")) + glob.glob(
+        os.path.join(ROOT, "include", "*.h"))
+    sources = sorted(glob.glob(os.path.join(HOST, "*.cc")))
+    link = ["-L" + HERE, "-lpluto_hip", "-Wl,-rpath,$ORIGIN"]
+    if force or not _newer(HOST_LIB, sources + headers + [LIB]):
         with concurrent.futures.ThreadPoolExecutor(max_workers=8) as pool:
-            objects = list(pool.map(lambda s: _compile(s, flags), host_sources))
-        _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", HOST_LIB] +
-             objects + ["-L" + HERE, "-lpluto_hip", "-Wl,-rpath,$ORIGIN"])
+            objects = list(pool.map(_compile_host, sources))
+        # libpluto_hip.so pulls in the HIP runtime, which is resolved when a
+        # process loads it; the link step only needs our own symbols.
+        _run([CXX, "-shared", "-fPIC", "-o", HOST_LIB] + objects + link +
+             ["-Wl,--allow-shlib-undefined"])
         if verbose:
             print("built", HOST_LIB)
+    tests = sorted(glob.glob(os.path.join(HOST_TEST_SOURCES, "*.cc")))
+    test_headers = glob.glob(os.path.join(HOST_TEST_SOURCES, "*.h"))
+    if tests and (force or not _newer(HOST_TEST, tests + test_headers + headers + [HOST_LIB])):
+        with concurrent.futures.ThreadPoolExecutor(max_workers=8) as pool:
+            objects = list(pool.map(_compile_host, tests))
+        _run([CXX, "-o", HOST_TEST] + objects +
+             ["-L" + HERE, "-lpluto_llm", "-lpluto_hip", "-Wl,-rpath,$ORIGIN/../../pluto_amd",
+              "-L" + os.path.join(ROOT, "oracle"), "-loracle",
+              "-Wl,-rpath,$ORIGIN/../../oracle",
+              "-Wl,--allow-shlib-undefined", "-Wl,-rpath,/opt/rocm/lib", "-lpthread"])
+        if verbose:
+            print("built", HOST_TEST)
+    return HOST_LIB
+
+
+def build(force=False, verbose=True):
+    build_device(force, verbose)
+    build_host(force, verbose)
     return LIB
 
 

@@ -94,6 +94,8 @@ SIGNATURES = {
     "pluto_hip_gqa_prefill": (_I, [_VP, ctypes.POINTER(AttentionParams), _I, _I, _VP,
                                    _VP, _VP, _VP, _VP, ctypes.POINTER(KvCacheView),
                                    _VP, _VP, _VP, _SZ]),
+    "pluto_hip_gqa_prefill_probabilities": (_I, [_VP, ctypes.POINTER(AttentionParams), _I, _I,
+                                                 ctypes.POINTER(KvCacheView), _VP, _SZ, _VP]),
     "pluto_hip_gqa_decode_workspace_bytes": (_SZ, [ctypes.POINTER(AttentionParams), _I,
                                                    ctypes.POINTER(_I), _I]),
     "pluto_hip_gqa_decode": (_I, [_VP, ctypes.POINTER(AttentionParams), _I, _I, _VP,
@@ -248,8 +250,10 @@ class KvCache:
 
 
 def gqa_prefill(p, qg, k, v, q_norm, k_norm, cache, start_position=0, want_lse=False,
-                stream=None):
-    """qg bf16 [T, qh, 2, d]; k, v bf16 [T, kh, d]; norms fp32 [d]."""
+                stream=None, want_probabilities=False):
+    """qg bf16 [T, qh, 2, d]; k, v bf16 [T, kh, d]; norms fp32 [d].
+
+    want_probabilities appends fp32 [qh, T, start_position + T] to the result."""
     T = qg.shape[0]
     out = torch.empty((T, p.query_heads, p.head_dim), dtype=torch.bfloat16, device=qg.device)
     lse = (torch.empty((T, p.query_heads), dtype=torch.float32, device=qg.device)
@@ -262,7 +266,15 @@ def gqa_prefill(p, qg, k, v, q_norm, k_norm, cache, start_position=0, want_lse=F
                                       ptr(k_norm), ctypes.byref(view), ptr(out), ptr(lse),
                                       ptr(workspace), size))
     cache.position = start_position + T
-    return (out, lse) if want_lse else out
+    result = (out, lse) if want_lse else out
+    if want_probabilities:
+        probabilities = torch.empty((p.query_heads, T, start_position + T), dtype=torch.float32,
+                                    device=qg.device)
+        check(lib().pluto_hip_gqa_prefill_probabilities(
+            stream or current_stream(), ctypes.byref(p), T, start_position, ctypes.byref(view),
+            ptr(workspace), size, ptr(probabilities)))
+        result = (result + (probabilities,)) if want_lse else (result, probabilities)
+    return result
 
 
 def gqa_decode_workspace(p, positions, split_tokens=0, device="cuda"):

@@ -95,11 +95,15 @@ int launch_decode_fast(hipStream_t stream, const DecodeArgs& args,
                        const DecodeBatch& batch);
 int launch_decode_combine(hipStream_t stream, const DecodeCombineArgs& args,
                           const DecodeBatch& batch);
-// Two-pass probability row of one sequence (any dtype, any shape):
-// AttentionProbabilitiesKernel, cached_attention_ops.cc:131-178.
-int launch_decode_probabilities(hipStream_t stream, const void* q, int q_dtype,
-                                const CacheView& cache, int query_heads,
-                                int key_value_heads, int head_dim, int length,
-                                float scale, float* probabilities);
+// Two-pass probability rows (any dtype, any shape): row r of `rows` sees the
+// first `first_visible + r` cache rows; output fp32 [query_heads, rows,
+// row_width], zero beyond the visible prefix
+// (AttentionProbabilitiesKernel, cached_attention_ops.cc:131-178; the probs
+// tensor of ForwardKernel, qwen_attention.cc:68-119).
+int launch_attention_probabilities(hipStream_t stream, const void* q, int q_dtype,
+                                   const CacheView& cache, int query_heads,
+                                   int key_value_heads, int head_dim, int rows,
+                                   int first_visible, int row_width, float scale,
+                                   float* probabilities);
 
 }  // namespace pluto_hip

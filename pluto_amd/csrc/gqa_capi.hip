@@ -175,6 +175,32 @@ int pluto_hip_gqa_prefill(void* stream, const pluto_hip_attention_params* p, int
   return launch_generic_forward(s, a, 1);
 }
 
+int pluto_hip_gqa_prefill_probabilities(void* stream, const pluto_hip_attention_params* p,
+                                        int length, int start_position,
+                                        const pluto_hip_kv_cache_view* cache,
+                                        const void* workspace, size_t workspace_bytes,
+                                        float* probabilities) {
+  int status = validate_params(p);
+  if (status != 0) return status;
+  if (length <= 0 || start_position < 0 || !probabilities) return PLUTO_HIP_EINVAL;
+  status = validate_cache(cache, p);
+  if (status != 0) return status;
+  if (static_cast<long long>(start_position) + length > p->capacity) return PLUTO_HIP_ERANGE;
+  const PrefillLayout layout = prefill_layout(p, length);
+  if (!workspace || workspace_bytes < layout.total) return PLUTO_HIP_EWORKSPACE;
+  const CacheView view{cache->keys, cache->values, cache->dtype, cache->token_stride,
+                       cache->head_stride};
+  const float scale = 1.0f / std::sqrt(static_cast<float>(p->head_dim));
+  const char* queries = static_cast<const char*>(workspace) + layout.queries;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  // The grid's second dimension holds at most 65535 rows per launch.
+  const int width = start_position + length;
+  if (length > 65535) return PLUTO_HIP_EUNSUPPORTED;
+  return launch_attention_probabilities(
+      s, queries, p->round_to_bfloat16 ? PLUTO_HIP_BF16 : PLUTO_HIP_F32, view, p->query_heads,
+      p->key_value_heads, p->head_dim, length, start_position + 1, width, scale, probabilities);
+}
+
 size_t pluto_hip_gqa_decode_workspace_bytes(const pluto_hip_attention_params* p, int batch,
                                             const int* positions, int split_tokens) {
   if (validate_params(p) != 0 || batch <= 0 || !positions) return 0;
@@ -340,8 +366,9 @@ int pluto_hip_gqa_decode(void* stream, const pluto_hip_attention_params* p, int 
                             static_cast<size_t>(b) * qh * d * element_bytes(q_dtype);
         const CacheView view{caches[b].keys, caches[b].values, c0.dtype, c0.token_stride,
                              c0.head_stride};
-        status = launch_decode_probabilities(s, qbase, q_dtype, view, qh, kh, d,
-                                             positions[b] + 1, scale, probabilities[b]);
+        status = launch_attention_probabilities(s, qbase, q_dtype, view, qh, kh, d, 1,
+                                                positions[b] + 1, positions[b] + 1, scale,
+                                                probabilities[b]);
         if (status != 0) return status;
       }
     }

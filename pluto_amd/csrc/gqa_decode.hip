@@ -231,18 +231,24 @@ decode_combine_kernel(DecodeCombineArgs a, DecodeBatch batch) {
   }
 }
 
-// Two-pass probability row for inspection: one workgroup per query head.
+// Two-pass probability rows for inspection: one workgroup per (query head,
+// query row).  Row r sees the first `first_visible + r` cache rows and is
+// stored at probabilities[(head * rows + r) * row_width ..], zero beyond the
+// visible prefix.
 __global__ void __launch_bounds__(256)
-decode_probabilities_kernel(const void* q, int q_dtype, CacheView cache, int query_heads,
-                            int key_value_heads, int head_dim, int length, float scale,
-                            float* probabilities) {
+attention_probabilities_kernel(const void* q, int q_dtype, CacheView cache, int query_heads,
+                               int key_value_heads, int head_dim, int rows, int first_visible,
+                               int row_width, float scale, float* probabilities) {
   __shared__ float query[256];
   __shared__ float reduce[4];
   const int head = blockIdx.x;
+  const int r = blockIdx.y;
+  const int length = first_visible + r;
   const int kv = head / (query_heads / key_value_heads);
-  float* row = probabilities + static_cast<long long>(head) * length;
+  float* row = probabilities + (static_cast<long long>(head) * rows + r) * row_width;
   for (int c = threadIdx.x; c < head_dim; c += 256)
-    query[c] = load_element(q, static_cast<long long>(head) * head_dim + c, q_dtype);
+    query[c] = load_element(
+        q, (static_cast<long long>(r) * query_heads + head) * head_dim + c, q_dtype);
   __syncthreads();
   float maximum = kMasked;
   for (int t = threadIdx.x; t < length; t += 256) {
@@ -270,6 +276,7 @@ decode_probabilities_kernel(const void* q, int q_dtype, CacheView cache, int que
   __syncthreads();
   sum = (reduce[0] + reduce[1]) + (reduce[2] + reduce[3]);
   for (int t = threadIdx.x; t < length; t += 256) row[t] = row[t] / sum;
+  for (int t = length + threadIdx.x; t < row_width; t += 256) row[t] = 0.0f;
 }
 
 template <int D>
@@ -315,12 +322,17 @@ int launch_decode_combine(hipStream_t stream, const DecodeCombineArgs& a,
   return launch_status();
 }
 
-int launch_decode_probabilities(hipStream_t stream, const void* q, int q_dtype,
-                                const CacheView& cache, int query_heads,
-                                int key_value_heads, int head_dim, int length,
-                                float scale, float* probabilities) {
-  decode_probabilities_kernel<<<query_heads, 256, 0, stream>>>(
-      q, q_dtype, cache, query_heads, key_value_heads, head_dim, length, scale, probabilities);
+int launch_attention_probabilities(hipStream_t stream, const void* q, int q_dtype,
+                                   const CacheView& cache, int query_heads,
+                                   int key_value_heads, int head_dim, int rows,
+                                   int first_visible, int row_width, float scale,
+                                   float* probabilities) {
+  if (rows <= 0 || rows > 65535 || first_visible <= 0 ||
+      static_cast<long long>(first_visible) + rows - 1 > row_width)
+    return PLUTO_HIP_EINVAL;
+  attention_probabilities_kernel<<<dim3(query_heads, rows), 256, 0, stream>>>(
+      q, q_dtype, cache, query_heads, key_value_heads, head_dim, rows, first_visible, row_width,
+      scale, probabilities);
   return launch_status();
 }
 

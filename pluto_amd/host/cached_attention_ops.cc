@@ -1,0 +1,135 @@
+#include "pluto_amd/host/cached_attention_ops.h"
+
+#include <cmath>
+#include <limits>
+
+namespace pluto::llm::cached_attention_ops {
+namespace {
+
+StatusOr<hip::Buffer> AllocateFloats(hip::Executor& executor, size_t count) {
+  if (count > std::numeric_limits<size_t>::max() / sizeof(float))
+    return ResourceExhaustedError("attention allocation size overflows");
+  return hip::Buffer::Allocate(executor, count * sizeof(float));
+}
+
+}  // namespace
+
+pluto_hip_attention_params ToAbi(const FullAttentionParameters& p) {
+  pluto_hip_attention_params abi{};
+  abi.query_heads = p.query_heads;
+  abi.key_value_heads = p.key_value_heads;
+  abi.head_dim = p.head_dim;
+  abi.rotary_dim = p.rotary_dim;
+  abi.capacity = p.capacity;
+  abi.rms_norm_epsilon = p.rms_norm_epsilon;
+  abi.rope_theta = p.rope_theta;
+  abi.round_to_bfloat16 = p.round_to_bfloat16 ? 1 : 0;
+  return abi;
+}
+
+pluto_hip_delta_params ToAbi(const DeltaNetParameters& p) {
+  pluto_hip_delta_params abi{};
+  abi.key_heads = p.key_heads;
+  abi.value_heads = p.value_heads;
+  abi.key_head_dim = p.key_head_dim;
+  abi.value_head_dim = p.value_head_dim;
+  abi.conv_kernel_dim = p.conv_kernel_dim;
+  abi.rms_norm_epsilon = p.rms_norm_epsilon;
+  abi.round_to_bfloat16 = p.round_to_bfloat16 ? 1 : 0;
+  return abi;
+}
+
+// src/llm/layers/util/cached_attention_ops.cc:283-306
+Status ValidateCachedAttention(hip::Executor& executor, const FullAttentionParameters& p,
+                               const KeyValueCache& cache) {
+  const pluto_hip_attention_params abi = ToAbi(p);
+  if (pluto_hip_attention_params_validate(&abi) != 0)
+    return InvalidArgumentError("invalid full-attention dimensions or parameters");
+  if (&cache.executor() != &executor)
+    return InvalidArgumentError("attention cache belongs to a different Executor");
+  if (cache.capacity() != p.capacity || cache.key_value_heads() != p.key_value_heads ||
+      cache.head_dim() != p.head_dim)
+    return InvalidArgumentError("attention cache shape or capacity does not match parameters");
+  if (cache.storage() == KeyValueCache::Storage::kBFloat16HeadMajor && !p.round_to_bfloat16)
+    return InvalidArgumentError("a bfloat16 attention cache requires round_to_bfloat16");
+  return OkStatus();
+}
+
+// src/llm/layers/util/cached_attention_ops.cc:308-353
+Status CachedAttentionStep(hip::Executor& executor, const FullAttentionParameters& p,
+                           KeyValueCache& cache, const float* q_gate, const float* k,
+                           const float* v, const float* q_norm, const float* k_norm,
+                           float* output, float* probabilities) {
+  RETURN_IF_ERROR(ValidateCachedAttention(executor, p, cache));
+  if (!q_gate || !k || !v || !q_norm || !k_norm || !output)
+    return InvalidArgumentError("attention requires non-null device pointers");
+  if (cache.position() >= cache.capacity())
+    return ResourceExhaustedError("full-attention cache capacity reached");
+  const pluto_hip_attention_params abi = ToAbi(p);
+  const int position = cache.position();
+  const pluto_hip_kv_cache_view view = cache.view();
+  // Stream-ordered scratch for the prepared query and the split-K partials,
+  // like the reference's temporary query storage (:321-323).
+  const size_t workspace_bytes = pluto_hip_gqa_decode_workspace_bytes(&abi, 1, &position, 0);
+  ASSIGN_OR_RETURN(auto workspace, hip::Buffer::Allocate(executor, workspace_bytes));
+  float* const probability_rows[1] = {probabilities};
+  RETURN_IF_ERROR(hip::HipStatus(
+      pluto_hip_gqa_decode(executor.stream(), &abi, 1, PLUTO_HIP_F32, q_gate, k, v, q_norm, k_norm,
+                           &position, &view, output, probabilities ? probability_rows : nullptr, 0,
+                           workspace.data(), workspace_bytes),
+      "Qwen full attention"));
+  return cache.Advance();
+}
+
+// src/llm/layers/util/cached_attention_ops.cc:369-399
+StatusOr<std::unique_ptr<DeltaNetState>> DeltaNetState::Create(hip::Executor& executor,
+                                                               DeltaNetParameters p) {
+  if (p.key_heads <= 0 || p.value_heads <= 0 || p.value_heads % p.key_heads != 0 ||
+      p.key_head_dim <= 0 || p.key_head_dim > 128 || p.value_head_dim <= 0 ||
+      p.value_head_dim > 256 || p.conv_kernel_dim <= 0 || p.conv_kernel_dim > 32 ||
+      !std::isfinite(p.rms_norm_epsilon) || p.rms_norm_epsilon <= 0.0f)
+    return InvalidArgumentError("invalid DeltaNet dimensions or parameters");
+  const size_t channels = 2 * static_cast<size_t>(p.key_heads) * p.key_head_dim +
+                          static_cast<size_t>(p.value_heads) * p.value_head_dim;
+  if (channels > static_cast<size_t>(std::numeric_limits<int>::max()) / p.conv_kernel_dim)
+    return ResourceExhaustedError("DeltaNet dimensions exceed indexing limit");
+  ASSIGN_OR_RETURN(auto convolution, AllocateFloats(executor, channels * p.conv_kernel_dim));
+  ASSIGN_OR_RETURN(auto recurrence,
+                   AllocateFloats(executor, static_cast<size_t>(p.value_heads) * p.key_head_dim *
+                                                p.value_head_dim));
+  const pluto_hip_delta_params abi = ToAbi(p);
+  ASSIGN_OR_RETURN(auto workspace,
+                   hip::Buffer::Allocate(executor, pluto_hip_gdn_step_workspace_bytes(&abi)));
+  std::unique_ptr<DeltaNetState> result(new DeltaNetState(
+      executor, p, std::move(convolution), std::move(recurrence), std::move(workspace)));
+  RETURN_IF_ERROR(result->Reset());
+  return result;
+}
+
+// src/llm/layers/util/cached_attention_ops.cc:401-431
+Status DeltaNetState::Step(const float* qkv, const float* z, const float* a, const float* b,
+                           const float* conv_weight, const float* a_log, const float* dt_bias,
+                           const float* norm_weight, float* output) {
+  if (!qkv || !z || !a || !b || !conv_weight || !a_log || !dt_bias || !norm_weight || !output)
+    return InvalidArgumentError("DeltaNet requires non-null device pointers");
+  const pluto_hip_delta_params abi = ToAbi(parameters_);
+  return hip::HipStatus(
+      pluto_hip_gdn_step(executor_.stream(), &abi, static_cast<float*>(convolution_state_.data()),
+                         static_cast<float*>(recurrent_state_.data()), qkv, z, a, b, conv_weight,
+                         a_log, dt_bias, norm_weight, output, workspace_.data(),
+                         workspace_.size_bytes()),
+      "Qwen gated delta step");
+}
+
+// src/llm/layers/util/cached_attention_ops.cc:433-443
+Status DeltaNetState::Reset() {
+  RETURN_IF_ERROR(hip::HipStatus(
+      pluto_hip_memset_async(executor_.stream(), convolution_state_.data(), 0,
+                             convolution_state_.size_bytes()),
+      "reset Qwen convolution state"));
+  return hip::HipStatus(pluto_hip_memset_async(executor_.stream(), recurrent_state_.data(), 0,
+                                               recurrent_state_.size_bytes()),
+                        "reset Qwen recurrent state");
+}
+
+}  // namespace pluto::llm::cached_attention_ops

@@ -1,0 +1,87 @@
+// Single-token cached attention and the single-token gated delta-net state:
+// the functions of src/llm/layers/util/cached_attention_ops.h:13-95 over the
+// C ABI.  Pointers are contiguous device FP32 arrays exactly as in the
+// reference; BF16 values are represented exactly in them.
+#pragma once
+
+#include <memory>
+
+#include "pluto_amd/host/executor.h"
+#include "pluto_amd/host/key_value_cache.h"
+
+namespace pluto::llm::cached_attention_ops {
+
+struct FullAttentionParameters {
+  int query_heads = 24;
+  int key_value_heads = 4;
+  int head_dim = 256;
+  int rotary_dim = 64;
+  int capacity = 4096;
+  float rms_norm_epsilon = 1e-6f;
+  float rope_theta = 10000000.0f;
+  bool round_to_bfloat16 = true;
+};
+
+pluto_hip_attention_params ToAbi(const FullAttentionParameters& parameters);
+
+// Parameter limits, and the cache's Executor, KV shape and capacity must
+// match.  A full cache is still compatible.  No GPU work.
+Status ValidateCachedAttention(hip::Executor& executor, const FullAttentionParameters& parameters,
+                               const KeyValueCache& cache);
+
+// One token of batch-one causal attention against an externally owned cache,
+// whose position is the only sequence counter.  q_gate [query_heads, 2,
+// head_dim], k/v [key_value_heads, head_dim], q_norm/k_norm [head_dim]
+// zero-centred; output [query_heads, head_dim] after sigmoid gating; optional
+// probabilities [query_heads, position()+1].  Validates pointers and remaining
+// capacity before GPU work and advances the cache once after every launch
+// succeeded.  A kBFloat16HeadMajor cache requires round_to_bfloat16.
+Status CachedAttentionStep(hip::Executor& executor, const FullAttentionParameters& parameters,
+                           KeyValueCache& cache, const float* q_gate, const float* k,
+                           const float* v, const float* q_norm, const float* k_norm,
+                           float* output, float* probabilities = nullptr);
+
+struct DeltaNetParameters {
+  int key_heads = 16;
+  int value_heads = 48;
+  int key_head_dim = 128;
+  int value_head_dim = 128;
+  int conv_kernel_dim = 4;
+  float rms_norm_epsilon = 1e-6f;
+  bool round_to_bfloat16 = true;
+};
+
+pluto_hip_delta_params ToAbi(const DeltaNetParameters& parameters);
+
+// Single-token causal depthwise convolution + gated delta rule.  The recurrent
+// matrix stays FP32 even when activation rounding is enabled.
+class DeltaNetState final {
+ public:
+  DeltaNetState(const DeltaNetState&) = delete;
+  DeltaNetState& operator=(const DeltaNetState&) = delete;
+  static StatusOr<std::unique_ptr<DeltaNetState>> Create(hip::Executor& executor,
+                                                         DeltaNetParameters parameters);
+
+  // qkv packs [all Q, all K, all V]; z [value_heads, value_head_dim]; a, b,
+  // a_log, dt_bias [value_heads]; conv_weight [qkv_channels, conv_kernel_dim]
+  // oldest to newest; norm_weight [value_head_dim], a plain multiplier.
+  // Output has z's shape, after RMSNorm and SiLU(z) gating.
+  Status Step(const float* qkv, const float* z, const float* a, const float* b,
+              const float* conv_weight, const float* a_log, const float* dt_bias,
+              const float* norm_weight, float* output);
+  Status Reset();
+
+ private:
+  DeltaNetState(hip::Executor& executor, DeltaNetParameters parameters,
+                hip::Buffer convolution_state, hip::Buffer recurrent_state, hip::Buffer workspace)
+      : executor_(executor), parameters_(parameters),
+        convolution_state_(std::move(convolution_state)),
+        recurrent_state_(std::move(recurrent_state)), workspace_(std::move(workspace)) {}
+  hip::Executor& executor_;
+  DeltaNetParameters parameters_;
+  hip::Buffer convolution_state_;
+  hip::Buffer recurrent_state_;
+  hip::Buffer workspace_;  // convolved QKV and core output of one token
+};
+
+}  // namespace pluto::llm::cached_attention_ops

@@ -398,3 +398,40 @@ def test_rejects_invalid_arguments_before_any_work(capi):
         assert code == capi.EINVAL
     torch.cuda.synchronize()
     assert torch.all(t == -13.0)
+
+
+@pytest.mark.parametrize("d,rotary,T", [(3, 2, 33), (256, 64, 3), (128, 32, 70)])
+def test_prefill_probabilities_are_causal_rows_that_match_decode(capi, oracle, d, rotary, T):
+    # qwen_attention_test.cc:155-200: [1, heads, T, T], zero above the diagonal,
+    # rows sum to one; each row equals the cached path's probabilities for that token.
+    qh, kh = 2, 1
+    kw = dict(query_heads=qh, key_value_heads=kh, head_dim=d, rotary_dim=rotary, capacity=40 + T,
+              rope_theta=73.0 if d == 3 else 1e7)
+    p, _ = both_params(capi, oracle, **kw)
+    rng = np.random.default_rng(d)
+    qg, k, v = make_sequence(oracle, rng, T, qh, kh, d)
+    qw, kw_ = values(d, 0.2, 0.3), values(d, 0.8, 0.4)
+    bf = torch.bfloat16
+    cache = capi.KvCache(40 + T, kh, d)
+    out, lse, probs = capi.gqa_prefill(p, dev(qg, bf), dev(k, bf), dev(v, bf), dev(qw), dev(kw_),
+                                       cache, want_lse=True, want_probabilities=True)
+    probs = probs.cpu().numpy()
+    assert probs.shape == (qh, T, T)
+    for row in range(T):
+        assert np.all(probs[:, row, row + 1:] == 0)
+    np.testing.assert_allclose(probs.astype(np.float64).sum(-1), 1.0, atol=2e-6)
+    stepped = capi.KvCache(40 + T, kh, d)
+    for t in range(T):
+        row = [torch.zeros((qh, t + 1), device="cuda")]
+        capi.gqa_decode(p, dev(qg[t:t + 1], bf), dev(k[t:t + 1], bf), dev(v[t:t + 1], bf),
+                        dev(qw), dev(kw_), [stepped], probabilities=row)
+        np.testing.assert_allclose(probs[:, t, :t + 1], row[0].cpu().numpy(), rtol=1e-5, atol=1e-7)
+    # a continuation reports [heads, length, start + length]
+    more = make_sequence(oracle, rng, 5, qh, kh, d)
+    _, tail = capi.gqa_prefill(p, dev(more[0], bf), dev(more[1], bf), dev(more[2], bf), dev(qw),
+                               dev(kw_), cache, start_position=T, want_probabilities=True)
+    tail = tail.cpu().numpy()
+    assert tail.shape == (qh, 5, T + 5)
+    np.testing.assert_allclose(tail.astype(np.float64).sum(-1), 1.0, atol=2e-6)
+    for row in range(5):
+        assert np.all(tail[:, row, T + row + 1:] == 0) and np.all(tail[:, row, :T + row + 1] > 0)
