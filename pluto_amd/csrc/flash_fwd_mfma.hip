@@ -1,20 +1,24 @@
 // Causal flash attention forward for bf16 activations on gfx950 matrix cores.
 //
-// One workgroup (4 wave64) owns 128 query rows of one (sequence, head); wave w
-// owns rows 32w..32w+31.  Key/value tiles of 64 rows are staged through LDS.
-// Both products are computed transposed with v_mfma_f32_32x32x16_bf16:
+// A workgroup of WAVES wave64 owns BM = 32*G*WAVES query rows of one
+// (sequence, head); a wave owns G groups of 32 consecutive rows.  Key/value
+// tiles of 64 rows are double-buffered in LDS, both row major, and are filled
+// by buffer loads that write LDS directly (no VGPR round trip, out-of-range
+// rows read as zero).  Both products are computed transposed with
+// v_mfma_f32_32x32x16_bf16:
 //
 //   S^T[key, query] = K[key, :] . Q[query, :]      A = K (LDS), B = Q (regs)
 //   O^T[d,   query] = V^T[d, key] . P^T[key, query] A = V^T (LDS), B = P^T
 //
 // In the 32x32 accumulator layout lane l holds column (l % 32), i.e. ONE query,
 // so the softmax row statistics are per-lane scalars and need a single
-// cross-lane exchange (lane ^ 32) per tile, and the probabilities leave the
-// accumulator registers already laid out as the B operand of the second
+// exchange between the two lane halves per block, and the probabilities leave
+// the accumulator registers already laid out as the B operand of the second
 // product: no shuffle, no LDS round trip.  The contraction index of an MFMA
-// may be enumerated in any order as long as A and B agree, so V^T is written to
-// LDS with its keys permuted to the order in which the accumulator registers
-// hold them.
+// may be enumerated in any order as long as A and B agree, so the V^T operand
+// gathers its keys in the order in which the accumulator registers hold them;
+// the gather itself is done by the LDS transpose read (ds_read_b64_tr_b16),
+// which hands each lane four keys of one channel from a row-major tile.
 //
 // Semantics follow FlashAttentionForwardKernel (src/llm/layers/attention.cc:
 // 98-170) and, with the gate epilogue, ForwardKernel
@@ -23,40 +27,88 @@
 // reference keeps them FP32, attention.cc:151-156).
 #include "flash_fwd_mfma.h"
 
+#include <cstdlib>
+
 #include "mfma_tile.h"
 
 namespace pluto_hip {
 namespace {
 
-constexpr int BM = 128;  // query rows per workgroup
-constexpr int BN = 64;   // keys per LDS tile
-constexpr int kThreads = 256;
+constexpr int BN = 64;  // keys per LDS tile
 
-template <int D>
-struct Smem {
-  static constexpr int KCH = D / 8;  // 16-byte chunks per K row
-  // K tile, row major: chunk (key, ch) at key*KCH + (ch ^ (key & 7)).
-  uint4 k[BN * KCH];
-  // V^T tile: row d holds BN keys as 8 chunks of 8 keys in accumulator order;
-  // chunk c of row d at d*(BN/8) + (c ^ swizzle_d(d)).
-  uint4 vt[D * (BN / 8)];
+typedef __attribute__((ext_vector_type(4))) short shortx4;
+typedef __attribute__((address_space(3))) void lds_void;
+
+// Buffer descriptor over [base, base + bytes): loads beyond `bytes` return 0.
+__device__ inline __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
+}
+
+// Four keys (rows r..r+3 chosen by the lane addresses) of one channel per lane.
+__device__ inline uint2 lds_transpose_read(const unsigned char* tile, int byte_offset) {
+  const shortx4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      (__attribute__((address_space(3))) shortx4*)(tile + byte_offset));
+  return __builtin_bit_cast(uint2, v);
+}
+
+// Maximum over both lane halves (lanes l and l ^ 32) of a per-lane value.
+__device__ inline float half_swap_max(float v) {
+  const uint32_t bits = __builtin_bit_cast(uint32_t, v);
+  const auto pair = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
+  return fmaxf(__builtin_bit_cast(float, pair[0]), __builtin_bit_cast(float, pair[1]));
+}
+
+// Queues the loads of one K tile and one V tile (keys k0..k0+63) into an LDS
+// stage.  Lane l of load i of a wave writes 16 bytes at chunk
+// (wave*LOADS + i)*64 + l of the tile; k_fill/v_fill say which global bytes it
+// fetches.  Rows at or beyond kv_rows read as zero.
+template <int D, int LOADS>
+__device__ inline void fill_stage(unsigned char* stage, int wave, const uint16_t* k_base,
+                                  const uint16_t* v_base, long long k_row_stride,
+                                  long long v_row_stride, int k0, int kv_rows,
+                                  const uint32_t* k_fill, const uint32_t* v_fill) {
+  constexpr int kTileBytes = BN * D * 2;
+  const long long rows_left = kv_rows - 1 - k0;
+  const __amdgpu_buffer_rsrc_t k_rsrc =
+      make_rsrc(k_base + static_cast<long long>(k0) * k_row_stride,
+                static_cast<uint32_t>((rows_left * k_row_stride + D) * 2));
+  const __amdgpu_buffer_rsrc_t v_rsrc =
+      make_rsrc(v_base + static_cast<long long>(k0) * v_row_stride,
+                static_cast<uint32_t>((rows_left * v_row_stride + D) * 2));
+#pragma unroll
+  for (int i = 0; i < LOADS; ++i) {
+    const int at = (wave * LOADS + i) * 1024;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, (lds_void*)(stage + at), 16, k_fill[i], 0, 0,
+                                             0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc, (lds_void*)(stage + kTileBytes + at), 16,
+                                             v_fill[i], 0, 0, 0);
+  }
+}
+
+template <int D, int G, int WAVES>
+struct Config {
+  static constexpr int kThreads = 64 * WAVES;
+  static constexpr int BM = 32 * G * WAVES;
+  static constexpr int KCH = D / 8;                // 16-byte chunks per row
+  static constexpr int kTileBytes = BN * D * 2;    // one K or V tile
+  static constexpr int kStageBytes = 2 * kTileBytes;
+  static constexpr int kLoads = BN * KCH / kThreads;  // 16-byte loads per lane per tensor
+  // waves per SIMD the register budget is sized for
+  static constexpr int kOccupancy = (D == 64 && G == 1) ? 3 : 2;
 };
 
-// Register budget: 4 waves per SIMD for 64-wide heads (128 VGPRs), 2 for
-// 128-wide heads, so that several workgroups per CU overlap their matrix-core
-// and vector phases.
-template <int D>
-__global__ void __launch_bounds__(kThreads)
-__attribute__((amdgpu_waves_per_eu(D == 64 ? 3 : 2, D == 64 ? 3 : 2)))
+template <int D, int G, int WAVES>
+__global__ void __launch_bounds__(64 * WAVES)
+__attribute__((amdgpu_waves_per_eu(Config<D, G, WAVES>::kOccupancy,
+                                   Config<D, G, WAVES>::kOccupancy)))
 flash_forward_kernel(FlashForwardArgs a) {
-  constexpr int KCH = D / 8;
-  constexpr int KS = D / 16;      // contraction steps of S^T
-  constexpr int DB = D / 32;      // 32-row blocks of O^T
-  constexpr int KB = BN / 32;     // 32-key blocks per tile
-  constexpr int OSTRIDE = D * 2 + 16;  // bytes per staged output row
-  __shared__ __attribute__((aligned(16))) unsigned char raw[
-      sizeof(Smem<D>) > BM * OSTRIDE ? sizeof(Smem<D>) : BM * OSTRIDE];
-  Smem<D>& sm = *reinterpret_cast<Smem<D>*>(raw);
+  using C = Config<D, G, WAVES>;
+  constexpr int KCH = C::KCH;
+  constexpr int KS = D / 16;   // contraction steps of S^T
+  constexpr int DB = D / 32;   // 32-row blocks of O^T
+  constexpr int KB = BN / 32;  // 32-key blocks per tile
+  constexpr int BM = C::BM;
+  __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * C::kStageBytes];
 
   const int tid = threadIdx.x;
   const int wave = tid / 64, lane = tid % 64;
@@ -83,61 +135,38 @@ flash_forward_kernel(FlashForwardArgs a) {
 #pragma unroll
   for (int e = 0; e < 8; ++e) ones[e] = static_cast<__bf16>(1.0f);
 
-  // Loader roles: waves 0-1 fetch K (row major), waves 2-3 fetch V and
-  // transpose it in registers.  Both move BN*D*2 bytes per tile with
-  // 16-byte loads.
-  constexpr int LOADS = BN * KCH / 128;  // 16-byte loads per loader thread
-  uint4 staged[LOADS];
-  const int ltid = tid % 128;
-  const bool loads_k = tid < 128;
-
-  auto fetch = [&](int tile) {
-    const int k0 = tile * BN;
-    if (loads_k) {
+  // ---- loop-invariant lane addresses ---------------------------------------
+  // Tile fill: load i of this lane lands at LDS chunk p = (wave*kLoads+i)*64 +
+  // lane of the tile (the hardware writes lane l at base + 16 l); which global
+  // chunk it fetches is chosen so that the tile ends up swizzled:
+  //   K: chunk c of row r at r*KCH + (c ^ (r & 7))        (16-byte row reads)
+  //   V: chunk c of row r at r*KCH + (c ^ (2 * (r & 3)))  (transpose reads)
+  uint32_t k_fill[C::kLoads], v_fill[C::kLoads];
 #pragma unroll
-      for (int i = 0; i < LOADS; ++i) {
-        const int c = ltid + 128 * i;
-        const int key = c / KCH, ch = c % KCH;
-        // rows beyond the valid prefix are clamped to its last row: their
-        // scores are masked, and a finite row keeps 0 * V finite
-        const int row = min(k0 + key, a.kv_rows - 1);
-        staged[i] = *reinterpret_cast<const uint4*>(
-            k_base + static_cast<long long>(row) * a.k_row_stride + 8 * ch);
-      }
-    } else {
-      // unit = (key quad, channel group); 4 loads (one per key) per unit.
+  for (int i = 0; i < C::kLoads; ++i) {
+    const int p = (wave * C::kLoads + i) * 64 + lane;
+    const int row = p / KCH, slot = p % KCH;
+    k_fill[i] = static_cast<uint32_t>(row * a.k_row_stride * 2 + (slot ^ (row & 7)) * 16);
+    v_fill[i] = static_cast<uint32_t>(row * a.v_row_stride * 2 + (slot ^ (2 * (row & 3))) * 16);
+  }
+  // K operand of key block kb, step ks: row 32kb + n, chunk 2ks + h.
+  int k_read[KS];
 #pragma unroll
-      for (int u = 0; u < LOADS / 4; ++u) {
-        const int unit = ltid + 128 * u;
-        const int quad = unit / KCH, g = unit % KCH;
+  for (int ks = 0; ks < KS; ++ks) k_read[ks] = (n * KCH + ((2 * ks + h) ^ (n & 7))) * 16;
+  // V^T operand: the 16 lanes of group gq = lane/16 receive channels
+  // 32db + 16(gq%2) + (lane%16) and keys 4(gq/2) + (0..3) of the addressed
+  // rows; as a source, lane (kk = (lane%16)/4, b = lane%4) supplies row kk,
+  // channels 4b..4b+3 of that 16-channel span.
+  int v_read[DB];
+  {
+    const int gq = lane / 16, kk = (lane % 16) / 4, b = lane % 4;
+    const int row = 4 * (gq / 2) + kk;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int row = min(k0 + 4 * quad + r, a.kv_rows - 1);
-          staged[4 * u + r] = *reinterpret_cast<const uint4*>(
-              v_base + static_cast<long long>(row) * a.v_row_stride + 8 * g);
-        }
-      }
+    for (int db = 0; db < DB; ++db) {
+      const int chunk = 4 * db + 2 * (gq % 2) + b / 2;
+      v_read[db] = (row * KCH + (chunk ^ (2 * kk))) * 16 + (b % 2) * 8;
     }
-  };
-
-  auto commit = [&]() {
-    if (loads_k) {
-#pragma unroll
-      for (int i = 0; i < LOADS; ++i) {
-        const int c = ltid + 128 * i;
-        const int key = c / KCH, ch = c % KCH;
-        sm.k[row_major_index<KCH>(key, ch)] = staged[i];
-      }
-    } else {
-#pragma unroll
-      for (int u = 0; u < LOADS / 4; ++u) {
-        const int unit = ltid + 128 * u;
-        transposed_store<BN>(sm.vt, unit / KCH, unit % KCH, staged[4 * u + 0],
-                             staged[4 * u + 1], staged[4 * u + 2],
-                             staged[4 * u + 3]);
-      }
-    }
-  };
+  }
 
   // A workgroup processes query tile (q_tiles-1-pair) and then tile `pair`:
   // under the causal mask their key counts add up to the same total for every
@@ -146,172 +175,217 @@ flash_forward_kernel(FlashForwardArgs a) {
     const int q_tile = pass == 0 ? q_tiles - 1 - pair : pair;
     if (pass == 1 && q_tile == q_tiles - 1 - pair) break;
     const int q0 = q_tile * BM;
-    const int q_row = q0 + 32 * wave + n;
+    const int wave_q0 = q0 + 32 * G * wave;
 
-    // Q fragments (B operand of S^T): row q_row, channels 16ks + 8h .. +7.
-    bf16x8 qf[KS];
+    // Q fragments (B operand of S^T): row, channels 16ks + 8h .. +7.
+    bf16x8 qf[G][KS];
+    int q_row[G], row_limit[G];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const int row = min(q_row, a.q_rows - 1);
-      qf[ks] = as_bf16x8(*reinterpret_cast<const uint4*>(
-          q_base + static_cast<long long>(row) * a.q_row_stride + 16 * ks + 8 * h));
+    for (int g = 0; g < G; ++g) {
+      q_row[g] = wave_q0 + 32 * g + n;
+      const int row = min(q_row[g], a.q_rows - 1);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        qf[g][ks] = as_bf16x8(*reinterpret_cast<const uint4*>(
+            q_base + static_cast<long long>(row) * a.q_row_stride + 16 * ks + 8 * h));
+      // keys up to row_limit are visible to this lane's query
+      row_limit[g] = min(a.start_position + q_row[g], a.kv_rows - 1);
     }
-    floatx16 o_acc[DB];
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) o_acc[db][i] = 0.0f;
+    floatx16 o_acc[G][DB];
+    // Row sums come out of the matrix cores: an all-ones A operand makes every
+    // row of this accumulator the sum over keys of the bf16 probabilities.
+    floatx16 l_acc[G];
     // Online softmax in the log2 domain with a lazily updated reference
     // point: probabilities are 2^(s*scale2 - m_used); m_used follows the
-    // running row maximum only when that has grown by more than kLazy, so
-    // the accumulator rescale is rare.  The true maximum is tracked
-    // separately and the saved statistics are converted to it at the end.
+    // running row maximum only when that has grown by more than kLazy, so the
+    // accumulator rescale is rare.  The true maximum is tracked separately and
+    // the saved statistics are converted to it at the end.
     constexpr float kLazy = 8.0f;
-    float m_used = kMasked;   // reference point, score * scale * log2(e) units
-    float m_true = kMasked;   // running maximum of the raw scores
-    // Row sums come out of the matrix cores: an all-ones A operand makes
-    // every row of this accumulator the sum over keys of the bf16
-    // probabilities.
-    floatx16 l_acc;
+    float m_used[G], m_true[G];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) l_acc[i] = 0.0f;
+    for (int g = 0; g < G; ++g) {
+      m_used[g] = kMasked;
+      m_true[g] = kMasked;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) l_acc[g][i] = 0.0f;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o_acc[g][db][i] = 0.0f;
+    }
 
     const int last_row = min(q0 + BM, a.q_rows) - 1;
     const int visible = min(a.kv_rows, a.start_position + last_row + 1);
     const int tiles = (visible + BN - 1) / BN;
-    const int wave_last_key = a.start_position + q0 + 32 * wave + 31;
-    // keys up to `row_limit` are visible to this lane's query
-    const int row_limit = min(a.start_position + q_row, a.kv_rows - 1);
 
-    if (tiles > 0) fetch(0);
+    if (tiles > 0)
+      fill_stage<D, C::kLoads>(lds + (0 & 1) * C::kStageBytes, wave, k_base, v_base,
+                                 a.k_row_stride, a.v_row_stride, (0) * BN, a.kv_rows, k_fill,
+                                 v_fill);
     for (int tile = 0; tile < tiles; ++tile) {
       const int k0 = tile * BN;
-      __syncthreads();  // everyone finished reading the previous tile
-      commit();
+      // The tile's loads have landed; every wave is done with the other stage.
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
-      if (tile + 1 < tiles) fetch(tile + 1);
+      if (tile + 1 < tiles)
+        fill_stage<D, C::kLoads>(lds + ((tile + 1) & 1) * C::kStageBytes, wave, k_base, v_base,
+                                 a.k_row_stride, a.v_row_stride, (tile + 1) * BN, a.kv_rows, k_fill,
+                                 v_fill);
+      const unsigned char* k_tile = lds + (tile & 1) * C::kStageBytes;
+      const unsigned char* v_tile = k_tile + C::kTileBytes;
 #pragma unroll
       for (int kb = 0; kb < KB; ++kb) {
         const int kb0 = k0 + 32 * kb;
-        if (kb0 > wave_last_key) continue;  // nothing visible to this wave's rows
+        // nothing of this block is visible to any of the wave's rows
+        if (kb0 > a.start_position + wave_q0 + 32 * G - 1) continue;
         // ---- S^T = K Q^T for 32 keys ------------------------------------
-        floatx16 s;
+        bf16x8 kf[KS];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) s[i] = 0.0f;
-        const int key = 32 * kb + n;
+        for (int ks = 0; ks < KS; ++ks)
+          kf[ks] = as_bf16x8(*reinterpret_cast<const uint4*>(
+              k_tile + k_read[ks] + kb * 32 * KCH * 16));
+        floatx16 s[G];
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          const bf16x8 kf = as_bf16x8(sm.k[row_major_index<KCH>(key, 2 * ks + h)]);
-          s = mfma32(kf, qf[ks], s);
+        for (int g = 0; g < G; ++g) {
+#pragma unroll
+          for (int i = 0; i < 16; ++i) s[g][i] = 0.0f;
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) s[g] = mfma32(kf[ks], qf[g][ks], s[g]);
         }
-        // ---- mask (diagonal and tail blocks only), row maximum ----------
-        if (kb0 + 31 > a.start_position + q0 + 32 * wave || kb0 + 32 > a.kv_rows) {
-          const int limit = row_limit - kb0 - 4 * h;
+        bf16x8 pf[G][2];
 #pragma unroll
-          for (int i = 0; i < 16; ++i) s[i] = (8 * (i / 4) + (i % 4) > limit) ? kMasked : s[i];
+        for (int g = 0; g < G; ++g) {
+          const int group_q0 = a.start_position + wave_q0 + 32 * g;
+          // ---- mask (diagonal and tail blocks only), row maximum ----------
+          if (kb0 + 31 > group_q0 || kb0 + 32 > a.kv_rows) {
+            const int limit = row_limit[g] - kb0 - 4 * h;
+#pragma unroll
+            for (int i = 0; i < 16; ++i)
+              s[g][i] = (8 * (i / 4) + (i % 4) > limit) ? kMasked : s[g][i];
+          }
+          float row_max = fmaxf(fmaxf(s[g][0], s[g][1]), s[g][2]);
+#pragma unroll
+          for (int i = 3; i < 15; i += 2) row_max = fmaxf(fmaxf(row_max, s[g][i]), s[g][i + 1]);
+          row_max = fmaxf(row_max, s[g][15]);
+          m_true[g] = fmaxf(m_true[g], half_swap_max(row_max));
+          const float candidate = m_true[g] * scale2;
+          if (__any(candidate > m_used[g] + kLazy)) {
+            const float m_new = candidate > m_used[g] + kLazy ? candidate : m_used[g];
+            const float alpha = __builtin_amdgcn_exp2f(m_used[g] - m_new);
+            m_used[g] = m_new;
+            l_acc[g][0] *= alpha;
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+              for (int i = 0; i < 16; ++i) o_acc[g][db][i] *= alpha;
+          }
+          // ---- P^T = 2^(S^T scale2 - m_used) as bf16 B operands -----------
+#pragma unroll
+          for (int s2 = 0; s2 < 2; ++s2) {
+            uint32_t packed[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              packed[e] = pack_bf16(
+                  __builtin_amdgcn_exp2f(__builtin_fmaf(s[g][8 * s2 + 2 * e], scale2, -m_used[g])),
+                  __builtin_amdgcn_exp2f(
+                      __builtin_fmaf(s[g][8 * s2 + 2 * e + 1], scale2, -m_used[g])));
+            pf[g][s2] = __builtin_bit_cast(
+                bf16x8, make_uint4(packed[0], packed[1], packed[2], packed[3]));
+          }
         }
-        float row_max = fmaxf(s[0], s[1]);
-#pragma unroll
-        for (int i = 2; i < 16; i += 2) row_max = fmaxf(row_max, fmaxf(s[i], s[i + 1]));
-        row_max = fmaxf(row_max, __shfl_xor(row_max, 32, 64));
-        m_true = fmaxf(m_true, row_max);
-        const float candidate = m_true * scale2;
-        if (__any(candidate > m_used + kLazy)) {
-          const float m_new = candidate > m_used + kLazy ? candidate : m_used;
-          const float alpha = __builtin_amdgcn_exp2f(m_used - m_new);
-          m_used = m_new;
-          l_acc[0] *= alpha;
-#pragma unroll
-          for (int db = 0; db < DB; ++db)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) o_acc[db][i] *= alpha;
-        }
-        // ---- P^T = 2^(S^T scale2 - m_used); O^T += V^T P^T; l += 1^T P^T
+        // ---- O^T += V^T P^T; l += 1^T P^T ----------------------------------
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2) {
-          uint32_t packed[4];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            floatx2 two;
-            two[0] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[8 * s2 + 2 * e], scale2, -m_used));
-            two[1] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[8 * s2 + 2 * e + 1], scale2, -m_used));
-            packed[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(two, bf16x2));
-          }
-          const bf16x8 pf =
-              __builtin_bit_cast(bf16x8, make_uint4(packed[0], packed[1], packed[2], packed[3]));
-          const int chunk = 4 * kb + 2 * s2 + h;
-          l_acc = mfma32(ones, pf, l_acc);
+          bf16x8 vf[DB];
 #pragma unroll
           for (int db = 0; db < DB; ++db) {
-            const int d = 32 * db + n;
-            const bf16x8 vf = as_bf16x8(sm.vt[transposed_index<BN>(d, chunk)]);
-            o_acc[db] = mfma32(vf, pf, o_acc[db]);
+            // keys 16 s2 + 4h + (0..3), then 16 s2 + 8 + 4h + (0..3)
+            const int at = v_read[db] + (32 * kb + 16 * s2) * KCH * 16;
+            const uint2 lo = lds_transpose_read(v_tile, at);
+            const uint2 hi = lds_transpose_read(v_tile, at + 8 * KCH * 16);
+            vf[db] = __builtin_bit_cast(bf16x8, make_uint4(lo.x, lo.y, hi.x, hi.y));
+          }
+#pragma unroll
+          for (int g = 0; g < G; ++g) {
+            l_acc[g] = mfma32(ones, pf[g][s2], l_acc[g]);
+#pragma unroll
+            for (int db = 0; db < DB; ++db) o_acc[g][db] = mfma32(vf[db], pf[g][s2], o_acc[g][db]);
           }
         }
       }
     }
 
     // ---- epilogue ----------------------------------------------------------
-    // l_acc holds the sum over all keys (both lane halves contract into the
-    // same accumulator column).
-    const float l_used = l_acc[0] > 0.0f ? l_acc[0] : 1.0f;
-    const float inverse = 1.0f / l_used;
-    __syncthreads();  // LDS is reused to transpose the output tile
-    {
-      unsigned char* row = raw + (32 * wave + n) * OSTRIDE;
+    // A lane owns, for its query, channels 32db + 8j + 4h .. +3: four bf16 =
+    // one 8-byte store; the eight stores of a lane pair cover the row's bytes.
 #pragma unroll
-      for (int db = 0; db < DB; ++db)
+    for (int g = 0; g < G; ++g) {
+      // l_acc holds the sum over all keys (both lane halves contract into the
+      // same accumulator column).
+      const float l_used = l_acc[g][0] > 0.0f ? l_acc[g][0] : 1.0f;
+      const float inverse = 1.0f / l_used;
+      const int row = q_row[g];
+      if (row < a.q_rows) {
+        uint16_t* o_row = o_base + static_cast<long long>(row) * a.o_row_stride;
+        const uint16_t* gate_row =
+            gate_base ? gate_base + static_cast<long long>(row) * a.gate_row_stride : nullptr;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const int d = 32 * db + 8 * j + 4 * h;
-          floatx2 lo = {o_acc[db][4 * j] * inverse, o_acc[db][4 * j + 1] * inverse};
-          floatx2 hi = {o_acc[db][4 * j + 2] * inverse, o_acc[db][4 * j + 3] * inverse};
-          uint2 packed;
-          packed.x = __builtin_bit_cast(uint32_t, __builtin_convertvector(lo, bf16x2));
-          packed.y = __builtin_bit_cast(uint32_t, __builtin_convertvector(hi, bf16x2));
-          *reinterpret_cast<uint2*>(row + 2 * d) = packed;
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const int d = 32 * db + 8 * j + 4 * h;
+            float c[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) c[e] = o_acc[g][db][4 * j + e] * inverse;
+            if (gate_row) {
+              // out = bf16(bf16(core) * bf16(sigmoid(gate))): qwen_attention.cc:103-108
+              const uint2 gate_bits = *reinterpret_cast<const uint2*>(gate_row + d);
+              const uint32_t gw[2] = {gate_bits.x, gate_bits.y};
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                const float logit = __uint_as_float(
+                    (e & 1) ? (gw[e / 2] & 0xffff0000u) : (gw[e / 2] << 16));
+                c[e] = round_to_bf16(c[e]) * round_to_bf16(1.0f / (1.0f + expf(-logit)));
+              }
+            }
+            uint2 packed;
+            packed.x = pack_bf16(c[0], c[1]);
+            packed.y = pack_bf16(c[2], c[3]);
+            *reinterpret_cast<uint2*>(o_row + d) = packed;
+          }
+        if (h == 0) {
+          // statistics relative to the true maximum: attention.cc:161-168
+          const float normalizer =
+              l_used * __builtin_amdgcn_exp2f(m_used[g] - m_true[g] * scale2);
+          const float maximum = m_true[g] * a.scale;
+          const long long stat =
+              (static_cast<long long>(seq) * a.query_heads + head) * a.q_rows + row;
+          if (a.maxima) a.maxima[stat] = maximum;
+          if (a.normalizers) a.normalizers[stat] = normalizer;
+          if (a.lse)
+            a.lse[(static_cast<long long>(seq) * a.q_rows + row) * a.query_heads + head] =
+                maximum + __logf(normalizer);
         }
-    }
-    if (h == 0 && q_row < a.q_rows) {
-      // statistics relative to the true maximum: attention.cc:161-168
-      const float normalizer = l_used * __builtin_amdgcn_exp2f(m_used - m_true * scale2);
-      const float maximum = m_true * a.scale;
-      const long long stat =
-          (static_cast<long long>(seq) * a.query_heads + head) * a.q_rows + q_row;
-      if (a.maxima) a.maxima[stat] = maximum;
-      if (a.normalizers) a.normalizers[stat] = normalizer;
-      if (a.lse)
-        a.lse[(static_cast<long long>(seq) * a.q_rows + q_row) * a.query_heads + head] =
-            maximum + __logf(normalizer);
-    }
-    __syncthreads();
-    for (int c = tid; c < BM * KCH; c += kThreads) {
-      const int r = c / KCH, ch = c % KCH;
-      const int row = q0 + r;
-      if (row >= a.q_rows) continue;
-      uint4 bits = *reinterpret_cast<const uint4*>(raw + r * OSTRIDE + 16 * ch);
-      if (gate_base) {
-        // out = bf16(bf16(core) * bf16(sigmoid(gate))): qwen_attention.cc:103-108
-        const uint4 gate_bits = *reinterpret_cast<const uint4*>(
-            gate_base + static_cast<long long>(row) * a.gate_row_stride + 8 * ch);
-        const uint32_t cw[4] = {bits.x, bits.y, bits.z, bits.w};
-        const uint32_t gw[4] = {gate_bits.x, gate_bits.y, gate_bits.z, gate_bits.w};
-        uint32_t ow[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const float c0 = __uint_as_float(cw[e] << 16), c1 = __uint_as_float(cw[e] & 0xffff0000u);
-          const float g0 = __uint_as_float(gw[e] << 16), g1 = __uint_as_float(gw[e] & 0xffff0000u);
-          const float s0 = round_to_bf16(1.0f / (1.0f + expf(-g0)));
-          const float s1 = round_to_bf16(1.0f / (1.0f + expf(-g1)));
-          ow[e] = static_cast<uint32_t>(float_to_bf16_bits(c0 * s0)) |
-                  (static_cast<uint32_t>(float_to_bf16_bits(c1 * s1)) << 16);
-        }
-        bits = make_uint4(ow[0], ow[1], ow[2], ow[3]);
       }
-      *reinterpret_cast<uint4*>(o_base + static_cast<long long>(row) * a.o_row_stride +
-                                8 * ch) = bits;
     }
+    // the next pass refills stage 0 while slower waves may still read a stage
+    __syncthreads();
   }
+}
+
+// Experiment hook: PLUTO_HIP_FWD_SHAPE=<groups><waves> (e.g. "22") selects
+// the per-wave query groups and waves per workgroup of the 64-wide kernel.
+int forward_shape() {
+  static const int shape = [] {
+    const char* value = std::getenv("PLUTO_HIP_FWD_SHAPE");
+    return value ? std::atoi(value) : 0;
+  }();
+  return shape;
+}
+
+long long grid_blocks(const FlashForwardArgs& a, int block_rows, int sequences) {
+  const long long q_tiles = (a.q_rows + block_rows - 1) / block_rows;
+  return ((q_tiles + 1) / 2) * a.query_heads * sequences;
 }
 
 }  // namespace
@@ -325,6 +399,10 @@ bool flash_forward_supported(const FlashForwardArgs& a, int head_dim) {
   if (!aligned(a.q) || !aligned(a.k) || !aligned(a.v) || !aligned(a.out))
     return false;
   if (a.gate && !aligned(a.gate)) return false;
+  // K and V of one (sequence, head) are addressed through 32-bit buffer offsets
+  const long long limit = 1LL << 31;
+  if (a.kv_rows * a.k_row_stride * 2 >= limit || a.kv_rows * a.v_row_stride * 2 >= limit)
+    return false;
   return mult8(a.q_seq_stride) && mult8(a.q_row_stride) && mult8(a.q_head_stride) &&
          mult8(a.k_seq_stride) && mult8(a.k_row_stride) && mult8(a.k_head_stride) &&
          mult8(a.v_seq_stride) && mult8(a.v_row_stride) && mult8(a.v_head_stride) &&
@@ -336,14 +414,20 @@ bool flash_forward_supported(const FlashForwardArgs& a, int head_dim) {
 int launch_flash_forward(hipStream_t stream, const FlashForwardArgs& a,
                          int head_dim, int sequences) {
   if (!flash_forward_supported(a, head_dim)) return PLUTO_HIP_EUNSUPPORTED;
-  const long long q_tiles = (a.q_rows + BM - 1) / BM;
-  const long long blocks = ((q_tiles + 1) / 2) * a.query_heads * sequences;
+  int groups = 1, waves = 4;
+  if (head_dim == 64 && forward_shape() == 22) groups = 2, waves = 2;
+  if (head_dim == 64 && forward_shape() == 24) groups = 2, waves = 4;
+  const long long blocks = grid_blocks(a, 32 * groups * waves, sequences);
   if (blocks <= 0 || blocks > 0x7fffffffLL) return PLUTO_HIP_EINVAL;
-  dim3 grid(static_cast<unsigned>(blocks));
-  if (head_dim == 64)
-    flash_forward_kernel<64><<<grid, kThreads, 0, stream>>>(a);
+  const dim3 grid(static_cast<unsigned>(blocks));
+  if (head_dim == 128)
+    flash_forward_kernel<128, 1, 4><<<grid, 256, 0, stream>>>(a);
+  else if (groups == 1)
+    flash_forward_kernel<64, 1, 4><<<grid, 256, 0, stream>>>(a);
+  else if (waves == 2)
+    flash_forward_kernel<64, 2, 2><<<grid, 128, 0, stream>>>(a);
   else
-    flash_forward_kernel<128><<<grid, kThreads, 0, stream>>>(a);
+    flash_forward_kernel<64, 2, 4><<<grid, 256, 0, stream>>>(a);
   return launch_status();
 }
 
