@@ -27,8 +27,6 @@
 // reference keeps them FP32, attention.cc:151-156).
 #include "flash_fwd_mfma.h"
 
-#include <cstdlib>
-
 #include "mfma_tile.h"
 
 namespace pluto_hip {
@@ -244,6 +242,20 @@ flash_forward_kernel(FlashForwardArgs a) {
         for (int ks = 0; ks < KS; ++ks)
           kf[ks] = as_bf16x8(*reinterpret_cast<const uint4*>(
               k_tile + k_read[ks] + kb * 32 * KCH * 16));
+        // V^T operands of this block are requested now, so that their LDS
+        // latency passes under the first product and the softmax
+        bf16x8 vf[2][DB];
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+          for (int db = 0; db < DB; ++db) {
+            // keys 16 s2 + 4h + (0..3), then 16 s2 + 8 + 4h + (0..3)
+            const int at = v_read[db] + (32 * kb + 16 * s2) * KCH * 16;
+            const uint2 lo = lds_transpose_read(v_tile, at);
+            const uint2 hi = lds_transpose_read(v_tile, at + 8 * KCH * 16);
+            vf[s2][db] = __builtin_bit_cast(bf16x8, make_uint4(lo.x, lo.y, hi.x, hi.y));
+          }
+        __builtin_amdgcn_sched_barrier(0);
         floatx16 s[G];
 #pragma unroll
         for (int g = 0; g < G; ++g) {
@@ -296,20 +308,12 @@ flash_forward_kernel(FlashForwardArgs a) {
         // ---- O^T += V^T P^T; l += 1^T P^T ----------------------------------
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2) {
-          bf16x8 vf[DB];
-#pragma unroll
-          for (int db = 0; db < DB; ++db) {
-            // keys 16 s2 + 4h + (0..3), then 16 s2 + 8 + 4h + (0..3)
-            const int at = v_read[db] + (32 * kb + 16 * s2) * KCH * 16;
-            const uint2 lo = lds_transpose_read(v_tile, at);
-            const uint2 hi = lds_transpose_read(v_tile, at + 8 * KCH * 16);
-            vf[db] = __builtin_bit_cast(bf16x8, make_uint4(lo.x, lo.y, hi.x, hi.y));
-          }
 #pragma unroll
           for (int g = 0; g < G; ++g) {
             l_acc[g] = mfma32(ones, pf[g][s2], l_acc[g]);
 #pragma unroll
-            for (int db = 0; db < DB; ++db) o_acc[g][db] = mfma32(vf[db], pf[g][s2], o_acc[g][db]);
+            for (int db = 0; db < DB; ++db)
+              o_acc[g][db] = mfma32(vf[s2][db], pf[g][s2], o_acc[g][db]);
           }
         }
       }
@@ -373,16 +377,6 @@ flash_forward_kernel(FlashForwardArgs a) {
   }
 }
 
-// Experiment hook: PLUTO_HIP_FWD_SHAPE=<groups><waves> (e.g. "22") selects
-// the per-wave query groups and waves per workgroup of the 64-wide kernel.
-int forward_shape() {
-  static const int shape = [] {
-    const char* value = std::getenv("PLUTO_HIP_FWD_SHAPE");
-    return value ? std::atoi(value) : 0;
-  }();
-  return shape;
-}
-
 long long grid_blocks(const FlashForwardArgs& a, int block_rows, int sequences) {
   const long long q_tiles = (a.q_rows + block_rows - 1) / block_rows;
   return ((q_tiles + 1) / 2) * a.query_heads * sequences;
@@ -414,20 +408,13 @@ bool flash_forward_supported(const FlashForwardArgs& a, int head_dim) {
 int launch_flash_forward(hipStream_t stream, const FlashForwardArgs& a,
                          int head_dim, int sequences) {
   if (!flash_forward_supported(a, head_dim)) return PLUTO_HIP_EUNSUPPORTED;
-  int groups = 1, waves = 4;
-  if (head_dim == 64 && forward_shape() == 22) groups = 2, waves = 2;
-  if (head_dim == 64 && forward_shape() == 24) groups = 2, waves = 4;
-  const long long blocks = grid_blocks(a, 32 * groups * waves, sequences);
+  const long long blocks = grid_blocks(a, 128, sequences);
   if (blocks <= 0 || blocks > 0x7fffffffLL) return PLUTO_HIP_EINVAL;
   const dim3 grid(static_cast<unsigned>(blocks));
   if (head_dim == 128)
     flash_forward_kernel<128, 1, 4><<<grid, 256, 0, stream>>>(a);
-  else if (groups == 1)
-    flash_forward_kernel<64, 1, 4><<<grid, 256, 0, stream>>>(a);
-  else if (waves == 2)
-    flash_forward_kernel<64, 2, 2><<<grid, 128, 0, stream>>>(a);
   else
-    flash_forward_kernel<64, 2, 4><<<grid, 256, 0, stream>>>(a);
+    flash_forward_kernel<64, 1, 4><<<grid, 256, 0, stream>>>(a);
   return launch_status();
 }
 
