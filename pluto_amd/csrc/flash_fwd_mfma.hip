@@ -34,28 +34,6 @@ namespace {
 
 constexpr int BN = 64;  // keys per LDS tile
 
-typedef __attribute__((ext_vector_type(4))) short shortx4;
-typedef __attribute__((address_space(3))) void lds_void;
-
-// Buffer descriptor over [base, base + bytes): loads beyond `bytes` return 0.
-__device__ inline __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
-}
-
-// Four keys (rows r..r+3 chosen by the lane addresses) of one channel per lane.
-__device__ inline uint2 lds_transpose_read(const unsigned char* tile, int byte_offset) {
-  const shortx4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-      (__attribute__((address_space(3))) shortx4*)(tile + byte_offset));
-  return __builtin_bit_cast(uint2, v);
-}
-
-// Maximum over both lane halves (lanes l and l ^ 32) of a per-lane value.
-__device__ inline float half_swap_max(float v) {
-  const uint32_t bits = __builtin_bit_cast(uint32_t, v);
-  const auto pair = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
-  return fmaxf(__builtin_bit_cast(float, pair[0]), __builtin_bit_cast(float, pair[1]));
-}
-
 // Queues the loads of one K tile and one V tile (keys k0..k0+63) into an LDS
 // stage.  Lane l of load i of a wave writes 16 bytes at chunk
 // (wave*LOADS + i)*64 + l of the tile; k_fill/v_fill say which global bytes it

@@ -84,6 +84,113 @@ __device__ inline floatx16 mfma32(bf16x8 a, bf16x8 b, floatx16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
 }
 
+typedef __attribute__((ext_vector_type(4))) short shortx4;
+typedef __attribute__((address_space(3))) void lds_void;
+
+// Buffer descriptor over [base, base + bytes): loads beyond `bytes` return 0.
+__device__ inline __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
+}
+
+// LDS transpose read (ds_read_b64_tr_b16).  Within every group of 16 lanes,
+// source lane s = 4*kk + b supplies 8 bytes (four 16-bit elements) at its
+// address, and destination lane L = 4*b + e receives element e of source lanes
+// b, b+4, b+8, b+12.  When source lane (kk, b) points at row kk, columns
+// 4b..4b+3 of a row-major tile, lane L ends up with column L of rows 0..3.
+__device__ inline uint2 lds_transpose_read(const unsigned char* tile, int byte_offset) {
+  const shortx4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      (__attribute__((address_space(3))) shortx4*)(tile + byte_offset));
+  return __builtin_bit_cast(uint2, v);
+}
+
+// Values of a per-lane quantity in the lower and in the upper lane half,
+// each broadcast to both halves.  v_permlane32_swap exchanges the upper half of
+// its first register with the lower half of its second; starting from two
+// copies of v the first ends up all-lower, the second all-upper.  Written as
+// inline assembly because both registers are results; the wait states around
+// it cover the instruction's hazards with neighbouring vector instructions,
+// which the compiler cannot see into.
+__device__ inline void half_swap(float v, float& lower, float& upper) {
+  float first = v, second = v;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1"
+               : "+v"(first), "+v"(second));
+  lower = first;
+  upper = second;
+}
+// Per-lane value combined over both lane halves (lanes l and l ^ 32).
+__device__ inline float half_swap_max(float v) {
+  float lower, upper;
+  half_swap(v, lower, upper);
+  return fmaxf(lower, upper);
+}
+__device__ inline float half_swap_sum(float v) {
+  float lower, upper;
+  half_swap(v, lower, upper);
+  return lower + upper;
+}
+
+// Row-major bf16 tile [rows][D] in LDS whose 16-byte chunk c of row r sits at
+// slot c ^ tile_swizzle(r) of the row.  The permutation serves both ways the
+// matrix cores read such a tile without bank conflicts: 16-byte row reads
+// (eight consecutive rows, same chunk -> eight different slots) and transpose
+// reads (four consecutive rows x two adjacent chunks -> eight different slots).
+__device__ inline int tile_swizzle(int row) { return 2 * (row & 3) + ((row >> 2) & 1); }
+
+// Queues the fill of a ROWS x D tile by direct-to-LDS buffer loads.  Load i of
+// a lane writes 16 bytes at chunk (wave*LOADS + i)*64 + lane of the tile;
+// offsets[i] = byte offset, from the tile's first row, of the chunk that
+// belongs there (see tile_fill_offset).  base points at row `row0`; rows at or
+// beyond `rows` read as zero.
+template <int D, int LOADS>
+__device__ inline void tile_fill(unsigned char* tile, int wave, const uint16_t* base,
+                                 long long row_stride, int row0, int rows,
+                                 const uint32_t* offsets) {
+  const long long rows_left = rows - 1 - row0;
+  const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(
+      base, rows_left < 0 ? 0u : static_cast<uint32_t>((rows_left * row_stride + D) * 2));
+#pragma unroll
+  for (int i = 0; i < LOADS; ++i)
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(
+        rsrc, (lds_void*)(tile + (wave * LOADS + i) * 1024), 16, offsets[i], 0, 0, 0);
+}
+
+template <int D>
+__device__ inline uint32_t tile_fill_offset(int position, long long row_stride) {
+  constexpr int KCH = D / 8;
+  const int row = position / KCH, slot = position % KCH;
+  return static_cast<uint32_t>(row * row_stride * 2 + (slot ^ tile_swizzle(row)) * 16);
+}
+
+// Byte offset of this lane's 16-byte row read: row n, chunk c.
+template <int D>
+__device__ inline int tile_row_read(int n, int chunk) {
+  return (n * (D / 8) + (chunk ^ tile_swizzle(n))) * 16;
+}
+
+// Byte offset of this lane's transpose read for channel block db (channels
+// 32db .. 32db+31 land on lanes n = lane % 32): as a source the lane supplies
+// row 4*(lane/32) + kk, channels 32db + 16*((lane/16)%2) + 4b .. +3, with
+// kk = (lane%16)/4 and b = lane%4.  Add (16*s2 + 8*part) rows for the keys of
+// contraction step s2, part 0 = slots 0..3, part 1 = slots 4..7.
+template <int D>
+__device__ inline int tile_transpose_read(int lane, int db) {
+  const int gq = lane / 16, kk = (lane % 16) / 4, b = lane % 4;
+  const int row = 4 * (gq / 2) + kk;
+  const int chunk = 4 * db + 2 * (gq % 2) + b / 2;
+  return (row * (D / 8) + (chunk ^ tile_swizzle(row))) * 16 + (b % 2) * 8;
+}
+
+// Transposed A operand (32 channels x 16 rows in accumulator order) from a
+// row-major tile: rows 16*s2 + {0..3, 8..11} + 4*(lane/32) of `block`.
+template <int D>
+__device__ inline bf16x8 tile_transposed_operand(const unsigned char* block, int lane_offset,
+                                                 int s2) {
+  const int at = lane_offset + 16 * s2 * (D / 8) * 16;
+  const uint2 lo = lds_transpose_read(block, at);
+  const uint2 hi = lds_transpose_read(block, at + 8 * (D / 8) * 16);
+  return __builtin_bit_cast(bf16x8, make_uint4(lo.x, lo.y, hi.x, hi.y));
+}
+
 // XCD-aware renumbering of a 1-D grid: hardware deals workgroups round-robin
 // to the 8 XCDs (each with a private L2); this makes consecutive logical ids
 // land on the same XCD.
