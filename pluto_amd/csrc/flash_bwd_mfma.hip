@@ -118,8 +118,9 @@ flash_dq_kernel(GenericBackwardArgs a, float* __restrict__ lse2,
     const float row_lse2 = a.maxima[stats_base + q_load] * kLog2e +
                            __log2f(normalizer > 0.0f ? normalizer : 1.0f);
     if (h == 0 && q_row < T) {
-      a.deltas[stats_base + q_row] = -row_delta;  // the key-owned kernel adds it
-      lse2[stats_base + q_row] = row_lse2;
+      // the key-owned kernel starts its accumulators from these
+      a.deltas[stats_base + q_row] = -row_delta;
+      lse2[stats_base + q_row] = -row_lse2 / scale2;
     }
     floatx16 dq_acc[DB];
 #pragma unroll
@@ -343,18 +344,16 @@ flash_dkv_kernel(GenericBackwardArgs a, const float* __restrict__ lse2,
             }
         }
         // accumulator register i = (query qb0 + 8(i/4) + 4h + i%4, key n); the
-        // dP accumulator starts from -delta of its query
+        // score accumulator starts from -lse/scale of its query, the dP
+        // accumulator from -delta
         floatx16 s, dp;
-        float l2v[16];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const float4 l2 = *reinterpret_cast<const float4*>(&stat_lse2[32 * qb + 8 * j + 4 * h]);
           const float4 dl = *reinterpret_cast<const float4*>(&stat_delta[32 * qb + 8 * j + 4 * h]);
-          l2v[4 * j + 0] = l2.x; l2v[4 * j + 1] = l2.y; l2v[4 * j + 2] = l2.z; l2v[4 * j + 3] = l2.w;
+          s[4 * j + 0] = l2.x; s[4 * j + 1] = l2.y; s[4 * j + 2] = l2.z; s[4 * j + 3] = l2.w;
           dp[4 * j + 0] = dl.x; dp[4 * j + 1] = dl.y; dp[4 * j + 2] = dl.z; dp[4 * j + 3] = dl.w;
         }
-#pragma unroll
-        for (int i = 0; i < 16; ++i) s[i] = 0.0f;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
           const bf16x8 qa = as_bf16x8(*reinterpret_cast<const uint4*>(q_block + row_read[ks]));
@@ -364,7 +363,7 @@ flash_dkv_kernel(GenericBackwardArgs a, const float* __restrict__ lse2,
         }
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-          const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], scale2, -l2v[i]));
+          const float p = __builtin_amdgcn_exp2f(s[i] * scale2);
           s[i] = p;
           dp[i] = p * dp[i];
         }
