@@ -190,45 +190,73 @@ decode_split_kernel(DecodeArgs a, DecodeBatch batch) {
   }
 }
 
-// One workgroup per (sequence, query head): combines the blocks in ascending
-// order and applies the sigmoid gate (cached_attention_ops.cc:119-125).
-__global__ void __launch_bounds__(64)
+// One workgroup (4 waves) per (sequence, query head).  Wave w folds the blocks
+// w, w+4, w+8, ... in ascending order, then the four partial results are added
+// in wave order: a fixed summation tree, hence bitwise repeatable.  Ends with
+// the sigmoid gate (cached_attention_ops.cc:119-125).
+__global__ void __launch_bounds__(256)
 decode_combine_kernel(DecodeCombineArgs a, DecodeBatch batch) {
+  __shared__ float wave_max_lds[4];
+  __shared__ float partial_o[4][256];
+  __shared__ float partial_l[4];
   const int b = blockIdx.x / a.query_heads, head = blockIdx.x % a.query_heads;
   const int seq = batch.first + b;
   const int group = a.query_heads / a.key_value_heads;
   const int g = head / group, hh = head % group;
   const int D = a.head_dim;
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const int first = batch.block_start[b], blocks = batch.block_start[b + 1] - first;
+  // partial results of block j live at slot0 + j * slot_step
+  const long long slot0 = ((a.block_base + first) * a.key_value_heads + g) * group + hh;
+  const long long slot_step = static_cast<long long>(a.key_value_heads) * group;
   float maximum = kMasked;
-  for (int j = 0; j < blocks; ++j) {
-    const long long slot = ((a.block_base + first + j) * a.key_value_heads + g) * group + hh;
-    maximum = fmaxf(maximum, a.part_m[slot]);
-  }
+  for (int j = threadIdx.x; j < blocks; j += 256)
+    maximum = fmaxf(maximum, a.part_m[slot0 + j * slot_step]);
+  maximum = wave_max(maximum);
+  if (lane == 0) wave_max_lds[wave] = maximum;
+  __syncthreads();
+  maximum = fmaxf(fmaxf(wave_max_lds[0], wave_max_lds[1]), fmaxf(wave_max_lds[2], wave_max_lds[3]));
   float normalizer = 0.0f;
   float o[4] = {0.0f, 0.0f, 0.0f, 0.0f};  // head_dim <= 256 = 4 channels per lane
-  for (int j = 0; j < blocks; ++j) {
-    const long long slot = ((a.block_base + first + j) * a.key_value_heads + g) * group + hh;
-    const float w = __builtin_amdgcn_exp2f(a.part_m[slot] - maximum);
-    normalizer += a.part_l[slot] * w;
+  // four blocks per step: all loads of a step are issued before their use
+  for (int j0 = wave; j0 < blocks; j0 += 16) {
+    float bm[4], bl[4], bo[4][4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int c = threadIdx.x + 64 * i;
-      if (c < D) o[i] += a.part_o[slot * D + c] * w;
+    for (int u = 0; u < 4; ++u) {
+      const int j = j0 + 4 * u;
+      const bool valid = j < blocks;
+      const long long slot = slot0 + (valid ? j : j0) * slot_step;
+      bm[u] = valid ? a.part_m[slot] : kMasked;
+      bl[u] = a.part_l[slot];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int c = lane + 64 * i;
+        bo[u][i] = c < D ? a.part_o[slot * D + c] : 0.0f;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const float w = j0 + 4 * u < blocks ? __builtin_amdgcn_exp2f(bm[u] - maximum) : 0.0f;
+      normalizer += bl[u] * w;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[i] += bo[u][i] * w;
     }
   }
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int c = threadIdx.x + 64 * i;
-    if (c >= D) continue;
-    const float core = o[i] / normalizer;
-    const long long at = static_cast<long long>(seq) * a.query_heads + head;
-    const float logit = load_element(a.q_gate, (at * 2 + 1) * D + c, a.io_dtype);
-    const float sigmoid = 1.0f / (1.0f + expf(-logit));
-    const float value = a.round ? round_to_bf16(round_to_bf16(core) * round_to_bf16(sigmoid))
-                                : core * sigmoid;
-    store_element(a.out, at * D + c, a.io_dtype, value);
-  }
+  for (int i = 0; i < 4; ++i) partial_o[wave][lane + 64 * i] = o[i];
+  if (lane == 0) partial_l[wave] = normalizer;
+  __syncthreads();
+  const int c = threadIdx.x;
+  if (c >= D) return;
+  const float total = ((partial_l[0] + partial_l[1]) + partial_l[2]) + partial_l[3];
+  const float sum = ((partial_o[0][c] + partial_o[1][c]) + partial_o[2][c]) + partial_o[3][c];
+  const float core = sum / total;
+  const long long at = static_cast<long long>(seq) * a.query_heads + head;
+  const float logit = load_element(a.q_gate, (at * 2 + 1) * D + c, a.io_dtype);
+  const float sigmoid = 1.0f / (1.0f + expf(-logit));
+  const float value = a.round ? round_to_bf16(round_to_bf16(core) * round_to_bf16(sigmoid))
+                              : core * sigmoid;
+  store_element(a.out, at * D + c, a.io_dtype, value);
 }
 
 // Two-pass probability rows for inspection: one workgroup per (query head,
@@ -318,7 +346,7 @@ int launch_decode_fast(hipStream_t stream, const DecodeArgs& a, const DecodeBatc
 
 int launch_decode_combine(hipStream_t stream, const DecodeCombineArgs& a,
                           const DecodeBatch& batch) {
-  decode_combine_kernel<<<batch.count * a.query_heads, 64, 0, stream>>>(a, batch);
+  decode_combine_kernel<<<batch.count * a.query_heads, 256, 0, stream>>>(a, batch);
   return launch_status();
 }
 
