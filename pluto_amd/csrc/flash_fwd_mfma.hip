@@ -94,10 +94,25 @@ flash_forward_kernel(FlashForwardArgs a) {
   // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.
   // Renumber them so that the workgroups sharing one (sequence, kv head) K/V
   // stream run on the same XCD.
-  const int logical = xcd_logical_block();
-  const int pair = logical % pairs;
-  const int head = (logical / pairs) % a.query_heads;
-  const int seq = logical / (pairs * a.query_heads);
+  // Two schedules.  Paired (kPaired): a workgroup processes query tile
+  // q_tiles-1-pair and then tile pair; under the causal mask every pair
+  // carries the same work, which balances perfectly when all workgroups are
+  // resident at once.  Unpaired: one tile per workgroup, heaviest tiles first,
+  // for kernels whose resident workgroups are fewer than the grid (the greedy
+  // dispatch of ever lighter tiles then fills the machine evenly).
+  constexpr bool kPaired = D == 64;
+  int pair, head, seq;
+  if constexpr (kPaired) {
+    const int logical = xcd_logical_block();
+    pair = logical % pairs;
+    head = (logical / pairs) % a.query_heads;
+    seq = logical / (pairs * a.query_heads);
+  } else {
+    const int units = gridDim.x / q_tiles;  // (sequence, head) pairs
+    pair = q_tiles - 1 - blockIdx.x / units;
+    head = (blockIdx.x % units) % a.query_heads;
+    seq = (blockIdx.x % units) / a.query_heads;
+  }
   const int kv_head = head / a.group;
 
   const uint16_t* q_base = a.q + seq * a.q_seq_stride + head * a.q_head_stride;
@@ -148,8 +163,8 @@ flash_forward_kernel(FlashForwardArgs a) {
   // under the causal mask their key counts add up to the same total for every
   // pair, so all workgroups carry equal work.
   for (int pass = 0; pass < 2; ++pass) {
-    const int q_tile = pass == 0 ? q_tiles - 1 - pair : pair;
-    if (pass == 1 && q_tile == q_tiles - 1 - pair) break;
+    const int q_tile = (kPaired && pass == 0) ? q_tiles - 1 - pair : pair;
+    if (pass == 1 && (!kPaired || q_tile == q_tiles - 1 - pair)) break;
     const int q0 = q_tile * BM;
     const int wave_q0 = q0 + 32 * G * wave;
 
@@ -355,9 +370,9 @@ flash_forward_kernel(FlashForwardArgs a) {
   }
 }
 
-long long grid_blocks(const FlashForwardArgs& a, int block_rows, int sequences) {
+long long grid_blocks(const FlashForwardArgs& a, int block_rows, int sequences, bool paired) {
   const long long q_tiles = (a.q_rows + block_rows - 1) / block_rows;
-  return ((q_tiles + 1) / 2) * a.query_heads * sequences;
+  return (paired ? (q_tiles + 1) / 2 : q_tiles) * a.query_heads * sequences;
 }
 
 }  // namespace
@@ -386,7 +401,7 @@ bool flash_forward_supported(const FlashForwardArgs& a, int head_dim) {
 int launch_flash_forward(hipStream_t stream, const FlashForwardArgs& a,
                          int head_dim, int sequences) {
   if (!flash_forward_supported(a, head_dim)) return PLUTO_HIP_EUNSUPPORTED;
-  const long long blocks = grid_blocks(a, 128, sequences);
+  const long long blocks = grid_blocks(a, 128, sequences, head_dim == 64);
   if (blocks <= 0 || blocks > 0x7fffffffLL) return PLUTO_HIP_EINVAL;
   const dim3 grid(static_cast<unsigned>(blocks));
   if (head_dim == 128)
