@@ -16,6 +16,11 @@ __device__ inline float maybe_round(float x, bool round) {
   return round ? round_to_bf16(x) : x;
 }
 
+// Two already bf16-representable floats as packed bf16 bits.
+__device__ inline uint32_t pack_bf16_bits(float lo, float hi) {
+  return (__float_as_uint(lo) >> 16) | (__float_as_uint(hi) & 0xffff0000u);
+}
+
 __device__ inline double wave_sum_f64(double v) {
   for (int offset = 32; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, 64);
   return v;
@@ -112,6 +117,95 @@ prefill_prepare_kernel(PrefillPrepareArgs a) {
   }
 }
 
+// Vectorised form of the same preparation for bf16 inputs, a bf16 query buffer
+// and a bf16 cache with rounding on: a thread owns 8 consecutive channels (one
+// 16-byte load and store), the D/8 threads of a (row, head) are neighbouring
+// lanes.  Requires rotary_dim/2 to be a multiple of 8 so that a thread's RoPE
+// partners all sit in one other thread.  Arithmetic and rounding points are
+// those of normalize_rotate above.
+template <int D>
+__global__ void __launch_bounds__(256)
+prefill_prepare_bf16_kernel(PrefillPrepareArgs a) {
+  constexpr int LANES = D / 8;
+  const int heads = a.query_heads + a.key_value_heads;
+  const long long thread = static_cast<long long>(blockIdx.x) * 256 + threadIdx.x;
+  const long long unit = thread / LANES;
+  if (unit >= static_cast<long long>(a.length) * heads) return;  // whole groups drop out
+  const int chunk = static_cast<int>(thread % LANES);
+  const int row = static_cast<int>(unit / heads);
+  const int head = static_cast<int>(unit % heads);
+  const int half = a.rotary_dim / 2;
+  const bool is_query = head < a.query_heads;
+  const int kv = head - a.query_heads;
+  const uint16_t* in;
+  uint16_t* out;
+  const float* weight;
+  if (is_query) {
+    in = static_cast<const uint16_t*>(a.qg) +
+         (static_cast<long long>(row) * a.query_heads + head) * 2 * D;
+    out = static_cast<uint16_t*>(a.q_out) + (static_cast<long long>(row) * a.query_heads + head) * D;
+    weight = a.q_norm;
+  } else {
+    in = static_cast<const uint16_t*>(a.k) +
+         (static_cast<long long>(row) * a.key_value_heads + kv) * D;
+    out = static_cast<uint16_t*>(a.cache.keys) +
+          static_cast<long long>(a.start_position + row) * a.cache.token_stride +
+          kv * a.cache.head_stride;
+    weight = a.k_norm;
+  }
+  const uint4 bits = *reinterpret_cast<const uint4*>(in + 8 * chunk);
+  const uint32_t words[4] = {bits.x, bits.y, bits.z, bits.w};
+  float x[8];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    x[2 * i] = __uint_as_float(words[i] << 16);
+    x[2 * i + 1] = __uint_as_float(words[i] & 0xffff0000u);
+  }
+  double square = 0.0;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) square += static_cast<double>(x[e] * x[e]);
+#pragma unroll
+  for (int offset = 1; offset < LANES; offset <<= 1) square += __shfl_xor(square, offset, 64);
+  const double inverse = 1.0 / sqrt(square / D + static_cast<double>(a.epsilon));
+  const float4 w0 = *reinterpret_cast<const float4*>(weight + 8 * chunk);
+  const float4 w1 = *reinterpret_cast<const float4*>(weight + 8 * chunk + 4);
+  const float w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+  float n[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e)
+    n[e] = round_to_bf16(static_cast<float>(x[e] * inverse * (1.0 + static_cast<double>(w[e]))));
+  // RoPE partner channels c +- half live `half / 8` lanes away.
+  const int first = 8 * chunk;
+  const bool rotated = first < a.rotary_dim;
+  const bool lower = first < half;
+  const int lane = threadIdx.x % 64;
+  const int partner_lane = lower ? lane + half / 8 : lane - half / 8;
+  float result[8];
+  const float* cos_row = a.cosines + static_cast<long long>(row) * half + (lower ? first : first - half);
+  const float* sin_row = a.sines + static_cast<long long>(row) * half + (lower ? first : first - half);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float np = __shfl(n[e], rotated ? partner_lane : lane, 64);
+    result[e] = n[e];
+    if (rotated) {
+      const float p = round_to_bf16(n[e] * cos_row[e]);
+      const float q = round_to_bf16(np * sin_row[e]);
+      result[e] = round_to_bf16(lower ? p - q : p + q);
+    }
+  }
+  *reinterpret_cast<uint4*>(out + 8 * chunk) =
+      make_uint4(pack_bf16_bits(result[0], result[1]), pack_bf16_bits(result[2], result[3]),
+                 pack_bf16_bits(result[4], result[5]), pack_bf16_bits(result[6], result[7]));
+  if (!is_query) {
+    const uint16_t* v_in = static_cast<const uint16_t*>(a.v) +
+                           (static_cast<long long>(row) * a.key_value_heads + kv) * D;
+    uint16_t* v_out = static_cast<uint16_t*>(a.cache.values) +
+                      static_cast<long long>(a.start_position + row) * a.cache.token_stride +
+                      kv * a.cache.head_stride;
+    *reinterpret_cast<uint4*>(v_out + 8 * chunk) = *reinterpret_cast<const uint4*>(v_in + 8 * chunk);
+  }
+}
+
 // Decode: one wave per (sequence, head); the angle is evaluated in place.
 __global__ void __launch_bounds__(256)
 decode_prepare_kernel(DecodePrepareArgs a, DecodeBatch batch) {
@@ -173,6 +267,26 @@ int launch_rope_table(hipStream_t stream, int start_position, int length,
 int launch_prefill_prepare(hipStream_t stream, const PrefillPrepareArgs& a) {
   const long long units =
       static_cast<long long>(a.length) * (a.query_heads + a.key_value_heads);
+  const int d = a.head_dim;
+  auto aligned = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
+  const bool vectorised =
+      a.round && a.q_out_dtype == PLUTO_HIP_BF16 && a.cache.dtype == PLUTO_HIP_BF16 &&
+      (d == 64 || d == 128 || d == 256) && (a.rotary_dim / 2) % 8 == 0 &&
+      a.cache.token_stride % 8 == 0 && a.cache.head_stride % 8 == 0 && aligned(a.qg) &&
+      aligned(a.k) && aligned(a.v) && aligned(a.q_out) && aligned(a.cache.keys) &&
+      aligned(a.cache.values) && aligned(a.q_norm) && aligned(a.k_norm) && aligned(a.cosines) &&
+      aligned(a.sines);
+  if (vectorised) {
+    const long long threads = units * (d / 8);
+    const unsigned blocks = static_cast<unsigned>((threads + 255) / 256);
+    if (d == 64)
+      prefill_prepare_bf16_kernel<64><<<blocks, 256, 0, stream>>>(a);
+    else if (d == 128)
+      prefill_prepare_bf16_kernel<128><<<blocks, 256, 0, stream>>>(a);
+    else
+      prefill_prepare_bf16_kernel<256><<<blocks, 256, 0, stream>>>(a);
+    return launch_status();
+  }
   prefill_prepare_kernel<<<static_cast<unsigned>((units + 3) / 4), 256, 0, stream>>>(a);
   return launch_status();
 }
