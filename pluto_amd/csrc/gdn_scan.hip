@@ -279,105 +279,342 @@ __device__ inline bf16x8 tiles_to_operand(const floatx4& lo, const floatx4& hi) 
   return out;
 }
 
-__global__ void __launch_bounds__(64)
+// LDS stage of the sequential kernel: the chunk's -W | cQ | A2 | Kt fragments
+// exactly as they sit in the scratch (56 KiB, contiguous there too) followed
+// by the 4 KiB slice of U of each computing wave and the chunk's tail.
+constexpr int kScanOperandBytes = static_cast<int>(kGdnOffsetDecay - kGdnOffsetW);  // 57344
+// Column slices (computing waves) per workgroup: they would share the operand
+// fragments of a stage, each with its own 4 KiB slice of U in it.
+constexpr int kScanGroup = 1;
+constexpr int kScanStageBytes = kScanOperandBytes + (4 * kScanGroup + 1) * 1024;
+constexpr int kScanStages = 2;
+
+typedef __attribute__((address_space(3))) unsigned char lds_byte;
+typedef __attribute__((address_space(3))) const uint32x4 lds_u32x4;
+typedef __attribute__((address_space(3))) const floatx4 lds_f32x4;
+__device__ inline bf16x8 words_to_bf16x8(uint32x4 v) { return __builtin_bit_cast(bf16x8, v); }
+
+// One direct-to-LDS load of 16 bytes per lane: lane l fetches
+// descriptor base + voffset(l) + soffset and the hardware writes it at LDS
+// byte lds_address + 16 l.  Issued as inline assembly on purpose: the compiler
+// does not see an LDS write, so it does not make later reads of the OTHER
+// stage wait for this load; the kernel orders the accesses itself with
+// s_waitcnt vmcnt (see gdn_chunk_scan).
+__device__ inline void lds_dma_16(uint32x4 descriptor, uint32_t lds_address, uint32_t voffset,
+                                  uint32_t soffset) {
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 0\n\t"
+      "buffer_load_dwordx4 %1, %2, %3 offen lds"
+      :
+      : "s"(lds_address), "v"(voffset), "s"(descriptor), "s"(soffset)
+      : "memory", "m0");
+}
+
+// The direct-to-LDS loads of one chunk: 56 + 4 * kScanGroup + 1 loads of 1 KiB
+// (operand fragments, this workgroup's slices of U, the chunk's tail with its
+// decay).
+// Loader wave LOADER of LOADERS issues every LOADERS-th of them.
+// `chunk_offset` is the byte offset of the chunk's scratch within the
+// (sequence, head) region the descriptor covers.
+constexpr int kScanFillLoads = kScanOperandBytes / 1024 + 4 * kScanGroup + 1;
+template <int LOADER, int LOADERS>
+__device__ __forceinline__ void scan_fill(uint32_t stage_address, uint32x4 descriptor,
+                                          uint32_t chunk_offset, int slice, int lane) {
+  const uint32_t lane_bytes = static_cast<uint32_t>(lane) * 16u;
+  // fully unrolled: a lone wave issues a loop's scalar bookkeeping far slower
+  // than the memory pipeline takes loads
+#pragma unroll
+  for (int f = LOADER; f < kScanFillLoads; f += LOADERS) {
+    if (f < kScanOperandBytes / 1024) {
+      lds_dma_16(descriptor, stage_address + f * 1024, lane_bytes,
+                 chunk_offset + static_cast<uint32_t>(kGdnOffsetW) + f * 1024);
+    } else if (f < kScanFillLoads - 1) {
+      // `slice` is the first of the workgroup's kScanGroup slices
+      const int j = f - kScanOperandBytes / 1024;
+      lds_dma_16(descriptor, stage_address + f * 1024, lane_bytes,
+                 chunk_offset + static_cast<uint32_t>(kGdnOffsetU) +
+                     ((j % 4) * SLICES + slice + j / 4) * 1024);
+    } else {
+      // the tail is shorter than 1 KiB: its offset goes through the
+      // bounds-checked lane offset so that lanes past the end of the scratch
+      // read zeros
+      lds_dma_16(descriptor, stage_address + f * 1024,
+                 lane_bytes + chunk_offset + static_cast<uint32_t>(kGdnOffsetDecay), 0);
+    }
+  }
+}
+
+// Loader waves per workgroup, and what each needs at run time: the fill for its
+// index, and a wait that lets exactly its share of one (the younger) fill stay
+// in flight.
+constexpr int kScanLoaders = 3;
+static_assert(kScanLoaders == 2 || kScanLoaders == 3, "scan_fill_as and scan_wait_older_fill list the loaders");
+constexpr int scan_fill_share(int loader) {
+  return (kScanFillLoads - loader + kScanLoaders - 1) / kScanLoaders;
+}
+// (a wave whose two fills exceed the 63 operations its vector-memory counter
+// holds merely stalls at the issue of the last few loads)
+static_assert(scan_fill_share(0) <= 63, "the wait for the older fill must be encodable");
+__device__ __forceinline__ void scan_fill_as(int loader, uint32_t stage_address, uint32x4 descriptor,
+                                             uint32_t chunk_offset, int slice, int lane) {
+  if (loader == 0) scan_fill<0, kScanLoaders>(stage_address, descriptor, chunk_offset, slice, lane);
+  else if (loader == 1 || kScanLoaders == 2)
+    scan_fill<1, kScanLoaders>(stage_address, descriptor, chunk_offset, slice, lane);
+  else scan_fill<kScanLoaders - 1, kScanLoaders>(stage_address, descriptor, chunk_offset, slice, lane);
+}
+__device__ __forceinline__ void scan_wait_older_fill(int loader) {
+  if (loader == 0) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(scan_fill_share(0)) : "memory");
+  else if (loader == 1 || kScanLoaders == 2)
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(scan_fill_share(1)) : "memory");
+  else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(scan_fill_share(kScanLoaders - 1)) : "memory");
+}
+
+// Pulls this workgroup's eighth of a future chunk's scratch through L2 so that
+// it is there by the time the workgroups of the (sequence, head) fetch it for
+// real: the loader waves cannot keep enough real loads in flight to cover the
+// latency of HBM.  These are full-width loads (1 KiB per instruction): what
+// bounds a compute unit is the number of requests it has in flight, and a
+// narrow load per cache sector is one request per lane.  They go straight to
+// an LDS dump area nobody reads, so they need no registers and the issuing
+// wave never waits for them.
+constexpr int kScanTouchBytes = (static_cast<int>(kGdnChunkBytes) / SLICES + 1023) / 1024 * 1024;
+constexpr int kScanTouchLoads = kScanTouchBytes / 1024;
+constexpr int kScanAhead = 4;
+__device__ inline void scan_touch(uint32x4 descriptor, uint32_t dump_address, uint32_t chunk_offset,
+                                  int slice, int lane) {
+  // the lane offset is the bounds-checked one: past the end of the scratch
+  // the loads return zeros
+  const uint32_t voffset = chunk_offset + static_cast<uint32_t>(slice) * (kGdnChunkBytes / SLICES) +
+                           static_cast<uint32_t>(lane) * 16u;
+#pragma unroll
+  for (int i = 0; i < kScanTouchLoads; ++i) lds_dma_16(descriptor, dump_address, voffset, i * 1024);
+}
+
+// One workgroup per (sequence, head, kScanGroup slices of 16 state columns),
+// one wave per SIMD so that a computing wave may use the whole register file:
+// kScanGroup computing waves, one per slice, and kScanLoaders loader waves.
+// A stage holds one chunk.  The computing wave moves the chunk's fragments into
+// registers as its matrix instructions need them and releases the stage before
+// the chunk's second phase; the loaders then stream chunk c+2 into it
+// (asynchronous direct-to-LDS loads), so each loader has two fills in flight.
+// Two workgroup barriers per chunk hand the stages over: "landed" and "free".
+// A wave that issues long runs of loads stalls at issue while the memory
+// pipeline digests them, which is why the computing wave issues only the few
+// loads that warm L2.
+//
+// Measured on MI355X at 2 x 16 heads x 16384 tokens (256 chunks, one workgroup
+// per compute unit), per chunk: the matrix instructions and the 60 KiB of LDS
+// reads take about 0.85 us when nothing else runs, the fill of a stage 0.65 us
+// when its data is in L2 and about 1 us when it comes from HBM; the two
+// overlap only in part (1.3 us).  Two slices per workgroup halve the traffic
+// from L2 but double the LDS reads of a compute unit, and measure slower.
+constexpr int kScanThreads = 64 * (kScanGroup + kScanLoaders);
+static_assert(kScanThreads <= 256, "one wave per SIMD");
+
+// The workgroup barriers that hand an LDS stage over.  A loader arrives at the
+// "landed" barrier once the stage's direct-to-LDS loads are complete (the
+// caller waits for them); a computing wave arrives at the "free" barrier once
+// its LDS reads are done, without waiting for its own vector-memory operations
+// (output stores, L2 touches), which nobody in the workgroup depends on.
+__device__ __forceinline__ void scan_barrier() { asm volatile("s_barrier" ::: "memory"); }
+__device__ __forceinline__ void scan_handover_compute() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+// One chunk of the sequential chain, computed from the operands in `stage`.
+struct ScanContext {
+  uint16_t* out;
+  int length, value_heads;
+  const char* base;
+  int chunks, slice, lane, hq, m, seq, head;
+};
+
+__device__ __forceinline__ void scan_step(const ScanContext ctx, const uint32x4 descriptor,
+                                          int chunk, const lds_byte* stage, floatx4 (&s)[8]) {
+  struct {
+    uint16_t* out;
+    int length, value_heads;
+  } a = {ctx.out, ctx.length, ctx.value_heads};
+  const int slice = ctx.slice, lane = ctx.lane, hq = ctx.hq, m = ctx.m;
+  const int seq = ctx.seq, head = ctx.head;
+  const float decay = *(const __attribute__((address_space(3))) float*)(stage + kScanStageBytes - 1024);
+  lds_u32x4* neg_w = (lds_u32x4*)(stage) + lane;
+  lds_u32x4* q_in = (lds_u32x4*)(stage + (kGdnOffsetQ - kGdnOffsetW)) + lane;
+  lds_u32x4* a2_in = (lds_u32x4*)(stage + (kGdnOffsetA2 - kGdnOffsetW)) + lane;
+  lds_u32x4* kt_in = (lds_u32x4*)(stage + (kGdnOffsetKt - kGdnOffsetW)) + lane;
+  lds_f32x4* u_in = (lds_f32x4*)(stage + kScanOperandBytes + 4096 * (slice % kScanGroup)) + lane;
+
+  // LDS reads are issued well ahead of the matrix instructions that consume
+  // them: the first-phase fragments (-W, cQ, U) one token tile ahead, the
+  // second-phase fragments (Kt, A2) a quarter per token tile behind those.
+  // Once the last of them is in registers, before the last token tile's
+  // products, the stage goes back to the loaders.
+  uint32x4 a2_reg[8], kt_reg[16];
+  uint32x4 w_reg[2][4], q_reg[2][4];
+  floatx4 u_reg[2];
+#pragma unroll
+  for (int kb = 0; kb < 4; ++kb) {
+    w_reg[0][kb] = neg_w[kb * 64];
+    q_reg[0][kb] = q_in[kb * 64];
+  }
+  u_reg[0] = u_in[0];
+  __builtin_amdgcn_sched_barrier(0);
+  bf16x8 sb[4];
+#pragma unroll
+  for (int kb = 0; kb < 4; ++kb) sb[kb] = tiles_to_operand(s[2 * kb], s[2 * kb + 1]);
+  // D = U - W S0 and the S0 part of O = exp(c) Q S0 + (M o Q K^T) D
+  floatx4 d[4], o[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    if (i + 1 < 4) {
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb) {
+        w_reg[(i + 1) % 2][kb] = neg_w[(4 * (i + 1) + kb) * 64];
+        q_reg[(i + 1) % 2][kb] = q_in[(4 * (i + 1) + kb) * 64];
+      }
+      u_reg[(i + 1) % 2] = u_in[(i + 1) * 64];
+#pragma unroll
+      for (int f = 0; f < 8; ++f) {
+        if (i < 2) kt_reg[8 * i + f] = kt_in[(8 * i + f) * 64];
+        else a2_reg[f] = a2_in[f * 64];
+      }
+    } else {
+      scan_handover_compute();
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    floatx4 acc = u_reg[i % 2];
+    floatx4 out_acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) {
+      acc = mfma16(words_to_bf16x8(w_reg[i % 2][kb]), sb[kb], acc);
+      out_acc = mfma16(words_to_bf16x8(q_reg[i % 2][kb]), sb[kb], out_acc);
+    }
+    d[i] = acc;
+    o[i] = out_acc;
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  bf16x8 db[2];
+  db[0] = tiles_to_operand(d[0], d[1]);
+  db[1] = tiles_to_operand(d[2], d[3]);
+  // S = exp(c_C) S0 + (diag(exp(c_C - c)) K)^T D, the chain the next chunk
+  // waits for, goes first and the outputs follow; in both, products that depend
+  // on each other are issued eight (four) instructions apart.
+#pragma unroll
+  for (int t = 0; t < 8; ++t) s[t] = s[t] * decay;
+#pragma unroll
+  for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+    for (int t = 0; t < 8; ++t) s[t] = mfma16(words_to_bf16x8(kt_reg[2 * t + kb]), db[kb], s[t]);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+#pragma unroll
+  for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = mfma16(words_to_bf16x8(a2_reg[2 * i + kb]), db[kb], o[i]);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  // outputs: rows 16i + 4hq + r of the chunk, column 16*slice + m
+  uint16_t* out_row = a.out +
+      ((static_cast<long long>(seq) * a.length + chunk * C + 4 * hq) * a.value_heads + head) * DV +
+      16 * slice + m;
+  const long long row_step = static_cast<long long>(a.value_heads) * DV;
+  if (chunk * C + C <= a.length) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) out_row[(16 * i + r) * row_step] = float_to_bf16_bits(o[i][r]);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (chunk * C + 16 * i + 4 * hq + r < a.length)
+          out_row[(16 * i + r) * row_step] = float_to_bf16_bits(o[i][r]);
+  }
+}
+
+__global__ void __launch_bounds__(kScanThreads)
 gdn_chunk_scan(GdnArgs a) {
-  const int lane = threadIdx.x, hq = lane / 16, m = lane % 16;
+  __shared__ __attribute__((aligned(1024))) unsigned char stage0[kScanStageBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char stage1[kScanStageBytes];
+  __shared__ __attribute__((aligned(256))) unsigned char dump[1024];
+  const int lane = threadIdx.x % 64, hq = lane / 16, m = lane % 16;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
   const int chunks = (a.length + C - 1) / C;
-  // The 8 column slices of one (sequence, head) read the same operands: keep
-  // them on one XCD so its L2 serves 7 of the 8 reads.
+  // The workgroups of one (sequence, head) read the same operands: keep them
+  // on one XCD so that its L2 serves all but the first read.
   int logical = blockIdx.x;
   if (gridDim.x % 8 == 0) logical = (blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8;
-  const int slice = logical % SLICES;
-  const int bh = logical / SLICES;
+  constexpr int kGroups = SLICES / kScanGroup;
+  const int first_slice = (logical % kGroups) * kScanGroup;
+  const int slice = first_slice + min(wave, kScanGroup - 1);
+  const int bh = logical / kGroups;
   const int head = bh % a.value_heads, seq = bh / a.value_heads;
   float* state = a.state + static_cast<size_t>(bh) * DK * DV;
+  const char* base = a.workspace + static_cast<size_t>(bh) * chunks * kGdnChunkBytes;
+  // raw buffer descriptor: base address, no stride, size in bytes, data format
+  const uint64_t address = reinterpret_cast<uint64_t>(base);
+  const uint32x4 descriptor = {static_cast<uint32_t>(address),
+                               static_cast<uint32_t>(address >> 32) & 0xffffu,
+                               static_cast<uint32_t>(chunks * kGdnChunkBytes), 0x00020000u};
+  const uint32_t stage0_address = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_byte*)stage0));
+  const uint32_t stage1_address = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_byte*)stage1));
 
+  // Every wave passes two barriers per chunk: "landed" (the chunk's stage is
+  // complete) and "free" (the computing waves have copied it to registers).
+  const uint32_t dump_address =
+      static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_byte*)dump));
+  if (wave >= kScanGroup) {
+    const int loader = wave - kScanGroup;
+    scan_fill_as(loader, stage0_address, descriptor, 0, first_slice, lane);
+    if (chunks > 1)
+      scan_fill_as(loader, stage1_address, descriptor, static_cast<uint32_t>(kGdnChunkBytes),
+                   first_slice, lane);
+    for (int chunk = 0; chunk < chunks; ++chunk) {
+      // loads complete in issue order: all but the younger fill have landed
+      if (chunk + 1 < chunks) scan_wait_older_fill(loader);
+      else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      scan_barrier();  // landed
+      scan_barrier();  // free
+      if (chunk + 2 < chunks)
+        scan_fill_as(loader, (chunk & 1) ? stage1_address : stage0_address, descriptor,
+                     static_cast<uint32_t>(chunk + 2) * static_cast<uint32_t>(kGdnChunkBytes),
+                     first_slice, lane);
+    }
+    return;
+  }
+
+  ScanContext ctx;
+  ctx.out = a.out;
+  ctx.length = a.length;
+  ctx.value_heads = a.value_heads;
+  ctx.base = base;
+  ctx.chunks = chunks;
+  ctx.slice = slice;
+  ctx.lane = lane;
+  ctx.hq = hq;
+  ctx.m = m;
+  ctx.seq = seq;
+  ctx.head = head;
   floatx4 s[8];  // rows 16t + 4hq + r, column 16*slice + m
 #pragma unroll
   for (int t = 0; t < 8; ++t)
 #pragma unroll
     for (int r = 0; r < 4; ++r)
       s[t][r] = state[(16 * t + 4 * hq + r) * DV + 16 * slice + m];
-
-  // Operands are fetched half an iteration ahead: the first-phase operands
-  // (U, -W, cQ) of chunk c+1 are requested before the second phase of chunk c
-  // runs, and the second-phase operands (A2, Kt) of chunk c before its first
-  // phase, so the dependent matrix-core chain does not wait on memory.
-  floatx4 u_reg[4];
-  uint4 w_reg[16], q_reg[16], a2_reg[8], kt_reg[16];
-  float decay = 1.0f;
-  const char* base = a.workspace + static_cast<size_t>(bh) * chunks * kGdnChunkBytes;
-  auto load_first = [&](int chunk) {
-    const char* in = base + static_cast<size_t>(chunk) * kGdnChunkBytes;
-    const floatx4* u_in = reinterpret_cast<const floatx4*>(in + kGdnOffsetU);
-    const uint4* neg_w = reinterpret_cast<const uint4*>(in + kGdnOffsetW);
-    const uint4* q_in = reinterpret_cast<const uint4*>(in + kGdnOffsetQ);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) u_reg[i] = u_in[(i * SLICES + slice) * 64 + lane];
-#pragma unroll
-    for (int f = 0; f < 16; ++f) {
-      w_reg[f] = neg_w[f * 64 + lane];
-      q_reg[f] = q_in[f * 64 + lane];
-    }
-  };
-  auto load_second = [&](int chunk) {
-    const char* in = base + static_cast<size_t>(chunk) * kGdnChunkBytes;
-    const uint4* a2_in = reinterpret_cast<const uint4*>(in + kGdnOffsetA2);
-    const uint4* kt_in = reinterpret_cast<const uint4*>(in + kGdnOffsetKt);
-#pragma unroll
-    for (int f = 0; f < 8; ++f) a2_reg[f] = a2_in[f * 64 + lane];
-#pragma unroll
-    for (int f = 0; f < 16; ++f) kt_reg[f] = kt_in[f * 64 + lane];
-    decay = *reinterpret_cast<const float*>(in + kGdnOffsetDecay);
-  };
-  load_first(0);
+  for (int chunk = 2; chunk < min(kScanAhead + 2, chunks); ++chunk)
+    scan_touch(descriptor, dump_address, static_cast<uint32_t>(chunk) * kGdnChunkBytes, slice, lane);
   for (int chunk = 0; chunk < chunks; ++chunk) {
-    load_second(chunk);
-    bf16x8 sb[4];
-#pragma unroll
-    for (int kb = 0; kb < 4; ++kb) sb[kb] = tiles_to_operand(s[2 * kb], s[2 * kb + 1]);
-    // D = U - W S0 and the S0 part of O = exp(c) Q S0 + (M o Q K^T) D
-    floatx4 d[4], o[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      floatx4 acc = u_reg[i];
-      floatx4 out_acc = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-      for (int kb = 0; kb < 4; ++kb) {
-        acc = mfma16(bits_to_bf16x8(w_reg[4 * i + kb]), sb[kb], acc);
-        out_acc = mfma16(bits_to_bf16x8(q_reg[4 * i + kb]), sb[kb], out_acc);
-      }
-      d[i] = acc;
-      o[i] = out_acc;
-    }
-    if (chunk + 1 < chunks) load_first(chunk + 1);
-    bf16x8 db[2];
-    db[0] = tiles_to_operand(d[0], d[1]);
-    db[1] = tiles_to_operand(d[2], d[3]);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      floatx4 acc = o[i];
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-        acc = mfma16(bits_to_bf16x8(a2_reg[2 * i + kb]), db[kb], acc);
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int token = chunk * C + 16 * i + 4 * hq + r;
-        if (token < a.length)
-          a.out[((static_cast<long long>(seq) * a.length + token) * a.value_heads + head) * DV +
-                16 * slice + m] = float_to_bf16_bits(acc[r]);
-      }
-    }
-    // S = exp(c_C) S0 + (diag(exp(c_C - c)) K)^T D
-#pragma unroll
-    for (int t = 0; t < 8; ++t) {
-      floatx4 acc = s[t] * decay;
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-        acc = mfma16(bits_to_bf16x8(kt_reg[2 * t + kb]), db[kb], acc);
-      s[t] = acc;
-    }
+    if (chunk + 2 + kScanAhead < chunks)
+      scan_touch(descriptor, dump_address,
+                 static_cast<uint32_t>(chunk + 2 + kScanAhead) * static_cast<uint32_t>(kGdnChunkBytes),
+                 slice, lane);
+    scan_barrier();  // landed
+    // passes the "free" barrier once all of the chunk it still needs is in registers
+    scan_step(ctx, descriptor, chunk, (chunk & 1) ? (lds_byte*)stage1 : (lds_byte*)stage0, s);
   }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
   for (int t = 0; t < 8; ++t)
 #pragma unroll
@@ -474,7 +711,7 @@ int launch_gdn_chunked(hipStream_t stream, const GdnArgs& a) {
   gdn_chunk_prepare<<<static_cast<unsigned>(heads * chunks), 256, 0, stream>>>(a);
   int status = launch_status();
   if (status != 0) return status;
-  gdn_chunk_scan<<<static_cast<unsigned>(heads * SLICES), 64, 0, stream>>>(a);
+  gdn_chunk_scan<<<static_cast<unsigned>(heads * (SLICES / kScanGroup)), kScanThreads, 0, stream>>>(a);
   return launch_status();
 }
 
