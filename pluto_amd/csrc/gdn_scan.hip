@@ -44,6 +44,35 @@ __device__ inline bf16x8 bits_to_bf16x8(uint4 v) { return __builtin_bit_cast(bf1
 // 32*kb + 16*(e/4) + 4*hq + e%4 (see file header of mfma_tile.h for the
 // 32x32 analogue).
 
+__device__ inline floatx4 mfma16(bf16x8 a, bf16x8 b, floatx4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+// Two stacked accumulator tiles as the B operand of a 32-deep product.
+__device__ inline bf16x8 tiles_to_operand(const floatx4& lo, const floatx4& hi) {
+  bf16x8 out;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    out[e] = static_cast<__bf16>(lo[e]);
+    out[4 + e] = static_cast<__bf16>(hi[e]);
+  }
+  return out;
+}
+
+// Two stacked accumulator tiles as a pair of B (or, read the other way, A)
+// operands whose sum carries about 16 mantissa bits: hi = bf16(v), lo =
+// bf16(v - hi).
+__device__ inline void split_operand(const floatx4& first, const floatx4& second, bf16x8& hi,
+                                     bf16x8& lo) {
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float v = e < 4 ? first[e] : second[e - 4];
+    const __bf16 h = static_cast<__bf16>(v);
+    hi[e] = h;
+    lo[e] = static_cast<__bf16>(v - static_cast<float>(h));
+  }
+}
+
 struct ChunkSmem {
   uint16_t k[C][DK + 8];    // raw K rows (bf16)
   uint16_t q[C][DK + 8];    // raw Q rows
@@ -165,53 +194,122 @@ gdn_chunk_prepare(GdnArgs a) {
   }
   __syncthreads();
 
-  // ---- forward substitution, one thread per column of [U | W] -------------
-  float x[C];
-  {
-    const bool is_u = tid < DV;
-    const int c = is_u ? tid : tid - DV;
-    const uint16_t* column = is_u ? &sm.vw[0][c] : &sm.k[0][c];  // same row stride
-    const float* factor = sm.rhs_factor[is_u ? 0 : 1];
+  // ---- (I + A) [U | W] = right-hand sides, by blocks of 16 rows on the matrix
+  // cores.  With T_b the inverse of diagonal block b of I + A,
+  //   X_b = T_b (R_b - sum_{k<b} A_bk X_k).
+  // Every factor enters as a sum of two bf16 numbers (value = hi + lo, products
+  // hi*hi + lo*hi + hi*lo), which keeps the result to about 2^-16 relative.
+  //
+  // T_b by forward substitution on the identity: wave b, lane = column; the
+  // result replaces the diagonal block of A, which nothing else reads.
+  if (lane < 16) {
+    const int base = 16 * wave;
+    float t[16];
 #pragma unroll
-    for (int i = 0; i < C; ++i) {
-      const float rhs = factor[i] * bf16_bits_to_float(column[i * (DK + 8)]);
-      // four partial sums shorten the dependent chain of a row
-      float acc0 = rhs, acc1 = 0.0f, acc2 = 0.0f, acc3 = 0.0f;
+    for (int i = 0; i < 16; ++i) {
+      float acc = (i == lane) ? 1.0f : 0.0f;
 #pragma unroll
       for (int j4 = 0; j4 < (i + 3) / 4; ++j4) {
-        const float4 row = *reinterpret_cast<const float4*>(&sm.a[i][4 * j4]);
-        // entries at or beyond the diagonal are zero
-        acc0 -= row.x * x[4 * j4];
-        if (4 * j4 + 1 < i) acc1 -= row.y * x[4 * j4 + 1];
-        if (4 * j4 + 2 < i) acc2 -= row.z * x[4 * j4 + 2];
-        if (4 * j4 + 3 < i) acc3 -= row.w * x[4 * j4 + 3];
+        const float4 row = *reinterpret_cast<const float4*>(&sm.a[base + i][base + 4 * j4]);
+        acc -= row.x * t[4 * j4];
+        if (4 * j4 + 1 < i) acc -= row.y * t[4 * j4 + 1];
+        if (4 * j4 + 2 < i) acc -= row.z * t[4 * j4 + 2];
+        if (4 * j4 + 3 < i) acc -= row.w * t[4 * j4 + 3];
       }
-      const float acc = (acc0 + acc1) + (acc2 + acc3);
-      // keep the scheduler from hoisting later rows' LDS reads over this row:
-      // that only lengthens live ranges until registers spill
-      asm volatile("" ::: "memory");
-      __builtin_amdgcn_sched_barrier(0);
-      x[i] = acc;
+      t[i] = acc;
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) sm.a[base + i][base + lane] = t[i];
+  }
+  __syncthreads();
+
+  // Wave w solves columns 64 (w % 2) .. +63 of U (w < 2) or of W, four column
+  // tiles of 16.  x[b][ct] is the 16x16 tile of block b in accumulator order:
+  // lane (hq, m) holds rows 16 b + 4 hq + r of column 16 ct + m.
+  floatx4 x[4][4];
+  const bool is_u = wave < 2;
+  const int col0 = 64 * (wave % 2);
+  {
+    const int hq = lane / 16, m = lane % 16;
+    const uint16_t(*source)[DK + 8] = is_u ? sm.vw : sm.k;  // same row stride
+    const float* factor = sm.rhs_factor[is_u ? 0 : 1];
+    const floatx4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+    bf16x8 pair_hi[4], pair_lo[4];  // blocks 0 and 1 stacked, as B operands
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      floatx4 r[4];
+#pragma unroll
+      for (int ct = 0; ct < 4; ++ct)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int row = 16 * b + 4 * hq + e;
+          r[ct][e] = factor[row] * bf16_bits_to_float(source[row][col0 + 16 * ct + m]);
+        }
+      // R_b -= [A_b,k0 | A_b,k1] [X_k0; X_k1]: contraction slot (hq, e) is row
+      // 4 hq + e % 4 of block k0 (e < 4) or k1
+#pragma unroll
+      for (int k0 = 0; k0 < b; k0 += 2) {
+        const bool both = k0 + 1 < b;
+        const float4 first = *reinterpret_cast<const float4*>(&sm.a[16 * b + m][16 * k0 + 4 * hq]);
+        float4 second = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if (both) second = *reinterpret_cast<const float4*>(&sm.a[16 * b + m][16 * k0 + 16 + 4 * hq]);
+        bf16x8 a_hi, a_lo;
+        split_operand(floatx4{-first.x, -first.y, -first.z, -first.w},
+                      floatx4{-second.x, -second.y, -second.z, -second.w}, a_hi, a_lo);
+#pragma unroll
+        for (int ct = 0; ct < 4; ++ct) {
+          bf16x8 b_hi, b_lo;
+          if (k0 == 0 && both) {
+            b_hi = pair_hi[ct];
+            b_lo = pair_lo[ct];
+          } else {
+            split_operand(x[k0][ct], zero, b_hi, b_lo);
+          }
+          r[ct] = mfma16(a_hi, b_hi, r[ct]);
+          r[ct] = mfma16(a_lo, b_hi, r[ct]);
+          r[ct] = mfma16(a_hi, b_lo, r[ct]);
+        }
+      }
+      // X_b = T_b R_b
+      const float4 t4 = *reinterpret_cast<const float4*>(&sm.a[16 * b + m][16 * b + 4 * hq]);
+      bf16x8 t_hi, t_lo;
+      split_operand(floatx4{t4.x, t4.y, t4.z, t4.w}, zero, t_hi, t_lo);
+#pragma unroll
+      for (int ct = 0; ct < 4; ++ct) {
+        bf16x8 r_hi, r_lo;
+        split_operand(r[ct], zero, r_hi, r_lo);
+        floatx4 acc = mfma16(t_hi, r_hi, zero);
+        acc = mfma16(t_lo, r_hi, acc);
+        x[b][ct] = mfma16(t_hi, r_lo, acc);
+      }
+      if (b == 1) {
+#pragma unroll
+        for (int ct = 0; ct < 4; ++ct) split_operand(x[0][ct], x[1][ct], pair_hi[ct], pair_lo[ct]);
+      }
     }
   }
   char* out = a.workspace + (static_cast<size_t>(bh) * chunks + chunk) * kGdnChunkBytes;
   float* u_out = reinterpret_cast<float*>(out + kGdnOffsetU);
   __syncthreads();  // everyone is done reading V before -W overwrites it
-  if (tid < DV) {
-    // U in accumulator order: [tile i][slice][lane = 16*hq + m][r]
-    const int slice = tid / 16, m = tid % 16;
+  if (is_u) {
+    // U in accumulator order: [block b][slice][lane = 16*hq + m][r], which is
+    // how the tiles sit in registers
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int b = 0; b < 4; ++b)
 #pragma unroll
-      for (int hq = 0; hq < 4; ++hq) {
-        const float4 value = make_float4(x[16 * i + 4 * hq], x[16 * i + 4 * hq + 1],
-                                         x[16 * i + 4 * hq + 2], x[16 * i + 4 * hq + 3]);
-        *reinterpret_cast<float4*>(u_out + ((i * SLICES + slice) * 64 + 16 * hq + m) * 4) = value;
+      for (int ct = 0; ct < 4; ++ct) {
+        const int slice = col0 / 16 + ct;
+        *reinterpret_cast<floatx4*>(u_out + ((b * SLICES + slice) * 64 + lane) * 4) = x[b][ct];
       }
   } else {
-    const int c = tid - DV;
+    const int hq = lane / 16, m = lane % 16;
 #pragma unroll
-    for (int i = 0; i < C; ++i) sm.vw[i][c] = float_to_bf16_bits(-x[i]);
+    for (int b = 0; b < 4; ++b)
+#pragma unroll
+      for (int ct = 0; ct < 4; ++ct)
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          sm.vw[16 * b + 4 * hq + e][col0 + 16 * ct + m] = float_to_bf16_bits(-x[b][ct][e]);
   }
   __syncthreads();
 
@@ -262,21 +360,6 @@ gdn_chunk_prepare(GdnArgs a) {
     kt_out[piece] = *reinterpret_cast<const uint4*>(packed);
   }
   if (tid == 0) *reinterpret_cast<float*>(out + kGdnOffsetDecay) = __expf(cum_last);
-}
-
-__device__ inline floatx4 mfma16(bf16x8 a, bf16x8 b, floatx4 c) {
-  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
-}
-
-// Two stacked accumulator tiles as the B operand of a 32-deep product.
-__device__ inline bf16x8 tiles_to_operand(const floatx4& lo, const floatx4& hi) {
-  bf16x8 out;
-#pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    out[e] = static_cast<__bf16>(lo[e]);
-    out[4 + e] = static_cast<__bf16>(hi[e]);
-  }
-  return out;
 }
 
 // LDS stage of the sequential kernel: the chunk's -W | cQ | A2 | Kt fragments
