@@ -10,7 +10,8 @@
 //
 //   scores  S^T[token, head] = K[token, :] . q[head, :] with
 //           v_mfma_f32_16x16x32_bf16: the A operand (16 tokens x 32 channels) is
-//           loaded straight from global memory, 64 contiguous bytes per lane;
+//           loaded straight from global memory, 16 bytes per lane, the four
+//           lanes of a token together one 64-byte sector per load;
 //           the group's heads are the (zero padded) 16 columns.
 //   values  O[head, :] += p[head, token] * V[token, :] on the vector ALU: 16
 //           bytes of V per lane, probabilities broadcast from LDS.  The kernel
@@ -43,11 +44,14 @@ template <int D, int GROUP>
 __global__ void __launch_bounds__(kThreads)
 decode_split_kernel(DecodeArgs a, DecodeBatch batch) {
   constexpr int KSTEPS = D / 32;
-  constexpr int QUARTER = D / 4;           // channels per lane quarter in phase 1
   constexpr int LANES_PER_ROW = D / 8;     // phase 2: 16-byte pieces per V row
   constexpr int ROWS_PER_PASS = 64 / LANES_PER_ROW;
-  __shared__ __attribute__((aligned(16))) float p_lds[kMaxSplit][8];
-  __shared__ __attribute__((aligned(16))) float o_lds[4][GROUP][D];
+  // The probabilities (phases 1-2) and the per-wave partial outputs (after
+  // phase 2) share one LDS area, so that eight workgroups fit a compute unit.
+  constexpr int kProbFloats = kMaxSplit * 8, kOutFloats = 4 * GROUP * D;
+  __shared__ __attribute__((aligned(16))) float shared_area[kProbFloats > kOutFloats ? kProbFloats : kOutFloats];
+  float (*p_lds)[8] = reinterpret_cast<float (*)[8]>(shared_area);
+  float (*o_lds)[GROUP][D] = reinterpret_cast<float (*)[GROUP][D]>(shared_area);
   __shared__ float wave_max[4][16];
   __shared__ float wave_sum_lds[4][16];
 
@@ -74,9 +78,23 @@ decode_split_kernel(DecodeArgs a, DecodeBatch batch) {
     if (n < GROUP)
       bits = *reinterpret_cast<const uint4*>(
           a.q + (static_cast<long long>(seq) * a.query_heads + g * GROUP + n) * D +
-          QUARTER * hq + 8 * ks);
+          32 * ks + 8 * hq);
     qf[ks] = __builtin_bit_cast(bf16x8, bits);
   }
+  // first batch of V rows for phase 2, requested now so that it travels while
+  // phase 1 computes (per_wave is a multiple of 16 rows, kBatch passes cover
+  // at most that)
+  constexpr int kBatch = 2;  // measured: 2 beats 1, 4, 8 and 16
+  const int sub = lane / LANES_PER_ROW, piece = lane % LANES_PER_ROW;
+  auto load_v = [&](int pass) {
+    const int token_local = wave * per_wave + pass * ROWS_PER_PASS + sub;
+    const int token = min(t0 + token_local, length - 1);
+    return *reinterpret_cast<const uint4*>(values + static_cast<long long>(token) * a.token_stride +
+                                           8 * piece);
+  };
+  uint4 v_next[kBatch];
+#pragma unroll
+  for (int i = 0; i < kBatch; ++i) v_next[i] = load_v(i);
   const int groups = per_wave / 16;  // 16-token groups per wave (<= 8)
   floatx4 s[kMaxSplit / 64];
   float local_max = kMasked;
@@ -86,11 +104,13 @@ decode_split_kernel(DecodeArgs a, DecodeBatch batch) {
       const int token_local = wave * per_wave + 16 * grp;
       int token = t0 + token_local + n;  // A operand row = lane % 16
       token = min(token, length - 1);    // stay inside the valid prefix
-      const uint16_t* row = keys + static_cast<long long>(token) * a.token_stride + QUARTER * hq;
+      // contraction step ks covers channels 32 ks .. 32 ks + 31: the four lanes
+      // of a token read one 64-byte sector per load
+      const uint16_t* row = keys + static_cast<long long>(token) * a.token_stride + 8 * hq;
       floatx4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
       for (int ks = 0; ks < KSTEPS; ++ks)
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(load_bf16x8(row + 8 * ks), qf[ks], acc,
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(load_bf16x8(row + 32 * ks), qf[ks], acc,
                                                       0, 0, 0);
       // accumulator register r = (token 4*hq + r of the group, head n)
 #pragma unroll
@@ -128,33 +148,43 @@ decode_split_kernel(DecodeArgs a, DecodeBatch batch) {
   __syncthreads();
 
   // ---- phase 2: O += p V ------------------------------------------------
-  const int sub = lane / LANES_PER_ROW, piece = lane % LANES_PER_ROW;
   float acc[GROUP][8];
 #pragma unroll
   for (int hh = 0; hh < GROUP; ++hh)
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[hh][e] = 0.0f;
   const int passes = per_wave / ROWS_PER_PASS;
-#pragma unroll 8
-  for (int pass = 0; pass < passes; ++pass) {
-    const int token_local = wave * per_wave + pass * ROWS_PER_PASS + sub;
-    const int token = min(t0 + token_local, length - 1);
-    const uint4 bits = *reinterpret_cast<const uint4*>(
-        values + static_cast<long long>(token) * a.token_stride + 8 * piece);
-    const float4 p0 = *reinterpret_cast<const float4*>(&p_lds[token_local][0]);
-    const float4 p1 = *reinterpret_cast<const float4*>(&p_lds[token_local][4]);
-    const float p[8] = {p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w};
-    const uint32_t w[4] = {bits.x, bits.y, bits.z, bits.w};
-    float v[8];
+  // V rows travel in batches of kBatch loads per lane; a batch is requested
+  // while the previous one is consumed (the first one before phase 1's
+  // barriers, see above).
+  for (int first = 0; first < passes; first += kBatch) {
+    uint4 now[kBatch];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      v[2 * i] = __uint_as_float(w[i] << 16);
-      v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    for (int i = 0; i < kBatch; ++i) now[i] = v_next[i];
+    if (first + kBatch < passes) {
+#pragma unroll
+      for (int i = 0; i < kBatch; ++i) v_next[i] = load_v(first + kBatch + i);
     }
 #pragma unroll
-    for (int hh = 0; hh < GROUP; ++hh)
+    for (int i = 0; i < kBatch; ++i) {
+      if (first + i >= passes) break;  // narrow heads with the smallest split
+      const int token_local = wave * per_wave + (first + i) * ROWS_PER_PASS + sub;
+      const uint4 bits = now[i];
+      const float4 p0 = *reinterpret_cast<const float4*>(&p_lds[token_local][0]);
+      const float4 p1 = *reinterpret_cast<const float4*>(&p_lds[token_local][4]);
+      const float p[8] = {p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w};
+      const uint32_t w[4] = {bits.x, bits.y, bits.z, bits.w};
+      float v[8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc[hh][e] += p[hh] * v[e];
+      for (int j = 0; j < 4; ++j) {
+        v[2 * j] = __uint_as_float(w[j] << 16);
+        v[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+      }
+#pragma unroll
+      for (int hh = 0; hh < GROUP; ++hh)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[hh][e] += p[hh] * v[e];
+    }
   }
 #pragma unroll
   for (int hh = 0; hh < GROUP; ++hh)
@@ -166,6 +196,7 @@ decode_split_kernel(DecodeArgs a, DecodeBatch batch) {
         x += __shfl_xor(x, offset, 64);
       acc[hh][e] = x;
     }
+  __syncthreads();  // every wave is done with the probabilities
   if (sub == 0) {
 #pragma unroll
     for (int hh = 0; hh < GROUP; ++hh) {
