@@ -198,6 +198,34 @@ int pluto_hip_gqa_prefill(void* stream, const pluto_hip_attention_params* p,
                           const pluto_hip_kv_cache_view* cache, void* out,
                           float* lse, void* workspace, size_t workspace_bytes);
 
+/* Backward of the whole-sequence layer
+ * (QwenAttentionLayer::SequenceBackward, qwen_attention.cc:450-499; kernels
+ * GateBackward :124-141, QueryBackward :146-174, KeyValueBackward :179-199,
+ * NormBackward :201-228, ReduceNorm :230-239).  Self-contained: it takes the
+ * layer's inputs and recomputes what the forward pass derived from them, so
+ * nothing quadratic (the reference saves probabilities and score gradients,
+ * [qh, length, length] each) is kept between the passes.
+ *   dy       fp32 [length, qh, d]     gradient of the layer output
+ *   dqg      fp32 [length, qh, 2, d]  query gradients at [..,0,:], gate at [..,1,:]
+ *   dk, dv   fp32 [length, kh, d]
+ *   dq_norm, dk_norm  optional fp32 [d]: the norm weights' gradients are ADDED
+ *            to them (shared weights accumulate over calls, as in the
+ *            reference); NULL skips that work.
+ * Rounding points are treated as identities, with the rounded forward values
+ * as operands where the reference uses them.  With round_to_bfloat16 set and
+ * head_dim 64 or 128 the attention part runs on the matrix cores with bf16
+ * operands; all other cases run FP32 kernels. */
+size_t pluto_hip_gqa_prefill_backward_workspace_bytes(const pluto_hip_attention_params* p,
+                                                      int length, int q_weight_grad,
+                                                      int k_weight_grad);
+int pluto_hip_gqa_prefill_backward(void* stream, const pluto_hip_attention_params* p,
+                                   int length, const void* qg, const void* k,
+                                   const void* v, const float* q_norm,
+                                   const float* k_norm, const float* dy, float* dqg,
+                                   float* dk, float* dv, float* dq_norm,
+                                   float* dk_norm, void* workspace,
+                                   size_t workspace_bytes);
+
 /* The FP32 probabilities tensor of the same ForwardKernel
  * (qwen_attention.cc:68-119, reported to attention_probabilities_hook at
  * :441-444), produced on request by a separate two-pass kernel:

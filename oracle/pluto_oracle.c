@@ -382,6 +382,152 @@ int pluto_oracle_gqa_sequence(const pluto_oracle_attention_params* p,
   return 0;
 }
 
+/* Backward of the whole-sequence layer: the five kernels of
+ * qwen_attention.cc:124-239 as launched by SequenceBackward (:450-499), in
+ * double precision.  Rounding points have derivative one; the operands are the
+ * values the reference's kernels use: dC = dy * Round(sigmoid) and
+ * d gate = dy * Round(core) * s(1-s) (:136-140); delta = dC . core with the
+ * unrounded core (:160-161); dS = P (dC . V - delta) (:168); dQ = sum dS K
+ * scale (:170); dK = sum dS Q scale, dV = sum P dC over the later rows of the
+ * kv head's query heads (:189-196); RoPE transposed with the rounded cos/sin
+ * and RMSNorm backward (:213-227); weight gradients are added to dq_norm /
+ * dk_norm (:230-239). */
+static void norm_rope_backward(const pluto_oracle_attention_params* p, int row,
+                               const float* input, const float* weight,
+                               const double* grad, double* dx, double* dw) {
+  const int d = p->head_dim, rotary = p->rotary_dim, half = rotary / 2;
+  double normalized[256];
+  for (int c = 0; c < d; ++c) {
+    double ng = grad[c];
+    if (c < rotary) {
+      const int frequency = c < half ? c : c - half;
+      const double angle = row * pow(p->rope_theta, -2.0 * frequency / rotary);
+      const double co = round_if(p, (float)cos(angle));
+      const double si = round_if(p, (float)sin(angle));
+      const double partner = grad[c < half ? c + half : c - half];
+      ng = grad[c] * co + (c < half ? partner * si : -partner * si);
+    }
+    normalized[c] = ng;
+  }
+  double square = 0.0;
+  for (int c = 0; c < d; ++c) square += (double)input[c] * input[c];
+  const double inv = 1.0 / sqrt(square / d + p->rms_norm_epsilon);
+  double dot = 0.0;
+  for (int c = 0; c < d; ++c) dot += normalized[c] * (1.0 + weight[c]) * input[c];
+  for (int c = 0; c < d; ++c) {
+    dx[c] = inv * normalized[c] * (1.0 + weight[c]) -
+            input[c] * (inv * inv * inv / d) * dot;
+    if (dw) dw[c] += normalized[c] * input[c] * inv;
+  }
+}
+
+int pluto_oracle_gqa_sequence_backward(const pluto_oracle_attention_params* p,
+                                       int length, const float* qg, const float* k,
+                                       const float* v, const float* q_norm,
+                                       const float* k_norm, const float* dy,
+                                       float* dqg, float* dk, float* dv,
+                                       float* dq_norm, float* dk_norm) {
+  if (!attention_params_ok(p) || length <= 0) return -1;
+  const int d = p->head_dim, qh = p->query_heads, kh = p->key_value_heads;
+  const int group = qh / kh;
+  const size_t qn = (size_t)length * qh * d, kn = (size_t)length * kh * d;
+  const double scale = 1.0 / sqrt((double)d);
+  float* queries = (float*)malloc(sizeof(float) * qn);
+  float* keys = (float*)malloc(sizeof(float) * kn);
+  float* values = (float*)malloc(sizeof(float) * kn);
+  double* dq_rope = (double*)calloc(qn, sizeof(double));
+  double* dk_rope = (double*)calloc(kn, sizeof(double));
+  double* dv_sum = (double*)calloc(kn, sizeof(double));
+  double* prob = (double*)malloc(sizeof(double) * (size_t)length);
+  double* dq_weight = (double*)calloc((size_t)d, sizeof(double));
+  double* dk_weight = (double*)calloc((size_t)d, sizeof(double));
+  if (!queries || !keys || !values || !dq_rope || !dk_rope || !dv_sum || !prob ||
+      !dq_weight || !dk_weight) {
+    free(queries); free(keys); free(values); free(dq_rope); free(dk_rope);
+    free(dv_sum); free(prob); free(dq_weight); free(dk_weight);
+    return -1;
+  }
+  for (int t = 0; t < length; ++t) {
+    for (int h = 0; h < kh; ++h) {
+      const size_t at = ((size_t)t * kh + h) * d;
+      pluto_oracle_gqa_normalize_rotate(p, t, k + at, k_norm, keys + at);
+      for (int c = 0; c < d; ++c) values[at + c] = round_if(p, v[at + c]);
+    }
+    for (int h = 0; h < qh; ++h)
+      pluto_oracle_gqa_normalize_rotate(p, t, qg + ((size_t)t * qh + h) * 2 * d, q_norm,
+                                        queries + ((size_t)t * qh + h) * d);
+  }
+  for (int row = 0; row < length; ++row)
+    for (int h = 0; h < qh; ++h) {
+      const int kv = h / group;
+      const float* query = queries + ((size_t)row * qh + h) * d;
+      double maximum = -INFINITY;
+      for (int t = 0; t <= row; ++t) {
+        double score = 0.0;
+        const float* key = keys + ((size_t)t * kh + kv) * d;
+        for (int c = 0; c < d; ++c) score += (double)query[c] * key[c];
+        prob[t] = score * scale;
+        if (prob[t] > maximum) maximum = prob[t];
+      }
+      double normalizer = 0.0;
+      for (int t = 0; t <= row; ++t) {
+        prob[t] = exp(prob[t] - maximum);
+        normalizer += prob[t];
+      }
+      for (int t = 0; t <= row; ++t) prob[t] /= normalizer;
+      double dc[256];
+      double delta = 0.0;
+      for (int c = 0; c < d; ++c) {
+        double sum = 0.0;
+        for (int t = 0; t <= row; ++t) sum += prob[t] * values[((size_t)t * kh + kv) * d + c];
+        const size_t at = ((size_t)row * qh + h) * d + c;
+        const double gate = qg[(((size_t)row * qh + h) * 2 + 1) * d + c];
+        const double sigmoid = 1.0 / (1.0 + exp(-gate));
+        const double grad = dy[at];
+        dc[c] = grad * round_if(p, (float)sigmoid);
+        dqg[(((size_t)row * qh + h) * 2 + 1) * d + c] =
+            (float)(grad * round_if(p, (float)sum) * sigmoid * (1.0 - sigmoid));
+        delta += dc[c] * sum;
+      }
+      for (int t = 0; t <= row; ++t) {
+        const size_t kv_at = ((size_t)t * kh + kv) * d;
+        double dp = 0.0;
+        for (int c = 0; c < d; ++c) dp += dc[c] * values[kv_at + c];
+        const double ds = prob[t] * (dp - delta);
+        for (int c = 0; c < d; ++c) {
+          dq_rope[((size_t)row * qh + h) * d + c] += ds * keys[kv_at + c] * scale;
+          dk_rope[kv_at + c] += ds * query[c] * scale;
+          dv_sum[kv_at + c] += prob[t] * dc[c];
+        }
+      }
+    }
+  double dx[256];
+  for (int row = 0; row < length; ++row) {
+    for (int h = 0; h < qh; ++h) {
+      const size_t unit = (size_t)row * qh + h;
+      norm_rope_backward(p, row, qg + unit * 2 * d, q_norm, dq_rope + unit * d, dx,
+                         dq_norm ? dq_weight : NULL);
+      for (int c = 0; c < d; ++c) dqg[unit * 2 * d + c] = (float)dx[c];
+    }
+    for (int h = 0; h < kh; ++h) {
+      const size_t unit = (size_t)row * kh + h;
+      norm_rope_backward(p, row, k + unit * d, k_norm, dk_rope + unit * d, dx,
+                         dk_norm ? dk_weight : NULL);
+      for (int c = 0; c < d; ++c) {
+        dk[unit * d + c] = (float)dx[c];
+        dv[unit * d + c] = (float)dv_sum[unit * d + c];
+      }
+    }
+  }
+  for (int c = 0; c < d; ++c) {
+    if (dq_norm) dq_norm[c] += (float)dq_weight[c];
+    if (dk_norm) dk_norm[c] += (float)dk_weight[c];
+  }
+  free(queries); free(keys); free(values); free(dq_rope); free(dk_rope);
+  free(dv_sum); free(prob); free(dq_weight); free(dk_weight);
+  return 0;
+}
+
 int pluto_oracle_gqa_attend(const pluto_oracle_attention_params* p, int length,
                             size_t head_stride, const float* q,
                             const float* gate, const float* keys,

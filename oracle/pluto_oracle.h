@@ -118,6 +118,18 @@ int pluto_oracle_gqa_sequence(const pluto_oracle_attention_params* p,
                               float* value_out, float* lse, int row_begin,
                               int row_end, int head_begin, int head_end);
 
+/* Gradients of pluto_oracle_gqa_sequence with respect to qg, k, v and the two
+ * norm weights for an upstream gradient dy [T, qh, d]
+ * (QwenAttentionLayer::SequenceBackward, qwen_attention.cc:450-499).  dqg
+ * [T, qh, 2, d], dk, dv [T, kh, d] are overwritten; dq_norm, dk_norm (nullable,
+ * [d]) are added to. */
+int pluto_oracle_gqa_sequence_backward(const pluto_oracle_attention_params* p,
+                                       int length, const float* qg, const float* k,
+                                       const float* v, const float* q_norm,
+                                       const float* k_norm, const float* dy,
+                                       float* dqg, float* dk, float* dv,
+                                       float* dq_norm, float* dk_norm);
+
 /* Attention of prepared queries against an existing cache, used for the
  * batched decode configuration: q is [qh, d] already normalised and rotated,
  * gate is [qh, d] raw logits, keys/values are [kh, length, d] head-major FP32

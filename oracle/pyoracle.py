@@ -217,6 +217,27 @@ def gqa_sequence(p, qg, k, v, q_norm, k_norm, rows=None, heads=None):
     return dict(out=out, keys=keys, values=values, lse=lse)
 
 
+def gqa_sequence_backward(p, qg, k, v, q_norm, k_norm, dy, weight_grads=True):
+    """Gradients of gqa_sequence for the upstream gradient dy [T, qh, d].
+    Returns dict(dqg [T, qh, 2, d], dk, dv [T, kh, d], dq_norm, dk_norm [d])."""
+    qg, k, v, dy = _f32(qg), _f32(k), _f32(v), _f32(dy)
+    q_norm, k_norm = _f32(q_norm), _f32(k_norm)
+    T = qg.shape[0]
+    dqg = np.zeros((T, p.query_heads, 2, p.head_dim), np.float32)
+    dk = np.zeros((T, p.key_value_heads, p.head_dim), np.float32)
+    dv = np.zeros_like(dk)
+    dq_norm = np.zeros(p.head_dim, np.float32)
+    dk_norm = np.zeros(p.head_dim, np.float32)
+    fn = lib().pluto_oracle_gqa_sequence_backward
+    fn.restype = ctypes.c_int
+    rc = fn(ctypes.byref(p), T, _ptr(qg), _ptr(k), _ptr(v), _ptr(q_norm), _ptr(k_norm),
+            _ptr(dy), _ptr(dqg), _ptr(dk), _ptr(dv),
+            _ptr(dq_norm) if weight_grads else None, _ptr(dk_norm) if weight_grads else None)
+    if rc != 0:
+        raise ValueError("oracle rejected the GQA sequence backward")
+    return dict(dqg=dqg, dk=dk, dv=dv, dq_norm=dq_norm, dk_norm=dk_norm)
+
+
 def gqa_attend(p, q, gate, keys, values):
     """q, gate [qh, d]; keys/values [kh, L, d] head-major float32."""
     q, gate = _f32(q), _f32(gate)

@@ -96,6 +96,10 @@ SIGNATURES = {
                                    _VP, _VP, _VP, _SZ]),
     "pluto_hip_gqa_prefill_probabilities": (_I, [_VP, ctypes.POINTER(AttentionParams), _I, _I,
                                                  ctypes.POINTER(KvCacheView), _VP, _SZ, _VP]),
+    "pluto_hip_gqa_prefill_backward_workspace_bytes": (_SZ, [ctypes.POINTER(AttentionParams), _I,
+                                                             _I, _I]),
+    "pluto_hip_gqa_prefill_backward": (_I, [_VP, ctypes.POINTER(AttentionParams), _I] +
+                                       [_VP] * 11 + [_VP, _SZ]),
     "pluto_hip_gqa_decode_workspace_bytes": (_SZ, [ctypes.POINTER(AttentionParams), _I,
                                                    ctypes.POINTER(_I), _I]),
     "pluto_hip_gqa_decode": (_I, [_VP, ctypes.POINTER(AttentionParams), _I, _I, _VP,
@@ -275,6 +279,25 @@ def gqa_prefill(p, qg, k, v, q_norm, k_norm, cache, start_position=0, want_lse=F
             ptr(workspace), size, ptr(probabilities)))
         result = (result + (probabilities,)) if want_lse else (result, probabilities)
     return result
+
+
+def gqa_prefill_backward(p, qg, k, v, q_norm, k_norm, dy, dq_norm=None, dk_norm=None,
+                         stream=None):
+    """Gradients of the whole-sequence layer: (dqg fp32 [T, qh, 2, d], dk, dv fp32 [T, kh, d]).
+
+    dq_norm / dk_norm: optional fp32 [d] accumulators the norm-weight gradients are added to."""
+    T = qg.shape[0]
+    dqg = torch.empty((T, p.query_heads, 2, p.head_dim), dtype=torch.float32, device=qg.device)
+    dk = torch.empty((T, p.key_value_heads, p.head_dim), dtype=torch.float32, device=qg.device)
+    dv = torch.empty_like(dk)
+    size = lib().pluto_hip_gqa_prefill_backward_workspace_bytes(
+        ctypes.byref(p), T, int(dq_norm is not None), int(dk_norm is not None))
+    workspace = torch.empty(max(size, 1), dtype=torch.uint8, device=qg.device)
+    check(lib().pluto_hip_gqa_prefill_backward(
+        stream or current_stream(), ctypes.byref(p), T, ptr(qg), ptr(k), ptr(v), ptr(q_norm),
+        ptr(k_norm), ptr(dy), ptr(dqg), ptr(dk), ptr(dv), ptr(dq_norm), ptr(dk_norm),
+        ptr(workspace), size))
+    return dqg, dk, dv
 
 
 def gqa_decode_workspace(p, positions, split_tokens=0, device="cuda"):

@@ -106,4 +106,19 @@ int launch_attention_probabilities(hipStream_t stream, const void* q, int q_dtyp
                                    int first_visible, int row_width, float scale,
                                    float* probabilities);
 
+// Pieces of the whole-sequence backward (gqa_backward.hip).
+int launch_pack_heads(hipStream_t stream, const void* q, const void* k, const void* v, int dtype,
+                      int length, int query_heads, int key_value_heads, int head_dim,
+                      void* packed);
+int launch_gate_backward(hipStream_t stream, const void* qg, const void* core, int core_dtype,
+                         const float* dy, int length, int query_heads, int head_dim, bool round,
+                         float* dc, float* dqg);
+int launch_norm_rope_backward(hipStream_t stream, const void* input, const float* weight,
+                              const float* packed_grad, const float* cosines, const float* sines,
+                              int length, int heads, int query_heads, int head_dim, int rotary_dim,
+                              int input_stride, float epsilon, bool key_mode, float* dx,
+                              float* dv, float* parts);
+int launch_reduce_norm(hipStream_t stream, const float* parts, long long rows, int head_dim,
+                       float* partial, int chunks, float* dw);
+
 }  // namespace pluto_hip

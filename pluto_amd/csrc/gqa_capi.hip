@@ -55,6 +55,52 @@ PrefillLayout prefill_layout(const pluto_hip_attention_params* p, int length) {
   return l;
 }
 
+// Scratch of the whole-sequence backward.
+struct PrefillBackwardLayout {
+  size_t cosines, sines, queries, keys, values, packed, core, maxima, normalizers, dc, d_packed,
+      q_parts, k_parts, partial, attention, total;
+  size_t attention_bytes;
+  int dtype;  // storage of the packed view and of the recomputed core
+};
+constexpr int kNormReduceChunks = 128;
+
+PrefillBackwardLayout prefill_backward_layout(const pluto_hip_attention_params* p, int length,
+                                              bool q_weight_grad, bool k_weight_grad) {
+  PrefillBackwardLayout l{};
+  const size_t T = static_cast<size_t>(length);
+  const size_t qh = p->query_heads, kh = p->key_value_heads, d = p->head_dim;
+  // bf16 storage (matrix-core kernels, bf16 tolerance) where those kernels
+  // exist; everything else runs the FP32 kernels on FP32 storage.
+  const bool flash = p->round_to_bfloat16 && (d == 64 || d == 128) && !force_generic();
+  l.dtype = flash ? PLUTO_HIP_BF16 : PLUTO_HIP_F32;
+  const size_t element = flash ? 2 : 4;
+  size_t at = 0;
+  auto take = [&](size_t bytes) {
+    const size_t offset = at;
+    at += align_up(bytes, 256);
+    return offset;
+  };
+  l.cosines = take(T * (p->rotary_dim / 2) * 4);
+  l.sines = take(T * (p->rotary_dim / 2) * 4);
+  l.queries = take(T * qh * d * element);
+  l.keys = take(T * kh * d * element);
+  l.values = take(T * kh * d * element);
+  l.packed = take(3 * T * qh * d * element);
+  l.core = take(T * qh * d * element);
+  l.maxima = take(T * qh * 4);
+  l.normalizers = take(T * qh * 4);
+  l.dc = take(T * qh * d * 4);
+  l.d_packed = take(3 * T * qh * d * 4);
+  l.q_parts = take(q_weight_grad ? T * qh * d * 4 : 0);
+  l.k_parts = take(k_weight_grad ? T * kh * d * 4 : 0);
+  l.partial = take((q_weight_grad || k_weight_grad) ? kNormReduceChunks * d * 4 : 0);
+  l.attention_bytes = pluto_hip_mha_backward_workspace_bytes(
+      l.dtype, length, length, p->query_heads, p->query_heads * p->head_dim);
+  l.attention = take(l.attention_bytes);
+  l.total = at;
+  return l;
+}
+
 int split_or_default(int split_tokens) { return split_tokens == 0 ? 512 : split_tokens; }
 
 long long decode_blocks(int batch, const int* positions, int split) {
@@ -173,6 +219,101 @@ int pluto_hip_gqa_prefill(void* stream, const pluto_hip_attention_params* p, int
   a.scale = scale;
   a.round_to_bf16 = round;
   return launch_generic_forward(s, a, 1);
+}
+
+size_t pluto_hip_gqa_prefill_backward_workspace_bytes(const pluto_hip_attention_params* p,
+                                                      int length, int q_weight_grad,
+                                                      int k_weight_grad) {
+  if (validate_params(p) != 0 || length <= 0) return 0;
+  return prefill_backward_layout(p, length, q_weight_grad != 0, k_weight_grad != 0).total;
+}
+
+int pluto_hip_gqa_prefill_backward(void* stream, const pluto_hip_attention_params* p, int length,
+                                   const void* qg, const void* k, const void* v,
+                                   const float* q_norm, const float* k_norm, const float* dy,
+                                   float* dqg, float* dk, float* dv, float* dq_norm,
+                                   float* dk_norm, void* workspace, size_t workspace_bytes) {
+  int status = validate_params(p);
+  if (status != 0) return status;
+  if (length <= 0) return PLUTO_HIP_EINVAL;
+  if (!qg || !k || !v || !q_norm || !k_norm || !dy || !dqg || !dk || !dv) return PLUTO_HIP_EINVAL;
+  const PrefillBackwardLayout l = prefill_backward_layout(p, length, dq_norm != nullptr,
+                                                          dk_norm != nullptr);
+  if (l.attention_bytes == 0) return PLUTO_HIP_EINVAL;
+  if (!workspace || workspace_bytes < l.total) return PLUTO_HIP_EWORKSPACE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  char* scratch = static_cast<char*>(workspace);
+  float* cosines = reinterpret_cast<float*>(scratch + l.cosines);
+  float* sines = reinterpret_cast<float*>(scratch + l.sines);
+  const bool round = p->round_to_bfloat16 != 0;
+  const int qh = p->query_heads, kh = p->key_value_heads, d = p->head_dim;
+  const int E = qh * d;
+
+  // Recompute what the forward pass derived from the inputs: normalised,
+  // rotated q and k (PrepareKernel, qwen_attention.cc:30-63), then the
+  // attention core with its row statistics.
+  status = launch_rope_table(s, 0, length, p->rotary_dim, p->rope_theta, round, cosines, sines);
+  if (status != 0) return status;
+  PrefillPrepareArgs prep;
+  prep.qg = qg;
+  prep.k = k;
+  prep.v = v;
+  prep.q_norm = q_norm;
+  prep.k_norm = k_norm;
+  prep.cosines = cosines;
+  prep.sines = sines;
+  prep.q_out = scratch + l.queries;
+  prep.q_out_dtype = l.dtype;
+  prep.cache = {scratch + l.keys, scratch + l.values, l.dtype, 1LL * kh * d, d};
+  prep.length = length;
+  prep.start_position = 0;
+  prep.query_heads = qh;
+  prep.key_value_heads = kh;
+  prep.head_dim = d;
+  prep.rotary_dim = p->rotary_dim;
+  prep.epsilon = p->rms_norm_epsilon;
+  prep.round = round;
+  status = launch_prefill_prepare(s, prep);
+  if (status != 0) return status;
+  status = launch_pack_heads(s, scratch + l.queries, scratch + l.keys, scratch + l.values, l.dtype,
+                             length, qh, kh, d, scratch + l.packed);
+  if (status != 0) return status;
+  float* maxima = reinterpret_cast<float*>(scratch + l.maxima);
+  float* normalizers = reinterpret_cast<float*>(scratch + l.normalizers);
+  status = pluto_hip_mha_forward(stream, l.dtype, scratch + l.packed, length, length, qh, E,
+                                 scratch + l.core, maxima, normalizers);
+  if (status != 0) return status;
+
+  float* dc = reinterpret_cast<float*>(scratch + l.dc);
+  status = launch_gate_backward(s, qg, scratch + l.core, l.dtype, dy, length, qh, d, round, dc, dqg);
+  if (status != 0) return status;
+  float* d_packed = reinterpret_cast<float*>(scratch + l.d_packed);
+  status = pluto_hip_mha_backward(stream, l.dtype, scratch + l.packed, scratch + l.core, dc, maxima,
+                                  normalizers, length, length, qh, E, d_packed,
+                                  scratch + l.attention, l.attention_bytes);
+  if (status != 0) return status;
+
+  float* q_parts = dq_norm ? reinterpret_cast<float*>(scratch + l.q_parts) : nullptr;
+  float* k_parts = dk_norm ? reinterpret_cast<float*>(scratch + l.k_parts) : nullptr;
+  status = launch_norm_rope_backward(s, qg, q_norm, d_packed, cosines, sines, length, qh, qh, d,
+                                     p->rotary_dim, 2 * d, p->rms_norm_epsilon, false, dqg, nullptr,
+                                     q_parts);
+  if (status != 0) return status;
+  status = launch_norm_rope_backward(s, k, k_norm, d_packed, cosines, sines, length, kh, qh, d,
+                                     p->rotary_dim, d, p->rms_norm_epsilon, true, dk, dv, k_parts);
+  if (status != 0) return status;
+  float* partial = reinterpret_cast<float*>(scratch + l.partial);
+  if (dq_norm) {
+    status = launch_reduce_norm(s, q_parts, 1LL * length * qh, d, partial, kNormReduceChunks,
+                                dq_norm);
+    if (status != 0) return status;
+  }
+  if (dk_norm) {
+    status = launch_reduce_norm(s, k_parts, 1LL * length * kh, d, partial, kNormReduceChunks,
+                                dk_norm);
+    if (status != 0) return status;
+  }
+  return 0;
 }
 
 int pluto_hip_gqa_prefill_probabilities(void* stream, const pluto_hip_attention_params* p,
