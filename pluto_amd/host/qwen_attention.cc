@@ -82,15 +82,13 @@ StatusOr<FwdResult> QwenAttentionLayer::fwd_impl(hip::Executor& executor,
   return SequenceForward(executor, inputs, hooks);
 }
 
-// src/llm/layers/qwen_attention.cc:362-369.  The reference differentiates the
-// sequence path (SequenceBackward, :450-545); that kernel chain is not part of
-// this library.
-StatusOr<BufferVec> QwenAttentionLayer::bwd_impl(hip::Executor&, Span<const Buffer>,
-                                                 BackwardState, LayerHooks*) {
+// src/llm/layers/qwen_attention.cc:362-369
+StatusOr<BufferVec> QwenAttentionLayer::bwd_impl(hip::Executor& executor,
+                                                 Span<const Buffer> gradients,
+                                                 BackwardState state, LayerHooks*) {
   if (cache_)
     return UnimplementedError("QwenAttentionLayer with a KV cache supports inference only");
-  return UnimplementedError(
-      "QwenAttentionLayer sequence backward is not implemented by the MI355X attention path");
+  return SequenceBackward(executor, gradients, std::move(state));
 }
 
 // src/llm/layers/qwen_attention.cc:371-412.  The decode kernels read and write
@@ -197,6 +195,44 @@ StatusOr<FwdResult> QwenAttentionLayer::SequenceForward(hip::Executor& executor,
   state.intermediates = {inputs[0], inputs[1], inputs[2], std::move(keys), std::move(values),
                          std::move(lse)};
   return FwdResult{{std::move(output)}, std::move(state)};
+}
+
+// src/llm/layers/qwen_attention.cc:450-499.  The library's backward entry is
+// self-contained (it recomputes what the forward pass derived from the
+// inputs), so only the three input handles of the saved state are used.
+StatusOr<BufferVec> QwenAttentionLayer::SequenceBackward(hip::Executor& executor,
+                                                         Span<const Buffer> gradients,
+                                                         BackwardState state) {
+  if (&executor != &executor_ || state.intermediates.size() != 6)
+    return InvalidArgumentError("sequence attention backward Executor/state mismatch");
+  const auto& p = parameters_;
+  const int t = sequence_length_, d = p.head_dim, qh = p.query_heads, kh = p.key_value_heads;
+  const size_t qn = static_cast<size_t>(t) * qh * d, kn = static_cast<size_t>(t) * kh * d;
+  if (gradients.size() != 1 || &gradients[0].executor() != &executor ||
+      gradients[0].size_bytes() != 4 * qn)
+    return InvalidArgumentError("sequence attention expects batch-one buffers on its Executor");
+  const auto& s = state.intermediates;
+  pluto_hip_attention_params abi = cached_attention_ops::ToAbi(p);
+  abi.capacity = t;
+  ASSIGN_OR_RETURN(auto dqg, Buffer::Allocate(executor, 2 * qn * sizeof(float)));
+  ASSIGN_OR_RETURN(auto dk, Buffer::Allocate(executor, kn * sizeof(float)));
+  ASSIGN_OR_RETURN(auto dv, Buffer::Allocate(executor, kn * sizeof(float)));
+  const bool q_active = q_norm_->active(), k_active = k_norm_->active();
+  const size_t workspace_bytes =
+      pluto_hip_gqa_prefill_backward_workspace_bytes(&abi, t, q_active, k_active);
+  ASSIGN_OR_RETURN(auto workspace, Buffer::Allocate(executor, workspace_bytes));
+  RETURN_IF_ERROR(hip::HipStatus(
+      pluto_hip_gqa_prefill_backward(
+          executor.stream(), &abi, t, s[0].data(), s[1].data(), s[2].data(),
+          static_cast<const float*>(weights_[0].data()),
+          static_cast<const float*>(weights_[1].data()),
+          static_cast<const float*>(gradients[0].data()), static_cast<float*>(dqg.data()),
+          static_cast<float*>(dk.data()), static_cast<float*>(dv.data()),
+          q_active ? static_cast<float*>(q_norm_->gradient().data()) : nullptr,
+          k_active ? static_cast<float*>(k_norm_->gradient().data()) : nullptr, workspace.data(),
+          workspace_bytes),
+      "sequence full attention backward"));
+  return BufferVec{std::move(dqg), std::move(dk), std::move(dv)};
 }
 
 }  // namespace pluto::llm

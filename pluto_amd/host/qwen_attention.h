@@ -69,6 +69,11 @@ class QwenAttentionLayer final : public Layer {
   StatusOr<FwdResult> SequenceForward(hip::Executor& executor, Span<const Buffer> inputs,
                                       LayerHooks* hooks) const;
 
+  // Returns FP32 Q/gate, K and V gradients; accumulates norm gradients only
+  // into parameters that are active.
+  StatusOr<BufferVec> SequenceBackward(hip::Executor& executor, Span<const Buffer> gradients,
+                                       BackwardState state);
+
   hip::Executor& executor_;
   FullAttentionParameters parameters_;
   std::shared_ptr<BlockParameter> q_norm_, k_norm_;

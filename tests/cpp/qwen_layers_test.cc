@@ -368,9 +368,126 @@ TEST(QwenAttentionTest, CachePointerSelectsBackwardContractAtLengthOne) {
   EXPECT_TRUE(Read<BFloat16>(sf->outputs[0]) == Read<BFloat16>(cf->outputs[0]));
   EXPECT_EQ((*cache)->position(), 1);
   EXPECT_TRUE(IsUnimplemented((*cached)->bwd(*executor, {*dy}, std::move(cf->state)).status()));
-  // the sequence path's backward is not part of this library either
-  EXPECT_TRUE(IsUnimplemented((*sequence)->bwd(*executor, {*dy}, std::move(sf->state)).status()));
+  // qwen_attention_test.cc:394-405: the sequence contract differentiates
+  auto backward = (*sequence)->bwd(*executor, {*dy}, std::move(sf->state));
+  ASSERT_TRUE(backward.ok());
+  ASSERT_EQ(backward->size(), 3u);
+  float value_magnitude = 0;
+  for (float gradient : Read<float>((*backward)[2])) {
+    EXPECT_TRUE(std::isfinite(gradient));
+    value_magnitude += std::fabs(gradient);
+  }
+  EXPECT_GT(value_magnitude, 1e-5f);
   EXPECT_EQ((*cache)->position(), 1);
+}
+
+TEST(QwenAttentionTest, FullBackwardMatchesTheOracleAndAccumulatesNormGradients) {
+  // qwen_attention_test.cc:230-300.  The oracle's backward is itself checked
+  // against finite differences of a frozen-rounding forward; here the layer is
+  // checked against the oracle, with the reference's bound of 3e-5.
+  for (bool use_bf16_rounding : {false, true}) {
+    auto executor = NewExecutor();
+    FullAttentionParameters p;
+    p.query_heads = 2;
+    p.key_value_heads = 1;
+    p.head_dim = 3;
+    p.rotary_dim = 2;
+    p.round_to_bfloat16 = use_bf16_rounding;
+    constexpr int t = 3;
+    const std::vector<float> qg = RoundedToBFloat16(Values(t * 12, .1)),
+                             k = RoundedToBFloat16(Values(t * 3, 1.2)),
+                             v = RoundedToBFloat16(Values(t * 3, 2.3)), qn = Values(3, .2),
+                             kn = Values(3, .4), upstream = Values(t * 6, .7);
+    auto qw = Parameter(*executor, qn), kw = Parameter(*executor, kn);
+    ASSERT_TRUE((*qw)->Activate().ok());
+    ASSERT_TRUE((*kw)->Activate().ok());
+    ASSERT_TRUE((*qw)->Activate().ok());  // idempotent
+    auto layer = QwenAttentionLayer::Create(*executor, p, *qw, *kw, t);
+    ASSERT_TRUE(layer.ok());
+    auto qgb = Upload<BFloat16>(*executor, qg), kb = Upload<BFloat16>(*executor, k),
+         vb = Upload<BFloat16>(*executor, v);
+    auto dy = Upload<float>(*executor, upstream);
+    auto fwd = (*layer)->fwd(*executor, {*qgb, *kb, *vb});
+    ASSERT_TRUE(fwd.ok());
+    auto backward = (*layer)->bwd(*executor, {*dy}, std::move(fwd->state));
+    ASSERT_TRUE(backward.ok());
+    std::vector<std::vector<float>> actual;
+    for (const auto& b : *backward) actual.push_back(Read<float>(b));
+    actual.push_back(Read<float>((*qw)->gradient()));
+    actual.push_back(Read<float>((*kw)->gradient()));
+
+    const pluto_hip_attention_params abi = cached_attention_ops::ToAbi(p);
+    pluto_oracle_attention_params oracle_p;
+    static_assert(sizeof(oracle_p) == sizeof(abi));
+    std::memcpy(&oracle_p, &abi, sizeof(abi));
+    std::vector<std::vector<float>> want = {std::vector<float>(t * 12), std::vector<float>(t * 3),
+                                            std::vector<float>(t * 3), std::vector<float>(3, 0.f),
+                                            std::vector<float>(3, 0.f)};
+    ASSERT_EQ(pluto_oracle_gqa_sequence_backward(&oracle_p, t, qg.data(), k.data(), v.data(),
+                                                 qn.data(), kn.data(), upstream.data(),
+                                                 want[0].data(), want[1].data(), want[2].data(),
+                                                 want[3].data(), want[4].data()),
+              0);
+    for (size_t which = 0; which < want.size(); ++which) {
+      ASSERT_EQ(actual[which].size(), want[which].size());
+      for (size_t i = 0; i < want[which].size(); ++i)
+        EXPECT_NEAR(actual[which][i], want[which][i], 3e-5);
+    }
+    // Shared norm gradients accumulate across backward calls, not overwrite.
+    auto second = (*layer)->fwd(*executor, {*qgb, *kb, *vb});
+    ASSERT_TRUE(second.ok());
+    auto repeated = (*layer)->bwd(*executor, {*dy}, std::move(second->state));
+    ASSERT_TRUE(repeated.ok());
+    for (size_t i = 0; i < repeated->size(); ++i)
+      EXPECT_TRUE(Read<float>((*repeated)[i]) == actual[i]);
+    const auto summed = Read<float>((*qw)->gradient());
+    for (size_t i = 0; i < summed.size(); ++i) EXPECT_NEAR(summed[i], 2 * actual[3][i], 1e-6);
+    EXPECT_TRUE((*layer)->gradients().empty());
+    // a state of the wrong shape is rejected
+    auto third = (*layer)->fwd(*executor, {*qgb, *kb, *vb});
+    ASSERT_TRUE(third.ok());
+    third->state.intermediates.pop_back();
+    EXPECT_TRUE(IsInvalidArgument((*layer)->bwd(*executor, {*dy}, std::move(third->state)).status()));
+    ASSERT_TRUE((*qw)->Deactivate().ok());
+    EXPECT_FALSE((*qw)->active());
+  }
+}
+
+TEST(QwenAttentionTest, FrozenNormsStillPropagateToEarlierTokens) {
+  // qwen_attention_test.cc:303-345
+  auto executor = NewExecutor();
+  FullAttentionParameters p;
+  p.query_heads = 2;
+  p.key_value_heads = 1;
+  p.head_dim = 4;
+  p.rotary_dim = 2;
+  auto qw = Parameter(*executor, Values(4, .2)), kw = Parameter(*executor, Values(4, .4));
+  auto layer = QwenAttentionLayer::Create(*executor, p, *qw, *kw, 3);
+  ASSERT_TRUE(layer.ok());
+  auto q = Upload<BFloat16>(*executor, Values(48, .1)), k = Upload<BFloat16>(*executor, Values(12, 1.2)),
+       v = Upload<BFloat16>(*executor, Values(12, 2.3));
+  auto result = (*layer)->fwd(*executor, {*q, *k, *v});
+  ASSERT_TRUE(result.ok());
+  std::vector<float> grad(24, 0.f);
+  for (int i = 16; i < 24; ++i) grad[i] = .5f;
+  auto dy = Upload<float>(*executor, grad);
+  auto backward = (*layer)->bwd(*executor, {*dy}, std::move(result->state));
+  ASSERT_TRUE(backward.ok());
+  const auto dk = Read<float>((*backward)[1]), dv = Read<float>((*backward)[2]);
+  float key_magnitude = 0, value_magnitude = 0;
+  for (int i = 0; i < 4; ++i) {
+    key_magnitude += std::fabs(dk[i]);
+    value_magnitude += std::fabs(dv[i]);
+  }
+  EXPECT_GT(key_magnitude, 1e-5f);
+  EXPECT_GT(value_magnitude, 1e-5f);
+  EXPECT_FALSE((*qw)->active());
+  EXPECT_FALSE((*kw)->active());
+  // a gradient buffer of the wrong size is rejected
+  auto again = (*layer)->fwd(*executor, {*q, *k, *v});
+  ASSERT_TRUE(again.ok());
+  auto short_dy = Upload<float>(*executor, std::vector<float>(23, 0.f));
+  EXPECT_TRUE(IsInvalidArgument((*layer)->bwd(*executor, {*short_dy}, std::move(again->state)).status()));
 }
 
 TEST(QwenAttentionTest, RejectsIncompatibleCacheAndSequenceContracts) {
