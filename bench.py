@@ -45,7 +45,8 @@ MEASURED_TRAFFIC_BYTES = {
 NAMES = ["mha_train_bf16", "mha_fwd_fp32", "gqa_prefill", "gqa_decode", "gdn_scan"]
 # "copy" is a plain device copy of known size: the calibration case for the
 # FETCH_SIZE / WRITE_SIZE counters that `roofline.traffic` is derived from.
-EXTRA = ["copy"]
+# "gqa_prefill_bwd" times the Qwen sequence backward on its own.
+EXTRA = ["copy", "gqa_prefill_bwd"]
 
 
 def parse_args():
@@ -148,6 +149,34 @@ def gqa_prefill(torch, capi):
                 cpu=None)
 
 
+def gqa_prefill_bwd(torch, capi):
+    """Backward of the whole-sequence Qwen layer at the prefill shape (the row
+    after the headline ones: not part of --workload all)."""
+    import numpy as np
+    T, qh, kh, d = 8192, 24, 4, 128
+    p = capi.attention_params(qh, kh, d, 32, capacity=T)
+    gen = torch.Generator(device="cuda").manual_seed(2)
+    bf = torch.bfloat16
+    qg = (0.5 * torch.randn((T, qh, 2, d), generator=gen, device="cuda")).to(bf)
+    k = (0.5 * torch.randn((T, kh, d), generator=gen, device="cuda")).to(bf)
+    v = (0.5 * torch.randn((T, kh, d), generator=gen, device="cuda")).to(bf)
+    dy = torch.randn((T, qh, d), generator=gen, device="cuda")
+    qw = torch.from_numpy(values(np, d, 0.2, 0.3)).cuda()
+    kw = torch.from_numpy(values(np, d, 0.8, 0.4)).cuda()
+
+    def step():
+        capi.gqa_prefill_backward(p, qg, k, v, qw, kw, dy)
+
+    work = 10.0 * qh * d * causal_pairs(T)
+    return dict(step=step, parts=[("backward", step, work)], work=work,
+                metric="gqa_sequence_backward_tflops", unit="TFLOP/s", dtype="bf16", bound="mfma",
+                peak=PEAK_BF16_TFLOPS,
+                config={"workload": "qwen_gqa_sequence_backward", "batch": 1, "seq_len": T,
+                        "query_heads": qh, "kv_heads": kh, "head_dim": d,
+                        "counted": "5 attention GEMMs; the call also recomputes the forward"},
+                cpu=None)
+
+
 def gqa_decode(torch, capi):
     import numpy as np
     batch, qh, kh, d, capacity = 32, 24, 4, 128, 32768
@@ -231,7 +260,8 @@ def copy(torch, capi):
 
 
 WORKLOADS = {"copy": copy, "mha_train_bf16": mha_train_bf16, "mha_fwd_fp32": mha_fwd_fp32,
-             "gqa_prefill": gqa_prefill, "gqa_decode": gqa_decode, "gdn_scan": gdn_scan}
+             "gqa_prefill": gqa_prefill, "gqa_prefill_bwd": gqa_prefill_bwd, "gqa_decode": gqa_decode,
+             "gdn_scan": gdn_scan}
 
 
 def cpu_baseline_mha(spec):

@@ -19,6 +19,11 @@
  *                            exact gate expectation and uniform 1/L rows of
  *                            cached_attention_ops_test.cc:364-398,472-503,
  *                            an independent float64 numpy restatement.
+ *   gqa_sequence_backward    central finite differences of a frozen-rounding
+ *                            double-precision forward (the reference's own
+ *                            check, qwen_attention_test.cc:22-99,230-300, at
+ *                            its bound of 3e-5, both rounding modes) and
+ *                            float64 autograd of the unrounded layer.
  *   gdn_*                    textbook delta rule special cases (beta=0, g=0
  *                            with orthonormal keys), softplus extremes,
  *                            independent float64 numpy recurrence.
