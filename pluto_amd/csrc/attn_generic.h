@@ -49,6 +49,10 @@ struct GenericBackwardArgs {
 
 int launch_generic_forward(hipStream_t stream, const GenericForwardArgs& args,
                            int sequences);
+// FP32 storage, FP32 matrix-core arithmetic, head widths 32/64/128, no gate
+// (attn_f32_mfma.hip).
+bool f32_forward_supported(const GenericForwardArgs& args);
+int launch_f32_forward(hipStream_t stream, const GenericForwardArgs& args, int sequences);
 int launch_generic_probabilities(hipStream_t stream,
                                  const GenericForwardArgs& args, int sequences,
                                  float* probabilities);

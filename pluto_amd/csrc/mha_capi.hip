@@ -101,6 +101,7 @@ int pluto_hip_mha_forward(void* stream, int dtype, const void* qkv, int rows,
   }
   const GenericForwardArgs a =
       packed_forward_args(dtype, qkv, rows, T, H, E, out, maxima, normalizers);
+  if (!force_generic() && f32_forward_supported(a)) return launch_f32_forward(s, a, sequences);
   return launch_generic_forward(s, a, sequences);
 }
 
