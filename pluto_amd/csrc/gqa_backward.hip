@@ -19,31 +19,28 @@ namespace pluto_hip {
 namespace {
 
 // [T, qh, d] prepared queries, [T, kh, d] prepared keys and values ->
-// packed [T, 3E] (E = qh * d): Q | K of the head's kv head | V of it.
+// packed [T, 3E] (E = qh * d): Q | K of the head's kv head | V of it.  Moved in
+// pieces of PIECE elements (16 bytes when the head width allows).
+template <typename Element, int PIECE>
 __global__ void __launch_bounds__(256)
-pack_heads_kernel(const void* q, const void* k, const void* v, int dtype, int length, int qh,
-                  int kh, int d, void* packed) {
-  const long long E = 1LL * qh * d;
-  const long long total = 3LL * length * E;
+pack_heads_kernel(const Element* q, const Element* k, const Element* v, int length, int qh,
+                  int kh, int d, Element* packed) {
+  struct alignas(sizeof(Element) * PIECE) Piece {
+    Element e[PIECE];
+  };
+  const int pieces_per_head = d / PIECE;
+  const long long pieces_per_part = 1LL * qh * pieces_per_head;
+  const long long total = 3LL * length * pieces_per_part;
   const int group = qh / kh;
   for (long long i = blockIdx.x * 256LL + threadIdx.x; i < total; i += 256LL * gridDim.x) {
-    const long long t = i / (3 * E);
-    const long long within = i % (3 * E);
-    const int part = static_cast<int>(within / E);
-    const int h = static_cast<int>((within % E) / d), c = static_cast<int>(within % d);
-    long long source;
-    const void* base;
-    if (part == 0) {
-      base = q;
-      source = (t * qh + h) * d + c;
-    } else {
-      base = part == 1 ? k : v;
-      source = (t * kh + h / group) * d + c;
-    }
-    if (dtype == PLUTO_HIP_BF16)
-      static_cast<uint16_t*>(packed)[i] = static_cast<const uint16_t*>(base)[source];
-    else
-      static_cast<float*>(packed)[i] = static_cast<const float*>(base)[source];
+    const long long t = i / (3 * pieces_per_part);
+    const long long within = i % (3 * pieces_per_part);
+    const int part = static_cast<int>(within / pieces_per_part);
+    const int h = static_cast<int>((within % pieces_per_part) / pieces_per_head);
+    const int c = static_cast<int>(within % pieces_per_head) * PIECE;
+    const Element* source = part == 0 ? q + (t * qh + h) * d + c
+                                      : (part == 1 ? k : v) + (t * kh + h / group) * d + c;
+    *reinterpret_cast<Piece*>(packed + i * PIECE) = *reinterpret_cast<const Piece*>(source);
   }
 }
 
@@ -184,8 +181,30 @@ int grid_for(long long elements) {
 
 int launch_pack_heads(hipStream_t stream, const void* q, const void* k, const void* v, int dtype,
                       int length, int qh, int kh, int d, void* packed) {
-  pack_heads_kernel<<<grid_for(3LL * length * qh * d), 256, 0, stream>>>(q, k, v, dtype, length,
-                                                                         qh, kh, d, packed);
+  const long long elements = 3LL * length * qh * d;
+  if (dtype == PLUTO_HIP_BF16) {
+    auto* qs = static_cast<const uint16_t*>(q);
+    auto* ks = static_cast<const uint16_t*>(k);
+    auto* vs = static_cast<const uint16_t*>(v);
+    auto* out = static_cast<uint16_t*>(packed);
+    if (d % 8 == 0)
+      pack_heads_kernel<uint16_t, 8><<<grid_for(elements / 8), 256, 0, stream>>>(qs, ks, vs, length,
+                                                                                 qh, kh, d, out);
+    else
+      pack_heads_kernel<uint16_t, 1><<<grid_for(elements), 256, 0, stream>>>(qs, ks, vs, length, qh,
+                                                                             kh, d, out);
+  } else {
+    auto* qs = static_cast<const float*>(q);
+    auto* ks = static_cast<const float*>(k);
+    auto* vs = static_cast<const float*>(v);
+    auto* out = static_cast<float*>(packed);
+    if (d % 4 == 0)
+      pack_heads_kernel<float, 4><<<grid_for(elements / 4), 256, 0, stream>>>(qs, ks, vs, length, qh,
+                                                                              kh, d, out);
+    else
+      pack_heads_kernel<float, 1><<<grid_for(elements), 256, 0, stream>>>(qs, ks, vs, length, qh, kh,
+                                                                          d, out);
+  }
   return launch_status();
 }
 
