@@ -740,6 +740,242 @@ int pluto_oracle_gdn_sequence(const pluto_oracle_delta_params* p, int length,
   return 0;
 }
 
+/* Backward of the whole layer: SequenceDeltaNetLayer::bwd_impl
+ * (sequence_delta_net.cc:482-561) with its kernels OutputBackward (:125-155),
+ * SumNormGradient (:157-166), RecurrenceBackward (:171-253), GatherQkGradient
+ * (:255-276), GatherScalarGradient (:278-305), ConvSiluBackward (:307-318),
+ * ConvInputBackward (:320-336), ConvWeightBackward (:338-355), in double
+ * precision.  Rounding points have derivative one; the operands are the saved
+ * (rounded) forward values where the reference reads them from its saved
+ * state.  Parameter gradients (nullable) are added to. */
+int pluto_oracle_gdn_sequence_backward(
+    const pluto_oracle_delta_params* p, int length, const float* qkv, const float* z,
+    const float* a, const float* b, const float* conv_weight, const float* a_log,
+    const float* dt_bias, const float* norm, const float* dy, float* dqkv, float* dz,
+    float* da, float* db, float* d_conv_weight, float* d_a_log, float* d_dt_bias,
+    float* d_norm) {
+  if (!delta_params_ok(p) || length <= 0) return -1;
+  const int kh = p->key_heads, vh = p->value_heads;
+  const int kd = p->key_head_dim, vd = p->value_head_dim;
+  const int kernel = p->conv_kernel_dim;
+  const int channels = 2 * kh * kd + vh * vd;
+  const int round = p->round_to_bfloat16;
+  const size_t state_size = (size_t)kd * vd;
+  double* pre = (double*)malloc(sizeof(double) * (size_t)length * channels);
+  double* post = (double*)malloc(sizeof(double) * (size_t)length * channels);
+  double* dpost = (double*)calloc((size_t)length * channels, sizeof(double));
+  double* dpre = (double*)malloc(sizeof(double) * (size_t)length * channels);
+  double* core = (double*)malloc(sizeof(double) * (size_t)length * vh * vd);
+  double* dcore = (double*)malloc(sizeof(double) * (size_t)length * vh * vd);
+  double* states = (double*)calloc((size_t)(length + 1) * state_size, sizeof(double));
+  double* dm = (double*)malloc(sizeof(double) * state_size);
+  double* tmp = (double*)malloc(sizeof(double) * (size_t)(8 * kd + 4 * vd));
+  if (!pre || !post || !dpost || !dpre || !core || !dcore || !states || !dm || !tmp) {
+    free(pre); free(post); free(dpost); free(dpre); free(core); free(dcore);
+    free(states); free(dm); free(tmp);
+    return -1;
+  }
+  for (int t = 0; t < length; ++t)
+    for (int c = 0; c < channels; ++c) {
+      double sum = 0;
+      for (int tap = 0; tap < kernel; ++tap) {
+        const int source = t + tap - kernel + 1;
+        if (source >= 0)
+          sum += (double)qkv[(size_t)source * channels + c] *
+                 (double)conv_weight[(size_t)c * kernel + tap];
+      }
+      sum = round_bf16_f64(sum, round);
+      pre[(size_t)t * channels + c] = sum;
+      post[(size_t)t * channels + c] = round_bf16_f64(sum / (1 + exp(-sum)), round);
+    }
+  double *raw_q = tmp, *raw_k = tmp + kd, *q = tmp + 2 * kd, *k = tmp + 3 * kd;
+  double *dq = tmp + 4 * kd, *dk = tmp + 5 * kd, *sum_q = tmp + 6 * kd, *sum_k = tmp + 7 * kd;
+  double *v = tmp + 8 * kd, *difference = v + vd, *delta = v + 2 * vd, *ddelta = v + 3 * vd;
+  for (int t = 0; t < length; ++t) {
+    memset(da + (size_t)t * vh, 0, sizeof(float) * (size_t)vh);
+    memset(db + (size_t)t * vh, 0, sizeof(float) * (size_t)vh);
+  }
+  for (int head = 0; head < vh; ++head) {
+    const int key_head = head / (vh / kh);
+    /* forward with every state kept (RecurrenceForward, :55-102) */
+    memset(states, 0, sizeof(double) * state_size);
+    for (int t = 0; t < length; ++t) {
+      const double* row = post + (size_t)t * channels;
+      double q_norm = 1e-6, k_norm = 1e-6;
+      for (int d = 0; d < kd; ++d) {
+        raw_q[d] = row[key_head * kd + d];
+        raw_k[d] = row[(kh + key_head) * kd + d];
+        q_norm += raw_q[d] * raw_q[d];
+        k_norm += raw_k[d] * raw_k[d];
+      }
+      for (int d = 0; d < kd; ++d) {
+        q[d] = raw_q[d] / sqrt(q_norm) / sqrt((double)kd);
+        k[d] = raw_k[d] / sqrt(k_norm);
+      }
+      const double alpha = (double)a[(size_t)t * vh + head] + (double)dt_bias[head];
+      const double softplus = fmax(alpha, 0.) + log1p(exp(-fabs(alpha)));
+      const double decay = exp(-exp((double)a_log[head]) * softplus);
+      const double beta =
+          round_bf16_f64(1 / (1 + exp(-(double)b[(size_t)t * vh + head])), round);
+      const double* previous = states + (size_t)t * state_size;
+      double* next = states + (size_t)(t + 1) * state_size;
+      for (int c = 0; c < vd; ++c) {
+        double prediction = 0;
+        for (int d = 0; d < kd; ++d) prediction += previous[(size_t)d * vd + c] * decay * k[d];
+        const double dl = (row[2 * kh * kd + head * vd + c] - prediction) * beta;
+        double out = 0;
+        for (int d = 0; d < kd; ++d) {
+          const double value = previous[(size_t)d * vd + c] * decay + k[d] * dl;
+          next[(size_t)d * vd + c] = value;
+          out += value * q[d];
+        }
+        core[((size_t)t * vh + head) * vd + c] = round_bf16_f64(out, round);
+      }
+    }
+    /* OutputBackward (:125-155) for this head's rows */
+    double norm_partial[256];
+    for (int c = 0; c < vd; ++c) norm_partial[c] = 0;
+    for (int t = 0; t < length; ++t) {
+      const size_t base = ((size_t)t * vh + head) * vd;
+      double sum = 0;
+      for (int c = 0; c < vd; ++c) sum += core[base + c] * core[base + c];
+      const double inverse = 1 / sqrt(sum / vd + (double)p->rms_norm_epsilon);
+      double dot = 0;
+      for (int c = 0; c < vd; ++c) {
+        const double gate = (double)z[base + c];
+        const double sigmoid = 1 / (1 + exp(-gate));
+        const double dn = (double)dy[base + c] * gate * sigmoid * (double)norm[c];
+        dot += dn * core[base + c];
+      }
+      for (int c = 0; c < vd; ++c) {
+        const double x = core[base + c];
+        const double gate = (double)z[base + c];
+        const double sigmoid = 1 / (1 + exp(-gate));
+        const double normalized = round_bf16_f64(x * inverse, round);
+        const double affine = round_bf16_f64(normalized * (double)norm[c], round);
+        const double dn = (double)dy[base + c] * gate * sigmoid * (double)norm[c];
+        dcore[base + c] = inverse * dn - x * inverse * inverse * inverse / vd * dot;
+        dz[base + c] = (float)((double)dy[base + c] * affine * sigmoid *
+                               (1 + gate * (1 - sigmoid)));
+        norm_partial[c] += (double)dy[base + c] * gate * sigmoid * normalized;
+      }
+    }
+    if (d_norm)
+      for (int c = 0; c < vd; ++c) d_norm[c] += (float)norm_partial[c];
+    /* RecurrenceBackward (:171-253) */
+    for (size_t i = 0; i < state_size; ++i) dm[i] = 0;
+    double head_dalog = 0, head_dbias = 0;
+    for (int t = length - 1; t >= 0; --t) {
+      const double* row = post + (size_t)t * channels;
+      double q_norm = 1e-6, k_norm = 1e-6;
+      for (int d = 0; d < kd; ++d) {
+        raw_q[d] = row[key_head * kd + d];
+        raw_k[d] = row[(kh + key_head) * kd + d];
+        q_norm += raw_q[d] * raw_q[d];
+        k_norm += raw_k[d] * raw_k[d];
+      }
+      const double iq = 1 / sqrt(q_norm), ik = 1 / sqrt(k_norm);
+      const double norm_scale = sqrt((double)kd);
+      for (int d = 0; d < kd; ++d) {
+        q[d] = raw_q[d] * iq / norm_scale;
+        k[d] = raw_k[d] * ik;
+      }
+      const double alpha = (double)a[(size_t)t * vh + head] + (double)dt_bias[head];
+      const double softplus = fmax(alpha, 0.) + log1p(exp(-fabs(alpha)));
+      const double rate = exp((double)a_log[head]);
+      const double decay = exp(-rate * softplus);
+      const double sigmoid = 1 / (1 + exp(-(double)b[(size_t)t * vh + head]));
+      const double beta = round_bf16_f64(sigmoid, round);
+      const double* previous = states + (size_t)t * state_size;
+      const double* matrix = states + (size_t)(t + 1) * state_size;
+      const double* grad = dcore + ((size_t)t * vh + head) * vd;
+      for (int c = 0; c < vd; ++c) {
+        double prediction = 0;
+        for (int d = 0; d < kd; ++d) prediction += previous[(size_t)d * vd + c] * decay * k[d];
+        difference[c] = row[2 * kh * kd + head * vd + c] - prediction;
+        delta[c] = difference[c] * beta;
+      }
+      for (int d = 0; d < kd; ++d) {
+        double sum = 0;
+        for (int c = 0; c < vd; ++c) {
+          sum += matrix[(size_t)d * vd + c] * grad[c];
+          dm[(size_t)d * vd + c] += q[d] * grad[c];
+        }
+        dq[d] = sum;
+      }
+      double dbeta = 0;
+      for (int c = 0; c < vd; ++c) {
+        double sum = 0;
+        for (int d = 0; d < kd; ++d) sum += dm[(size_t)d * vd + c] * k[d];
+        ddelta[c] = sum;
+        dbeta += sum * difference[c];
+        dpost[(size_t)t * channels + 2 * kh * kd + head * vd + c] = sum * beta;
+      }
+      double dg = 0;
+      for (int d = 0; d < kd; ++d) {
+        double sum = 0;
+        for (int c = 0; c < vd; ++c) {
+          const double dvalue = ddelta[c] * beta;
+          const double decayed = previous[(size_t)d * vd + c] * decay;
+          sum += dm[(size_t)d * vd + c] * delta[c] - decayed * dvalue;
+          const double ddecayed = dm[(size_t)d * vd + c] - k[d] * dvalue;
+          dg += ddecayed * previous[(size_t)d * vd + c];
+          dm[(size_t)d * vd + c] = ddecayed * decay;
+        }
+        dk[d] = sum;
+      }
+      const double dalpha = -dg * decay * rate / (1 + exp(-alpha));
+      da[(size_t)t * vh + head] = (float)dalpha;
+      db[(size_t)t * vh + head] = (float)(dbeta * sigmoid * (1 - sigmoid));
+      head_dalog += -dg * decay * rate * softplus;
+      head_dbias += dalpha;
+      double q_dot = 0, k_dot = 0;
+      for (int d = 0; d < kd; ++d) {
+        q_dot += dq[d] * raw_q[d];
+        k_dot += dk[d] * raw_k[d];
+      }
+      for (int d = 0; d < kd; ++d) {
+        sum_q[d] = (dq[d] * iq - raw_q[d] * iq * iq * iq * q_dot) / norm_scale;
+        sum_k[d] = dk[d] * ik - raw_k[d] * ik * ik * ik * k_dot;
+        /* GatherQkGradient (:255-276): heads of a key head add up */
+        dpost[(size_t)t * channels + key_head * kd + d] += sum_q[d];
+        dpost[(size_t)t * channels + (kh + key_head) * kd + d] += sum_k[d];
+      }
+    }
+    if (d_a_log) d_a_log[head] += (float)head_dalog;
+    if (d_dt_bias) d_dt_bias[head] += (float)head_dbias;
+  }
+  /* ConvSiluBackward, ConvInputBackward, ConvWeightBackward (:307-355) */
+  for (size_t i = 0; i < (size_t)length * channels; ++i) {
+    const double x = pre[i];
+    const double sigmoid = 1 / (1 + exp(-x));
+    dpre[i] = dpost[i] * sigmoid * (1 + x * (1 - sigmoid));
+  }
+  for (int t = 0; t < length; ++t)
+    for (int c = 0; c < channels; ++c) {
+      double sum = 0;
+      for (int tap = 0; tap < kernel; ++tap) {
+        const int future = t + kernel - 1 - tap;
+        if (future < length)
+          sum += dpre[(size_t)future * channels + c] *
+                 (double)conv_weight[(size_t)c * kernel + tap];
+      }
+      dqkv[(size_t)t * channels + c] = (float)sum;
+    }
+  if (d_conv_weight)
+    for (int c = 0; c < channels; ++c)
+      for (int tap = 0; tap < kernel; ++tap) {
+        double sum = 0;
+        for (int t = kernel - 1 - tap; t < length; ++t)
+          sum += dpre[(size_t)t * channels + c] *
+                 (double)qkv[(size_t)(t + tap - kernel + 1) * channels + c];
+        d_conv_weight[(size_t)c * kernel + tap] += (float)sum;
+      }
+  free(pre); free(post); free(dpost); free(dpre); free(core); free(dcore);
+  free(states); free(dm); free(tmp);
+  return 0;
+}
+
 int pluto_oracle_gdn_step(const pluto_oracle_delta_params* p,
                           float* conv_state, double* recurrent_state,
                           const float* qkv, const float* z, const float* a,

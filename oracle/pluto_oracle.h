@@ -187,6 +187,18 @@ int pluto_oracle_gdn_sequence(const pluto_oracle_delta_params* p, int length,
                               const float* norm, float* output, float* core,
                               double* final_state);
 
+/* Gradients of pluto_oracle_gdn_sequence with respect to its four activation
+ * inputs and four parameters for an upstream gradient dy [T, vh*vd]
+ * (SequenceDeltaNetLayer::bwd_impl, sequence_delta_net.cc:482-561).  dqkv
+ * [T, channels], dz [T, vh*vd], da, db [T, vh] are overwritten; the parameter
+ * gradients (nullable; shapes of the parameters) are added to. */
+int pluto_oracle_gdn_sequence_backward(
+    const pluto_oracle_delta_params* p, int length, const float* qkv, const float* z,
+    const float* a, const float* b, const float* conv_weight, const float* a_log,
+    const float* dt_bias, const float* norm, const float* dy, float* dqkv, float* dz,
+    float* da, float* db, float* d_conv_weight, float* d_a_log, float* d_dt_bias,
+    float* d_norm);
+
 /* Single-token step with persistent state: cached_attention_ops_test.cc:
  * 133-220 (scalar specification of DeltaNetState::Step,
  * cached_attention_ops.cc:401-431).  conv_state is FP32 [channels, kernel],

@@ -296,6 +296,30 @@ def gdn_sequence(p, qkv, z, a, b, conv_weight, a_log, dt_bias, norm):
     return dict(out=out, core=core, state=state)
 
 
+def gdn_sequence_backward(p, qkv, z, a, b, conv_weight, a_log, dt_bias, norm, dy,
+                          parameter_grads=True):
+    """Gradients of gdn_sequence for the upstream gradient dy [T, vh*vd].
+    Returns dict(dqkv, dz, da, db, d_conv_weight, d_a_log, d_dt_bias, d_norm)."""
+    qkv, z, a, b, dy = _f32(qkv), _f32(z), _f32(a), _f32(b), _f32(dy)
+    conv_weight, a_log = _f32(conv_weight), _f32(a_log)
+    dt_bias, norm = _f32(dt_bias), _f32(norm)
+    T = qkv.shape[0]
+    out = dict(dqkv=np.zeros_like(qkv), dz=np.zeros_like(z), da=np.zeros_like(a),
+               db=np.zeros_like(b), d_conv_weight=np.zeros_like(conv_weight),
+               d_a_log=np.zeros_like(a_log), d_dt_bias=np.zeros_like(dt_bias),
+               d_norm=np.zeros_like(norm))
+    fn = lib().pluto_oracle_gdn_sequence_backward
+    fn.restype = ctypes.c_int
+    grads = [_ptr(out[n]) if parameter_grads else None
+             for n in ("d_conv_weight", "d_a_log", "d_dt_bias", "d_norm")]
+    rc = fn(ctypes.byref(p), T, _ptr(qkv), _ptr(z), _ptr(a), _ptr(b), _ptr(conv_weight),
+            _ptr(a_log), _ptr(dt_bias), _ptr(norm), _ptr(dy), _ptr(out["dqkv"]), _ptr(out["dz"]),
+            _ptr(out["da"]), _ptr(out["db"]), *grads)
+    if rc != 0:
+        raise ValueError("oracle rejected the delta-net backward")
+    return out
+
+
 class DeltaNetStep:
     """Stateful mirror of the reference test's DeltaReference."""
 
