@@ -340,6 +340,31 @@ int pluto_hip_gdn_layer_forward(void* stream, const pluto_hip_delta_params* p,
                                 float* state, void* out, void* workspace,
                                 size_t workspace_bytes);
 
+/* Backward of the whole layer: SequenceDeltaNetLayer::bwd_impl
+ * (sequence_delta_net.cc:482-561; kernels OutputBackward :125-155,
+ * RecurrenceBackward :171-253, the two gathers :255-305, the convolution
+ * backward kernels :307-355).  Self-contained: it takes the layer's inputs and
+ * repeats the forward pass, keeping the recurrent state after every token in
+ * the workspace ((length + 1) * vh * kd * vd floats, as the reference's saved
+ * state does), so it is meant for training-length sequences (length <= 65535
+ * and as far as that scratch fits).  FP32 arithmetic, token by token.
+ *   dy    fp32 [batch, length, vh*vd]
+ *   dqkv  fp32 [batch, length, channels];  dz fp32 [batch, length, vh*vd]
+ *   da, db  fp32 [batch, length, vh]
+ *   d_conv_weight [channels, kernel], d_a_log, d_dt_bias [vh], d_norm [vd]:
+ *        optional; the parameters' gradients are ADDED to them. */
+size_t pluto_hip_gdn_layer_backward_workspace_bytes(const pluto_hip_delta_params* p,
+                                                    int length, int norm_grad);
+int pluto_hip_gdn_layer_backward(void* stream, const pluto_hip_delta_params* p,
+                                 int batch, int length, const void* qkv,
+                                 const void* z, const void* a, const void* b,
+                                 const float* conv_weight, const float* a_log,
+                                 const float* dt_bias, const float* norm,
+                                 const float* dy, float* dqkv, float* dz, float* da,
+                                 float* db, float* d_conv_weight, float* d_a_log,
+                                 float* d_dt_bias, float* d_norm, void* workspace,
+                                 size_t workspace_bytes);
+
 /* DeltaNetState::Step (src/llm/layers/util/cached_attention_ops.cc:401-431:
  * ConvolutionKernel :180-203, DeltaRecurrenceKernel :205-251, DeltaOutputKernel
  * :253-272): one token, contiguous FP32 device arrays as in the reference.

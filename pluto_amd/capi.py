@@ -112,6 +112,9 @@ SIGNATURES = {
     "pluto_hip_gdn_layer_workspace_bytes": (_SZ, [ctypes.POINTER(DeltaParams), _I, _I]),
     "pluto_hip_gdn_layer_forward": (_I, [_VP, ctypes.POINTER(DeltaParams), _I, _I] + [_VP] * 10 +
                                     [_VP, _SZ]),
+    "pluto_hip_gdn_layer_backward_workspace_bytes": (_SZ, [ctypes.POINTER(DeltaParams), _I, _I]),
+    "pluto_hip_gdn_layer_backward": (_I, [_VP, ctypes.POINTER(DeltaParams), _I, _I] + [_VP] * 17 +
+                                     [_VP, _SZ]),
     "pluto_hip_gdn_step_workspace_bytes": (_SZ, [ctypes.POINTER(DeltaParams)]),
     "pluto_hip_gdn_step": (_I, [_VP, ctypes.POINTER(DeltaParams)] + [_VP] * 11 + [_VP, _SZ]),
     "pluto_hip_gdn_recurrence": (_I, [_VP, ctypes.POINTER(DeltaParams), _I, _I, _VP, _VP,
@@ -388,6 +391,28 @@ def gdn_layer_forward(p, qkv, z, a, b, conv_weight, a_log, dt_bias, norm, state,
                                             ptr(conv_weight), ptr(a_log), ptr(dt_bias), ptr(norm),
                                             ptr(state), ptr(out), ptr(workspace), workspace.numel()))
     return out
+
+
+def gdn_layer_backward(p, qkv, z, a, b, conv_weight, a_log, dt_bias, norm, dy,
+                       parameter_grads=None, stream=None):
+    """Gradients of gdn_layer_forward (zero initial state) for dy fp32 [B, T, vh*vd].
+
+    Returns (dqkv, dz, da, db), all fp32 with the inputs' shapes.  parameter_grads: optional
+    dict with fp32 accumulators "conv_weight", "a_log", "dt_bias", "norm" (any subset)."""
+    batch, length = qkv.shape[0], qkv.shape[1]
+    grads = parameter_grads or {}
+    f32 = dict(dtype=torch.float32, device=qkv.device)
+    dqkv, dz = torch.empty(qkv.shape, **f32), torch.empty(z.shape, **f32)
+    da, db = torch.empty(a.shape, **f32), torch.empty(b.shape, **f32)
+    size = lib().pluto_hip_gdn_layer_backward_workspace_bytes(ctypes.byref(p), length,
+                                                              int("norm" in grads))
+    workspace = torch.empty(max(size, 16), dtype=torch.uint8, device=qkv.device)
+    check(lib().pluto_hip_gdn_layer_backward(
+        stream or current_stream(), ctypes.byref(p), batch, length, ptr(qkv), ptr(z), ptr(a),
+        ptr(b), ptr(conv_weight), ptr(a_log), ptr(dt_bias), ptr(norm), ptr(dy), ptr(dqkv), ptr(dz),
+        ptr(da), ptr(db), ptr(grads.get("conv_weight")), ptr(grads.get("a_log")),
+        ptr(grads.get("dt_bias")), ptr(grads.get("norm")), ptr(workspace), size))
+    return dqkv, dz, da, db
 
 
 class DeltaNetStep:

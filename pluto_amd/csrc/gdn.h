@@ -68,4 +68,15 @@ int launch_gdn_output(hipStream_t stream, const void* core, int core_dtype, cons
                       int z_dtype, const float* norm, long long rows, int value_dim,
                       float epsilon, bool round, void* out, int out_dtype);
 
+// Backward of the whole layer for one sequence (gdn_backward.hip): the forward
+// pass is repeated with every per-token state kept in `workspace`.
+constexpr int kGdnSumChunks = 128;
+size_t gdn_backward_workspace_bytes(const pluto_hip_delta_params* p, int length, bool norm_grad);
+int launch_gdn_backward(hipStream_t stream, const pluto_hip_delta_params* p, int length,
+                        const void* qkv, const void* z, const void* a, const void* b,
+                        const float* conv_weight, const float* a_log, const float* dt_bias,
+                        const float* norm, const float* dy, float* dqkv, float* dz, float* da,
+                        float* db, float* d_conv_weight, float* d_a_log, float* d_dt_bias,
+                        float* d_norm, void* workspace);
+
 }  // namespace pluto_hip

@@ -1,0 +1,529 @@
+// Backward of the gated delta-net layer over a sequence
+// (SequenceDeltaNetLayer::bwd_impl, src/llm/layers/sequence_delta_net.cc:
+// 482-561) in FP32, token by token as the reference does it: the forward pass
+// is repeated with every state S_t kept, then the recurrence is differentiated
+// in reverse.  Kernels and the reference kernels they follow:
+//   conv_train_kernel            ConvForward            (:31-51), keeps `pre`
+//   recurrence_states_kernel     RecurrenceForward      (:55-102)
+//   output_backward_kernel       OutputBackward         (:125-155)
+//   recurrence_backward_kernel   RecurrenceBackward     (:171-253)
+//   gather_qk_kernel             GatherQkGradient       (:255-276)
+//   gather_scalar_kernel         GatherScalarGradient   (:278-305)
+//   conv_silu_backward_kernel    ConvSiluBackward       (:307-318)
+//   conv_input_backward_kernel   ConvInputBackward      (:320-336)
+//   conv_weight_backward_kernel  ConvWeightBackward     (:338-355)
+//   sum_rows_*_kernel            SumNormGradient        (:157-166), two levels
+//
+// The two recurrence kernels share one layout: a workgroup owns the
+// [key_dim, 32] slice of one head's state (as the reference's programs do),
+// thread (kg, c) = (tid / 32, tid % 32) holds rows 16 kg .. 16 kg + 15 of
+// column c in registers.  Sums over rows go through LDS (8 partials a column),
+// sums over columns through lane shuffles within a 32-lane half.
+#include "gdn.h"
+
+namespace pluto_hip {
+namespace {
+
+constexpr int kRows = 16;        // state rows per thread
+constexpr int kGroups = 8;       // row groups per workgroup
+constexpr int kColumns = 32;     // state columns per workgroup
+constexpr int kMaxKey = kRows * kGroups;  // 128
+
+__device__ inline float round_if(float x, bool round) { return round ? round_to_bf16(x) : x; }
+
+__global__ void __launch_bounds__(256)
+conv_train_kernel(const uint16_t* input, const float* __restrict__ weight, int length,
+                  int channels, int kernel, bool round, float* pre, float* post) {
+  const long long total = 1LL * length * channels;
+  const long long i = blockIdx.x * 256LL + threadIdx.x;
+  if (i >= total) return;
+  const int c = static_cast<int>(i % channels), t = static_cast<int>(i / channels);
+  float sum = 0.0f;
+  for (int tap = 0; tap < kernel; ++tap) {
+    const int source = t + tap - kernel + 1;
+    if (source >= 0)
+      sum += bf16_bits_to_float(input[1LL * source * channels + c]) * weight[1LL * c * kernel + tap];
+  }
+  sum = round_if(sum, round);
+  pre[i] = sum;
+  post[i] = round_if(sum / (1.0f + expf(-sum)), round);
+}
+
+struct RecurrenceArgs {
+  const float* post = nullptr;     // [T, channels]
+  const uint16_t* a = nullptr;     // bf16 [T, vh]
+  const uint16_t* b = nullptr;
+  const float* a_log = nullptr;
+  const float* dt_bias = nullptr;
+  float* states = nullptr;         // [(T + 1), vh, kd, vd]
+  float* core = nullptr;           // [T, vh, vd]
+  const float* dcore = nullptr;    // [T, vh, vd]
+  float* qk_partials = nullptr;    // [T, vh, tiles, 2, kd]
+  float* scalar_partials = nullptr;  // [T, vh, tiles, 3]
+  float* dpost = nullptr;          // [T, channels]; the value part is written here
+  int length = 0, kh = 0, vh = 0, kd = 0, vd = 0;
+  bool round = true;
+};
+
+struct TokenScalars {
+  float alpha, softplus, rate, decay, sigmoid, beta;
+};
+
+__device__ inline TokenScalars token_scalars(const RecurrenceArgs& a, int t, int head) {
+  TokenScalars s;
+  s.alpha = bf16_bits_to_float(a.a[1LL * t * a.vh + head]) + a.dt_bias[head];
+  s.softplus = fmaxf(s.alpha, 0.0f) + logf(1.0f + expf(-fabsf(s.alpha)));
+  s.rate = expf(a.a_log[head]);
+  s.decay = expf(-s.rate * s.softplus);
+  s.sigmoid = 1.0f / (1.0f + expf(-bf16_bits_to_float(a.b[1LL * t * a.vh + head])));
+  s.beta = round_if(s.sigmoid, a.round);
+  return s;
+}
+
+// Raw q and k of one token into LDS together with 1/|q|, 1/|k| (1e-6 added to
+// the sums of squares, sequence_delta_net.cc:84-85).
+__device__ inline void load_token_qk(const RecurrenceArgs& a, int t, int key_head, float* raw_q,
+                                     float* raw_k, float* inverses) {
+  const int channels = 2 * a.kh * a.kd + a.vh * a.vd;
+  const int tid = threadIdx.x;
+  if (tid < 64) {
+    float qq = 0.0f, kk = 0.0f;
+    for (int d = tid; d < kMaxKey; d += 64) {
+      float qv = 0.0f, kv = 0.0f;
+      if (d < a.kd) {
+        qv = a.post[1LL * t * channels + key_head * a.kd + d];
+        kv = a.post[1LL * t * channels + (a.kh + key_head) * a.kd + d];
+      }
+      raw_q[d] = qv;
+      raw_k[d] = kv;
+      qq += qv * qv;
+      kk += kv * kv;
+    }
+    qq = wave_sum(qq);
+    kk = wave_sum(kk);
+    if (tid == 0) {
+      inverses[0] = rsqrtf(qq + 1e-6f);
+      inverses[1] = rsqrtf(kk + 1e-6f);
+    }
+  }
+}
+
+// Sum over the kGroups row groups of a per-column partial.
+__device__ inline float column_total(float partial, float (*scratch)[kColumns], int kg, int c) {
+  scratch[kg][c] = partial;
+  __syncthreads();
+  float total = 0.0f;
+#pragma unroll
+  for (int g = 0; g < kGroups; ++g) total += scratch[g][c];
+  __syncthreads();
+  return total;
+}
+
+__device__ inline float half_wave_sum(float v) {
+#pragma unroll
+  for (int offset = 16; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, 64);
+  return v;
+}
+
+__global__ void __launch_bounds__(256)
+recurrence_states_kernel(RecurrenceArgs a) {
+  __shared__ float raw_q[kMaxKey], raw_k[kMaxKey], inverses[2];
+  __shared__ float scratch[kGroups][kColumns];
+  const int tiles = (a.vd + kColumns - 1) / kColumns;
+  const int head = blockIdx.x / tiles, tile = blockIdx.x % tiles;
+  const int key_head = head / (a.vh / a.kh);
+  const int kg = threadIdx.x / kColumns, c = threadIdx.x % kColumns;
+  const int column = tile * kColumns + c;
+  const bool column_ok = column < a.vd;
+  const int channels = 2 * a.kh * a.kd + a.vh * a.vd;
+  const size_t stride = static_cast<size_t>(a.vh) * a.kd * a.vd;
+  const float norm_scale = sqrtf(static_cast<float>(a.kd));
+  float m[kRows];
+#pragma unroll
+  for (int r = 0; r < kRows; ++r) {
+    m[r] = 0.0f;
+    const int row = kg * kRows + r;
+    if (row < a.kd && column_ok) a.states[(static_cast<size_t>(head) * a.kd + row) * a.vd + column] = 0.0f;
+  }
+  for (int t = 0; t < a.length; ++t) {
+    load_token_qk(a, t, key_head, raw_q, raw_k, inverses);
+    __syncthreads();
+    const TokenScalars s = token_scalars(a, t, head);
+    const float iq = inverses[0], ik = inverses[1];
+    float prediction = 0.0f;
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) {
+      m[r] *= s.decay;
+      prediction += m[r] * (raw_k[kg * kRows + r] * ik);
+    }
+    prediction = column_total(prediction, scratch, kg, c);
+    const float v = column_ok ? a.post[1LL * t * channels + 2 * a.kh * a.kd + head * a.vd + column] : 0.0f;
+    const float delta = (v - prediction) * s.beta;
+    float out = 0.0f;
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) {
+      const int row = kg * kRows + r;
+      m[r] += (raw_k[row] * ik) * delta;
+      out += m[r] * (raw_q[row] * iq / norm_scale);
+      if (row < a.kd && column_ok)
+        a.states[(t + 1) * stride + (static_cast<size_t>(head) * a.kd + row) * a.vd + column] = m[r];
+    }
+    out = column_total(out, scratch, kg, c);
+    if (kg == 0 && column_ok) a.core[(1LL * t * a.vh + head) * a.vd + column] = round_if(out, a.round);
+  }
+}
+
+__global__ void __launch_bounds__(256)
+recurrence_backward_kernel(RecurrenceArgs a) {
+  __shared__ float raw_q[kMaxKey], raw_k[kMaxKey], inverses[2];
+  __shared__ float scratch[kGroups][kColumns];
+  __shared__ float dq_rows[kMaxKey], dk_rows[kMaxKey];
+  __shared__ float block_sums[4][3];
+  const int tiles = (a.vd + kColumns - 1) / kColumns;
+  const int head = blockIdx.x / tiles, tile = blockIdx.x % tiles;
+  const int key_head = head / (a.vh / a.kh);
+  const int tid = threadIdx.x, wave = tid / 64;
+  const int kg = tid / kColumns, c = tid % kColumns;
+  const int column = tile * kColumns + c;
+  const bool column_ok = column < a.vd;
+  const int channels = 2 * a.kh * a.kd + a.vh * a.vd;
+  const size_t stride = static_cast<size_t>(a.vh) * a.kd * a.vd;
+  const float norm_scale = sqrtf(static_cast<float>(a.kd));
+  float dm[kRows];
+#pragma unroll
+  for (int r = 0; r < kRows; ++r) dm[r] = 0.0f;
+  for (int t = a.length - 1; t >= 0; --t) {
+    load_token_qk(a, t, key_head, raw_q, raw_k, inverses);
+    __syncthreads();
+    const TokenScalars s = token_scalars(a, t, head);
+    const float iq = inverses[0], ik = inverses[1];
+    float previous[kRows], decayed[kRows], q[kRows], k[kRows];
+    float prediction = 0.0f;
+    const float dy = column_ok ? a.dcore[(1LL * t * a.vh + head) * a.vd + column] : 0.0f;
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) {
+      const int row = kg * kRows + r;
+      const bool ok = row < a.kd && column_ok;
+      const size_t at = (static_cast<size_t>(head) * a.kd + row) * a.vd + column;
+      previous[r] = ok ? a.states[t * stride + at] : 0.0f;
+      const float matrix = ok ? a.states[(t + 1) * stride + at] : 0.0f;
+      q[r] = raw_q[row] * iq / norm_scale;
+      k[r] = raw_k[row] * ik;
+      decayed[r] = previous[r] * s.decay;
+      prediction += decayed[r] * k[r];
+      // dq[row] = sum over columns of S_{t+1}[row, column] dy[column]
+      const float dq_row = half_wave_sum(matrix * dy);
+      if (c == 0) dq_rows[row] = dq_row;
+      dm[r] += q[r] * dy;
+    }
+    prediction = column_total(prediction, scratch, kg, c);
+    const float v = column_ok ? a.post[1LL * t * channels + 2 * a.kh * a.kd + head * a.vd + column] : 0.0f;
+    const float difference = v - prediction;
+    const float delta = difference * s.beta;
+    float ddelta = 0.0f;
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) ddelta += dm[r] * k[r];
+    ddelta = column_total(ddelta, scratch, kg, c);
+    const float dv = ddelta * s.beta;
+    if (kg == 0 && column_ok)
+      a.dpost[1LL * t * channels + 2 * a.kh * a.kd + head * a.vd + column] = dv;
+    float dg = 0.0f;
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) {
+      const int row = kg * kRows + r;
+      const float dk_row = half_wave_sum(dm[r] * delta - decayed[r] * dv);
+      if (c == 0) dk_rows[row] = dk_row;
+      const float ddecayed = dm[r] - k[r] * dv;
+      dg += ddecayed * previous[r];
+      dm[r] = ddecayed * s.decay;
+    }
+    // workgroup sums: dg over every element, d beta over the columns
+    float db_partial = kg == 0 ? ddelta * difference : 0.0f;
+    dg = wave_sum(dg);
+    db_partial = wave_sum(db_partial);
+    if (tid % 64 == 0) {
+      block_sums[wave][0] = dg;
+      block_sums[wave][1] = db_partial;
+    }
+    __syncthreads();
+    const long long partial = (1LL * t * a.vh + head) * tiles + tile;
+    if (tid < 64) {
+      // the two row-space gradients back through the L2 normalisation
+      float q_dot = 0.0f, k_dot = 0.0f;
+      for (int d = tid; d < kMaxKey; d += 64) {
+        q_dot += dq_rows[d] * raw_q[d];
+        k_dot += dk_rows[d] * raw_k[d];
+      }
+      q_dot = wave_sum(q_dot);
+      k_dot = wave_sum(k_dot);
+      for (int d = tid; d < a.kd; d += 64) {
+        a.qk_partials[partial * 2 * a.kd + d] =
+            (dq_rows[d] * iq - raw_q[d] * iq * iq * iq * q_dot) / norm_scale;
+        a.qk_partials[partial * 2 * a.kd + a.kd + d] =
+            dk_rows[d] * ik - raw_k[d] * ik * ik * ik * k_dot;
+      }
+      if (tid == 0) {
+        const float dg_total = (block_sums[0][0] + block_sums[1][0]) + (block_sums[2][0] + block_sums[3][0]);
+        const float db_total = (block_sums[0][1] + block_sums[1][1]) + (block_sums[2][1] + block_sums[3][1]);
+        a.scalar_partials[partial * 3 + 0] = -dg_total * s.decay * s.rate / (1.0f + expf(-s.alpha));
+        a.scalar_partials[partial * 3 + 1] = db_total * s.sigmoid * (1.0f - s.sigmoid);
+        a.scalar_partials[partial * 3 + 2] = -dg_total * s.decay * s.rate * s.softplus;
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// One wave per (token, head) row of value_dim <= 256 channels.
+__global__ void __launch_bounds__(64)
+output_backward_kernel(const float* core, const uint16_t* z, const float* __restrict__ norm,
+                       const float* dy, int vd, float epsilon, bool round, float* dcore,
+                       float* dz, float* norm_partials) {
+  const long long row = blockIdx.x;
+  const int lane = threadIdx.x;
+  float x[4], dn[4], gate[4], sigmoid[4], grad[4];
+  float squares = 0.0f, dot = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int c = lane + 64 * j;
+    x[j] = dn[j] = gate[j] = sigmoid[j] = grad[j] = 0.0f;
+    if (c < vd) {
+      x[j] = core[row * vd + c];
+      gate[j] = bf16_bits_to_float(z[row * vd + c]);
+      sigmoid[j] = 1.0f / (1.0f + expf(-gate[j]));
+      grad[j] = dy[row * vd + c];
+      dn[j] = grad[j] * gate[j] * sigmoid[j] * norm[c];
+    }
+    squares += x[j] * x[j];
+    dot += dn[j] * x[j];
+  }
+  squares = wave_sum(squares);
+  dot = wave_sum(dot);
+  const float inverse = rsqrtf(squares / static_cast<float>(vd) + epsilon);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int c = lane + 64 * j;
+    if (c >= vd) continue;
+    const float normalized = round_if(x[j] * inverse, round);
+    const float affine = round_if(normalized * norm[c], round);
+    dcore[row * vd + c] = inverse * dn[j] - x[j] * inverse * inverse * inverse / static_cast<float>(vd) * dot;
+    dz[row * vd + c] = grad[j] * affine * sigmoid[j] * (1.0f + gate[j] * (1.0f - sigmoid[j]));
+    if (norm_partials) norm_partials[row * vd + c] = grad[j] * gate[j] * sigmoid[j] * normalized;
+  }
+}
+
+// Heads of a key head and their column tiles add up, in ascending order.
+__global__ void __launch_bounds__(128)
+gather_qk_kernel(const float* partials, int kh, int vh, int kd, int tiles, int channels,
+                 float* dpost) {
+  const int key_head = blockIdx.x, t = blockIdx.y, d = threadIdx.x;
+  if (d >= kd) return;
+  const int group = vh / kh;
+  float dq = 0.0f, dk = 0.0f;
+  for (int h = key_head * group; h < (key_head + 1) * group; ++h)
+    for (int tile = 0; tile < tiles; ++tile) {
+      const long long at = ((1LL * t * vh + h) * tiles + tile) * 2 * kd;
+      dq += partials[at + d];
+      dk += partials[at + kd + d];
+    }
+  dpost[1LL * t * channels + key_head * kd + d] = dq;
+  dpost[1LL * t * channels + (kh + key_head) * kd + d] = dk;
+}
+
+// da, db per token; the two per-head parameter gradients summed over the
+// sequence by one workgroup per head in a fixed order.
+__global__ void __launch_bounds__(256)
+gather_scalar_kernel(const float* partials, int length, int vh, int tiles, float* da, float* db,
+                     float* da_log, float* ddt_bias) {
+  __shared__ float sums[256][2];
+  const int head = blockIdx.x, tid = threadIdx.x;
+  float log_sum = 0.0f, bias_sum = 0.0f;
+  for (int t = tid; t < length; t += 256) {
+    float ga = 0.0f, gb = 0.0f, glog = 0.0f;
+    for (int tile = 0; tile < tiles; ++tile) {
+      const long long at = ((1LL * t * vh + head) * tiles + tile) * 3;
+      ga += partials[at];
+      gb += partials[at + 1];
+      glog += partials[at + 2];
+    }
+    da[1LL * t * vh + head] = ga;
+    db[1LL * t * vh + head] = gb;
+    log_sum += glog;
+    bias_sum += ga;
+  }
+  sums[tid][0] = log_sum;
+  sums[tid][1] = bias_sum;
+  __syncthreads();
+  for (int width = 128; width > 0; width >>= 1) {
+    if (tid < width) {
+      sums[tid][0] += sums[tid + width][0];
+      sums[tid][1] += sums[tid + width][1];
+    }
+    __syncthreads();
+  }
+  if (tid == 0) {
+    if (da_log) da_log[head] += sums[0][0];
+    if (ddt_bias) ddt_bias[head] += sums[0][1];
+  }
+}
+
+__global__ void __launch_bounds__(256)
+conv_silu_backward_kernel(const float* pre, const float* dpost, long long elements, float* dpre) {
+  const long long i = blockIdx.x * 256LL + threadIdx.x;
+  if (i >= elements) return;
+  const float x = pre[i];
+  const float sigmoid = 1.0f / (1.0f + expf(-x));
+  dpre[i] = dpost[i] * sigmoid * (1.0f + x * (1.0f - sigmoid));
+}
+
+__global__ void __launch_bounds__(256)
+conv_input_backward_kernel(const float* dpre, const float* __restrict__ weight, int length,
+                           int channels, int kernel, float* dx) {
+  const long long i = blockIdx.x * 256LL + threadIdx.x;
+  if (i >= 1LL * length * channels) return;
+  const int c = static_cast<int>(i % channels), t = static_cast<int>(i / channels);
+  float sum = 0.0f;
+  for (int tap = 0; tap < kernel; ++tap) {
+    const int future = t + kernel - 1 - tap;
+    if (future < length) sum += dpre[1LL * future * channels + c] * weight[1LL * c * kernel + tap];
+  }
+  dx[i] = sum;
+}
+
+__global__ void __launch_bounds__(256)
+conv_weight_backward_kernel(const uint16_t* input, const float* dpre, int length, int channels,
+                            int kernel, float* dw) {
+  const int c = blockIdx.x * 256 + threadIdx.x, tap = blockIdx.y;
+  if (c >= channels) return;
+  float sum = 0.0f;
+  for (int t = kernel - 1 - tap; t < length; ++t)
+    sum += dpre[1LL * t * channels + c] *
+           bf16_bits_to_float(input[1LL * (t + tap - kernel + 1) * channels + c]);
+  dw[1LL * c * kernel + tap] += sum;
+}
+
+// gradient[c] += sum over rows of partials[row, c], two levels, fixed order.
+__global__ void __launch_bounds__(256)
+sum_rows_partial_kernel(const float* parts, long long rows, int width, int chunks, float* partial) {
+  const int c = threadIdx.x;
+  if (c >= width) return;
+  const long long per = (rows + chunks - 1) / chunks;
+  const long long first = blockIdx.x * per;
+  const long long last = first + per < rows ? first + per : rows;
+  float sum = 0.0f;
+  for (long long row = first; row < last; ++row) sum += parts[row * width + c];
+  partial[1LL * blockIdx.x * width + c] = sum;
+}
+
+__global__ void __launch_bounds__(256)
+sum_rows_final_kernel(const float* partial, int chunks, int width, float* gradient) {
+  const int c = threadIdx.x;
+  if (c >= width) return;
+  float sum = 0.0f;
+  for (int chunk = 0; chunk < chunks; ++chunk) sum += partial[1LL * chunk * width + c];
+  gradient[c] += sum;
+}
+
+unsigned blocks_for(long long elements) { return static_cast<unsigned>((elements + 255) / 256); }
+
+}  // namespace
+
+size_t gdn_backward_workspace_bytes(const pluto_hip_delta_params* p, int length, bool norm_grad) {
+  const size_t T = static_cast<size_t>(length);
+  const size_t kh = p->key_heads, vh = p->value_heads, kd = p->key_head_dim, vd = p->value_head_dim;
+  const size_t channels = 2 * kh * kd + vh * vd;
+  const size_t tiles = (vd + kColumns - 1) / kColumns;
+  size_t bytes = 0;
+  bytes += 4 * align_up(T * channels * 4, 256);          // pre, post, dpost, dpre
+  bytes += 2 * align_up(T * vh * vd * 4, 256);           // core, dcore
+  bytes += align_up((T + 1) * vh * kd * vd * 4, 256);    // states
+  bytes += align_up(T * vh * tiles * 2 * kd * 4, 256);   // q/k partials
+  bytes += align_up(T * vh * tiles * 3 * 4, 256);        // scalar partials
+  if (norm_grad) bytes += align_up(T * vh * vd * 4, 256) + align_up(kGdnSumChunks * vd * 4, 256);
+  return bytes;
+}
+
+int launch_gdn_backward(hipStream_t stream, const pluto_hip_delta_params* p, int length,
+                        const void* qkv, const void* z, const void* a, const void* b,
+                        const float* conv_weight, const float* a_log, const float* dt_bias,
+                        const float* norm, const float* dy, float* dqkv, float* dz, float* da,
+                        float* db, float* d_conv_weight, float* d_a_log, float* d_dt_bias,
+                        float* d_norm, void* workspace) {
+  const size_t T = static_cast<size_t>(length);
+  const int kh = p->key_heads, vh = p->value_heads, kd = p->key_head_dim, vd = p->value_head_dim;
+  const int channels = 2 * kh * kd + vh * vd, kernel = p->conv_kernel_dim;
+  const int tiles = (vd + kColumns - 1) / kColumns;
+  const bool round = p->round_to_bfloat16 != 0;
+  char* at = static_cast<char*>(workspace);
+  auto take = [&](size_t bytes) {
+    char* result = at;
+    at += align_up(bytes, 256);
+    return reinterpret_cast<float*>(result);
+  };
+  float* pre = take(T * channels * 4);
+  float* post = take(T * channels * 4);
+  float* dpost = take(T * channels * 4);
+  float* dpre = take(T * channels * 4);
+  float* core = take(T * vh * vd * 4);
+  float* dcore = take(T * vh * vd * 4);
+  float* states = take((T + 1) * vh * kd * vd * 4);
+  float* qk_partials = take(T * vh * tiles * 2 * kd * 4);
+  float* scalar_partials = take(T * vh * tiles * 3 * 4);
+  float* norm_partials = d_norm ? take(T * vh * vd * 4) : nullptr;
+  float* norm_chunks = d_norm ? take(static_cast<size_t>(kGdnSumChunks) * vd * 4) : nullptr;
+
+  const long long elements = 1LL * length * channels;
+  conv_train_kernel<<<blocks_for(elements), 256, 0, stream>>>(
+      static_cast<const uint16_t*>(qkv), conv_weight, length, channels, kernel, round, pre, post);
+  int status = launch_status();
+  if (status != 0) return status;
+  RecurrenceArgs r;
+  r.post = post;
+  r.a = static_cast<const uint16_t*>(a);
+  r.b = static_cast<const uint16_t*>(b);
+  r.a_log = a_log;
+  r.dt_bias = dt_bias;
+  r.states = states;
+  r.core = core;
+  r.dcore = dcore;
+  r.qk_partials = qk_partials;
+  r.scalar_partials = scalar_partials;
+  r.dpost = dpost;
+  r.length = length;
+  r.kh = kh;
+  r.vh = vh;
+  r.kd = kd;
+  r.vd = vd;
+  r.round = round;
+  recurrence_states_kernel<<<vh * tiles, 256, 0, stream>>>(r);
+  status = launch_status();
+  if (status != 0) return status;
+  output_backward_kernel<<<static_cast<unsigned>(length) * vh, 64, 0, stream>>>(
+      core, static_cast<const uint16_t*>(z), norm, dy, vd, p->rms_norm_epsilon, round, dcore, dz,
+      norm_partials);
+  status = launch_status();
+  if (status != 0) return status;
+  if (d_norm) {
+    sum_rows_partial_kernel<<<kGdnSumChunks, 256, 0, stream>>>(norm_partials, 1LL * length * vh, vd,
+                                                               kGdnSumChunks, norm_chunks);
+    sum_rows_final_kernel<<<1, 256, 0, stream>>>(norm_chunks, kGdnSumChunks, vd, d_norm);
+    status = launch_status();
+    if (status != 0) return status;
+  }
+  recurrence_backward_kernel<<<vh * tiles, 256, 0, stream>>>(r);
+  status = launch_status();
+  if (status != 0) return status;
+  gather_qk_kernel<<<dim3(kh, length), 128, 0, stream>>>(qk_partials, kh, vh, kd, tiles, channels,
+                                                         dpost);
+  gather_scalar_kernel<<<vh, 256, 0, stream>>>(scalar_partials, length, vh, tiles, da, db, d_a_log,
+                                               d_dt_bias);
+  conv_silu_backward_kernel<<<blocks_for(elements), 256, 0, stream>>>(pre, dpost, elements, dpre);
+  conv_input_backward_kernel<<<blocks_for(elements), 256, 0, stream>>>(dpre, conv_weight, length,
+                                                                      channels, kernel, dqkv);
+  if (d_conv_weight)
+    conv_weight_backward_kernel<<<dim3((channels + 255) / 256, kernel), 256, 0, stream>>>(
+        static_cast<const uint16_t*>(qkv), dpre, length, channels, kernel, d_conv_weight);
+  return launch_status();
+}
+
+}  // namespace pluto_hip

@@ -187,6 +187,48 @@ int pluto_hip_gdn_layer_forward(void* stream, const pluto_hip_delta_params* p, i
                            p->rms_norm_epsilon, round, out, PLUTO_HIP_BF16);
 }
 
+size_t pluto_hip_gdn_layer_backward_workspace_bytes(const pluto_hip_delta_params* p, int length,
+                                                    int norm_grad) {
+  if (validate_delta(p) != 0 || length <= 0 || length > 65535) return 0;
+  return gdn_backward_workspace_bytes(p, length, norm_grad != 0);
+}
+
+int pluto_hip_gdn_layer_backward(void* stream, const pluto_hip_delta_params* p, int batch,
+                                 int length, const void* qkv, const void* z, const void* a,
+                                 const void* b, const float* conv_weight, const float* a_log,
+                                 const float* dt_bias, const float* norm, const float* dy,
+                                 float* dqkv, float* dz, float* da, float* db,
+                                 float* d_conv_weight, float* d_a_log, float* d_dt_bias,
+                                 float* d_norm, void* workspace, size_t workspace_bytes) {
+  int status = validate_delta(p);
+  if (status != 0) return status;
+  // the q/k gather runs one grid row per token
+  if (batch <= 0 || length <= 0 || length > 65535) return PLUTO_HIP_EINVAL;
+  if (!qkv || !z || !a || !b || !conv_weight || !a_log || !dt_bias || !norm || !dy || !dqkv ||
+      !dz || !da || !db)
+    return PLUTO_HIP_EINVAL;
+  const size_t needed = gdn_backward_workspace_bytes(p, length, d_norm != nullptr);
+  if (!workspace || workspace_bytes < needed) return PLUTO_HIP_EWORKSPACE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const size_t channels =
+      2ull * p->key_heads * p->key_head_dim + 1ull * p->value_heads * p->value_head_dim;
+  const size_t width = 1ull * p->value_heads * p->value_head_dim, heads = p->value_heads;
+  const size_t T = static_cast<size_t>(length);
+  // Sequences are independent and share the scratch: they run one after the
+  // other on the stream; parameter gradients accumulate over all of them.
+  for (int sequence = 0; sequence < batch; ++sequence) {
+    const size_t at = static_cast<size_t>(sequence) * T;
+    status = launch_gdn_backward(
+        s, p, length, static_cast<const uint16_t*>(qkv) + at * channels,
+        static_cast<const uint16_t*>(z) + at * width, static_cast<const uint16_t*>(a) + at * heads,
+        static_cast<const uint16_t*>(b) + at * heads, conv_weight, a_log, dt_bias, norm,
+        dy + at * width, dqkv + at * channels, dz + at * width, da + at * heads, db + at * heads,
+        d_conv_weight, d_a_log, d_dt_bias, d_norm, workspace);
+    if (status != 0) return status;
+  }
+  return 0;
+}
+
 size_t pluto_hip_gdn_step_workspace_bytes(const pluto_hip_delta_params* p) {
   if (validate_delta(p) != 0) return 0;
   const size_t channels = 2 * static_cast<size_t>(p->key_heads) * p->key_head_dim +
