@@ -45,8 +45,8 @@ MEASURED_TRAFFIC_BYTES = {
 NAMES = ["mha_train_bf16", "mha_fwd_fp32", "gqa_prefill", "gqa_decode", "gdn_scan"]
 # "copy" is a plain device copy of known size: the calibration case for the
 # FETCH_SIZE / WRITE_SIZE counters that `roofline.traffic` is derived from.
-# "gqa_prefill_bwd" times the Qwen sequence backward on its own.
-EXTRA = ["copy", "gqa_prefill_bwd"]
+# "gqa_prefill_bwd" and "gdn_layer_bwd" time the two sequence backward passes.
+EXTRA = ["copy", "gqa_prefill_bwd", "gdn_layer_bwd"]
 
 
 def parse_args():
@@ -177,6 +177,39 @@ def gqa_prefill_bwd(torch, capi):
                 cpu=None)
 
 
+def gdn_layer_bwd(torch, capi):
+    """Backward of the gated delta-net layer (token-serial FP32 kernels that keep
+    one state per token): a row after the headline ones, not part of --workload all."""
+    import numpy as np
+    B, T, H, dk, dv, K = 1, 2048, 16, 128, 128, 4
+    p = capi.delta_params(H, H, dk, dv, K)
+    channels = 2 * H * dk + H * dv
+    gen = torch.Generator(device="cuda").manual_seed(4)
+    bf = torch.bfloat16
+    qkv = torch.randn((B, T, channels), generator=gen, device="cuda").to(bf)
+    z = torch.randn((B, T, H * dv), generator=gen, device="cuda").to(bf)
+    a = torch.randn((B, T, H), generator=gen, device="cuda").to(bf)
+    b = torch.randn((B, T, H), generator=gen, device="cuda").to(bf)
+    conv = 0.5 * torch.randn((channels, K), generator=gen, device="cuda")
+    a_log = torch.zeros(H, device="cuda")
+    dt_bias = torch.zeros(H, device="cuda")
+    norm = torch.ones(dv, device="cuda")
+    dy = torch.randn((B, T, H * dv), generator=gen, device="cuda")
+
+    def step():
+        capi.gdn_layer_backward(p, qkv, z, a, b, conv, a_log, dt_bias, norm, dy)
+
+    # every per-token state is written once and read twice (as S_t and as S_{t+1})
+    work = 3.0 * B * (T + 1) * H * dk * dv * 4
+    return dict(step=step, parts=[("backward", step, work)], work=work,
+                metric="gdn_layer_backward_hbm_gbs", unit="GB/s", dtype="f32", bound="hbm",
+                peak=PEAK_HBM_GBS,
+                config={"workload": "gated_delta_net_layer_backward", "batch": B, "seq_len": T,
+                        "heads": H, "d_k": dk, "d_v": dv, "conv_kernel": K,
+                        "counted": "per-token state traffic (1 write + 2 reads)"},
+                cpu=None)
+
+
 def gqa_decode(torch, capi):
     import numpy as np
     batch, qh, kh, d, capacity = 32, 24, 4, 128, 32768
@@ -260,7 +293,8 @@ def copy(torch, capi):
 
 
 WORKLOADS = {"copy": copy, "mha_train_bf16": mha_train_bf16, "mha_fwd_fp32": mha_fwd_fp32,
-             "gqa_prefill": gqa_prefill, "gqa_prefill_bwd": gqa_prefill_bwd, "gqa_decode": gqa_decode,
+             "gqa_prefill": gqa_prefill, "gqa_prefill_bwd": gqa_prefill_bwd, "gdn_layer_bwd": gdn_layer_bwd,
+             "gqa_decode": gqa_decode,
              "gdn_scan": gdn_scan}
 
 

@@ -24,6 +24,9 @@
  *                            check, qwen_attention_test.cc:22-99,230-300, at
  *                            its bound of 3e-5, both rounding modes) and
  *                            float64 autograd of the unrounded layer.
+ *   gdn_sequence_backward    the same two checks (frozen-rounding finite
+ *                            differences at 3e-5, float64 autograd) for all
+ *                            four inputs and four parameters.
  *   gdn_*                    textbook delta rule special cases (beta=0, g=0
  *                            with orthonormal keys), softplus extremes,
  *                            independent float64 numpy recurrence.

@@ -190,10 +190,28 @@ recurrence_backward_kernel(RecurrenceArgs a) {
   const size_t stride = static_cast<size_t>(a.vh) * a.kd * a.vd;
   const float norm_scale = sqrtf(static_cast<float>(a.kd));
   float dm[kRows];
+  // S_{t+1} of a token is S_t of the token processed just before it, and S_t is
+  // requested one token ahead: no load of a state is waited for inside a token.
+  float after[kRows], before[kRows];
 #pragma unroll
-  for (int r = 0; r < kRows; ++r) dm[r] = 0.0f;
+  for (int r = 0; r < kRows; ++r) {
+    dm[r] = 0.0f;
+    const int row = kg * kRows + r;
+    const bool ok = row < a.kd && column_ok;
+    const size_t at = (static_cast<size_t>(head) * a.kd + row) * a.vd + column;
+    after[r] = ok ? a.states[a.length * stride + at] : 0.0f;
+    before[r] = ok ? a.states[(a.length - 1) * stride + at] : 0.0f;
+  }
   for (int t = a.length - 1; t >= 0; --t) {
     load_token_qk(a, t, key_head, raw_q, raw_k, inverses);
+    float ahead[kRows];
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) {
+      const int row = kg * kRows + r;
+      const bool ok = row < a.kd && column_ok && t > 0;
+      ahead[r] = ok ? a.states[(t - 1) * stride + (static_cast<size_t>(head) * a.kd + row) * a.vd + column]
+                    : 0.0f;
+    }
     __syncthreads();
     const TokenScalars s = token_scalars(a, t, head);
     const float iq = inverses[0], ik = inverses[1];
@@ -203,10 +221,8 @@ recurrence_backward_kernel(RecurrenceArgs a) {
 #pragma unroll
     for (int r = 0; r < kRows; ++r) {
       const int row = kg * kRows + r;
-      const bool ok = row < a.kd && column_ok;
-      const size_t at = (static_cast<size_t>(head) * a.kd + row) * a.vd + column;
-      previous[r] = ok ? a.states[t * stride + at] : 0.0f;
-      const float matrix = ok ? a.states[(t + 1) * stride + at] : 0.0f;
+      previous[r] = before[r];
+      const float matrix = after[r];
       q[r] = raw_q[row] * iq / norm_scale;
       k[r] = raw_k[row] * ik;
       decayed[r] = previous[r] * s.decay;
@@ -236,6 +252,8 @@ recurrence_backward_kernel(RecurrenceArgs a) {
       const float ddecayed = dm[r] - k[r] * dv;
       dg += ddecayed * previous[r];
       dm[r] = ddecayed * s.decay;
+      after[r] = before[r];
+      before[r] = ahead[r];
     }
     // workgroup sums: dg over every element, d beta over the columns
     float db_partial = kg == 0 ? ddelta * difference : 0.0f;

@@ -98,12 +98,63 @@ StatusOr<FwdResult> SequenceDeltaNetLayer::fwd_impl(hip::Executor& executor,
   return FwdResult{{std::move(output)}, std::move(state)};
 }
 
-// The reference differentiates through the whole history
-// (sequence_delta_net.cc:482-600); that kernel chain is not part of this library.
-StatusOr<BufferVec> SequenceDeltaNetLayer::bwd_impl(hip::Executor&, Span<const Buffer>,
-                                                    BackwardState, LayerHooks*) {
-  return UnimplementedError(
-      "SequenceDeltaNetLayer backward is not implemented by the MI355X attention path");
+// src/llm/layers/sequence_delta_net.cc:482-561.  The library's backward entry
+// repeats the forward pass itself (keeping every per-token state in its
+// workspace, as the reference's saved state does), so the saved state only
+// supplies the four input handles.
+StatusOr<BufferVec> SequenceDeltaNetLayer::bwd_impl(hip::Executor& executor,
+                                                    Span<const Buffer> gradients,
+                                                    BackwardState state, LayerHooks*) {
+  if (&executor != &executor_ || gradients.size() != 1 || state.intermediates.size() != 5)
+    return InvalidArgumentError("invalid DeltaNet backward state or gradient");
+  const auto& p = parameters_;
+  const int t = sequence_length_;
+  if (t > kMaximumBackwardLength)
+    return UnimplementedError(
+        "SequenceDeltaNetLayer backward keeps one state per token and supports T<=65535");
+  const size_t channels =
+      2ull * p.key_heads * p.key_head_dim + 1ull * p.value_heads * p.value_head_dim;
+  const size_t output_width = 1ull * p.value_heads * p.value_head_dim;
+  const size_t rows = static_cast<size_t>(t);
+  const auto& saved = state.intermediates;
+  const size_t expected[] = {rows * channels * 2, rows * output_width * 2, rows * p.value_heads * 2,
+                             rows * p.value_heads * 2};
+  if (&gradients[0].executor() != &executor ||
+      gradients[0].size_bytes() != rows * output_width * sizeof(float))
+    return InvalidArgumentError(
+        "SequenceDeltaNetLayer requires batch-one buffers of the declared sequence shape on its "
+        "Executor");
+  for (int i = 0; i < 4; ++i)
+    if (&saved[i].executor() != &executor || saved[i].size_bytes() != expected[i])
+      return InvalidArgumentError(
+          "SequenceDeltaNetLayer requires batch-one buffers of the declared sequence shape on its "
+          "Executor");
+  ASSIGN_OR_RETURN(auto dqkv, Buffer::Allocate(executor, rows * channels * sizeof(float)));
+  ASSIGN_OR_RETURN(auto dz, Buffer::Allocate(executor, rows * output_width * sizeof(float)));
+  ASSIGN_OR_RETURN(auto da, Buffer::Allocate(executor, rows * p.value_heads * sizeof(float)));
+  ASSIGN_OR_RETURN(auto db, Buffer::Allocate(executor, rows * p.value_heads * sizeof(float)));
+  const pluto_hip_delta_params abi = cached_attention_ops::ToAbi(p);
+  auto active_gradient = [](const std::shared_ptr<BlockParameter>& parameter) -> float* {
+    return parameter->active() ? static_cast<float*>(parameter->gradient().data()) : nullptr;
+  };
+  float* const d_norm = active_gradient(parameters_owned_[3]);
+  const size_t workspace_bytes =
+      pluto_hip_gdn_layer_backward_workspace_bytes(&abi, t, d_norm != nullptr);
+  ASSIGN_OR_RETURN(auto workspace, Buffer::Allocate(executor, workspace_bytes));
+  RETURN_IF_ERROR(hip::HipStatus(
+      pluto_hip_gdn_layer_backward(
+          executor.stream(), &abi, 1, t, saved[0].data(), saved[1].data(), saved[2].data(),
+          saved[3].data(), static_cast<const float*>(weights_[0].data()),
+          static_cast<const float*>(weights_[1].data()),
+          static_cast<const float*>(weights_[2].data()),
+          static_cast<const float*>(weights_[3].data()),
+          static_cast<const float*>(gradients[0].data()), static_cast<float*>(dqkv.data()),
+          static_cast<float*>(dz.data()), static_cast<float*>(da.data()),
+          static_cast<float*>(db.data()), active_gradient(parameters_owned_[0]),
+          active_gradient(parameters_owned_[1]), active_gradient(parameters_owned_[2]), d_norm,
+          workspace.data(), workspace_bytes),
+      "sequence DeltaNet backward"));
+  return BufferVec{std::move(dqkv), std::move(dz), std::move(da), std::move(db)};
 }
 
 }  // namespace pluto::llm

@@ -5,8 +5,9 @@
 // BF16 [1,T,V].  QKV packs all Q, then all K, then all V.  The forward pass
 // runs the chunked (64-token) matrix-core scan instead of a token loop, so any
 // sequence length up to kMaximumSequenceLength is accepted (the reference
-// stops at 128); the per-token state snapshots the reference keeps for its
-// backward pass are not produced, and backward reports Unimplemented.
+// stops at 128).  The per-token state snapshots the reference keeps for its
+// backward pass are not produced by forward: backward repeats the forward pass
+// token by token and keeps them in its own scratch.
 #pragma once
 
 #include <memory>
@@ -20,6 +21,8 @@ namespace pluto::llm {
 class SequenceDeltaNetLayer final : public Layer {
  public:
   static constexpr int kMaximumSequenceLength = 1 << 20;
+  // bwd keeps one recurrent state per token in scratch (as the reference does)
+  static constexpr int kMaximumBackwardLength = 65535;
 
   // Convolution is [QKV,kernel], A_log and dt_bias are [value_heads], and
   // norm is [value_head_dim], a plain multiplier rather than 1 + weight.

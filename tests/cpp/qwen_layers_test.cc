@@ -598,7 +598,8 @@ void SequenceMatchesOracleAndCachedTokens(DeltaNetParameters p, int length) {
     const auto got = Read<BFloat16>(forward->outputs[0]);
     if (repetition == 0) first = got;
     EXPECT_TRUE(got == first);
-    EXPECT_TRUE(IsUnimplemented(
+    // a gradient of the wrong type/size is rejected before any work
+    EXPECT_TRUE(IsInvalidArgument(
         (*sequence)->bwd(*executor, {*dz}, std::move(forward->state)).status()));
   }
   double scale = 0;
@@ -624,6 +625,106 @@ void SequenceMatchesOracleAndCachedTokens(DeltaNetParameters p, int length) {
     }
     ASSERT_TRUE((*cached)->Reset().ok());
   }
+}
+
+void BackwardMatchesOracle(DeltaNetParameters p, int length, bool rounding) {
+  // sequence_delta_net_test.cc:299-380: every input and parameter gradient; the
+  // oracle's backward is itself pinned by finite differences.
+  p.round_to_bfloat16 = rounding;
+  auto executor = NewExecutor();
+  const int channels = 2 * p.key_heads * p.key_head_dim + p.value_heads * p.value_head_dim;
+  const int width = p.value_heads * p.value_head_dim;
+  const auto qkv = RoundedToBFloat16(Values(static_cast<size_t>(length) * channels, .1));
+  const auto z = RoundedToBFloat16(Values(static_cast<size_t>(length) * width, 1.1));
+  const auto a = RoundedToBFloat16(Values(static_cast<size_t>(length) * p.value_heads, 2.1));
+  const auto b = RoundedToBFloat16(Values(static_cast<size_t>(length) * p.value_heads, 3.1));
+  const auto conv = Values(static_cast<size_t>(channels) * p.conv_kernel_dim, .3, .5);
+  const auto a_log = Values(p.value_heads, .5, .4), dt_bias = Values(p.value_heads, .7, .3);
+  auto norm = Values(p.value_head_dim, .9, .2);
+  for (float& value : norm) value += 1.0f;
+  const auto upstream = Values(static_cast<size_t>(length) * width, .7);
+  const pluto_hip_delta_params abi = cached_attention_ops::ToAbi(p);
+  pluto_oracle_delta_params oracle_p;
+  std::memcpy(&oracle_p, &abi, sizeof(abi));
+  std::vector<std::vector<float>> want = {
+      std::vector<float>(qkv.size()),  std::vector<float>(z.size()),
+      std::vector<float>(a.size()),    std::vector<float>(b.size()),
+      std::vector<float>(conv.size(), 0.f), std::vector<float>(a_log.size(), 0.f),
+      std::vector<float>(dt_bias.size(), 0.f), std::vector<float>(norm.size(), 0.f)};
+  ASSERT_EQ(pluto_oracle_gdn_sequence_backward(
+                &oracle_p, length, qkv.data(), z.data(), a.data(), b.data(), conv.data(),
+                a_log.data(), dt_bias.data(), norm.data(), upstream.data(), want[0].data(),
+                want[1].data(), want[2].data(), want[3].data(), want[4].data(), want[5].data(),
+                want[6].data(), want[7].data()),
+            0);
+  std::shared_ptr<BlockParameter> parameters[4];
+  const std::vector<float>* weights[] = {&conv, &a_log, &dt_bias, &norm};
+  for (int i = 0; i < 4; ++i) {
+    auto parameter = Parameter(*executor, *weights[i]);
+    ASSERT_TRUE(parameter.ok());
+    parameters[i] = *parameter;
+    ASSERT_TRUE(parameters[i]->Activate().ok());
+  }
+  auto layer = SequenceDeltaNetLayer::Create(*executor, p, parameters[0], parameters[1],
+                                             parameters[2], parameters[3], length);
+  ASSERT_TRUE(layer.ok());
+  auto dqkv = Upload<BFloat16>(*executor, qkv), dz = Upload<BFloat16>(*executor, z),
+       da = Upload<BFloat16>(*executor, a), db = Upload<BFloat16>(*executor, b);
+  auto dy = Upload<float>(*executor, upstream);
+  std::vector<std::vector<float>> first;
+  for (int call = 0; call < 2; ++call) {
+    auto forward = (*layer)->fwd(*executor, {*dqkv, *dz, *da, *db});
+    ASSERT_TRUE(forward.ok());
+    auto backward = (*layer)->bwd(*executor, {*dy}, std::move(forward->state));
+    ASSERT_TRUE(backward.ok());
+    ASSERT_EQ(backward->size(), 4u);
+    std::vector<std::vector<float>> actual;
+    for (const auto& gradient : *backward) actual.push_back(Read<float>(gradient));
+    for (int i = 0; i < 4; ++i) actual.push_back(Read<float>(parameters[i]->gradient()));
+    if (call == 0) {
+      first = actual;
+      for (size_t which = 0; which < want.size(); ++which) {
+        ASSERT_EQ(actual[which].size(), want[which].size());
+        double scale = 0;
+        for (float value : want[which]) scale = std::max(scale, std::fabs(double(value)));
+        // FP32 token-serial arithmetic against the double-precision oracle; with
+        // rounding, operands that straddle a bf16 tie differ by one ulp
+        const double bound = (rounding ? 1e-2 : 2e-4) * scale + 1e-6;
+        for (size_t i = 0; i < want[which].size(); ++i)
+          EXPECT_NEAR(actual[which][i], want[which][i], bound);
+      }
+    } else {
+      // activation gradients repeat bit for bit, parameter gradients accumulate
+      for (int which = 0; which < 4; ++which) EXPECT_TRUE(actual[which] == first[which]);
+      for (int which = 4; which < 8; ++which)
+        for (size_t i = 0; i < actual[which].size(); ++i)
+          EXPECT_NEAR(actual[which][i], 2 * first[which][i], 1e-5 * (1 + std::fabs(first[which][i])));
+    }
+  }
+  // frozen parameters: the activation gradients are the same, nothing accumulates
+  for (auto& parameter : parameters) ASSERT_TRUE(parameter->Deactivate().ok());
+  auto forward = (*layer)->fwd(*executor, {*dqkv, *dz, *da, *db});
+  ASSERT_TRUE(forward.ok());
+  auto state_copy = forward->state;
+  auto backward = (*layer)->bwd(*executor, {*dy}, std::move(forward->state));
+  ASSERT_TRUE(backward.ok());
+  for (int which = 0; which < 4; ++which)
+    EXPECT_TRUE(Read<float>((*backward)[which]) == first[which]);
+  state_copy.intermediates.pop_back();
+  EXPECT_TRUE(IsInvalidArgument((*layer)->bwd(*executor, {*dy}, std::move(state_copy)).status()));
+}
+
+TEST(SequenceDeltaNetTest, BackwardMatchesOracleOnSmallOddShape) {
+  for (bool rounding : {false, true}) BackwardMatchesOracle(SmallDelta(), 9, rounding);
+}
+
+TEST(SequenceDeltaNetTest, BackwardMatchesOracleOnFullWidthHeads) {
+  DeltaNetParameters p;
+  p.key_heads = 1;
+  p.value_heads = 2;
+  p.key_head_dim = 128;
+  p.value_head_dim = 128;
+  BackwardMatchesOracle(p, 70, true);
 }
 
 TEST(SequenceDeltaNetTest, SmallOddShapeMatchesOracleAndCachedTokenInference) {
