@@ -18,7 +18,9 @@
 // [key_dim, 32] slice of one head's state (as the reference's programs do),
 // thread (kg, c) = (tid / 32, tid % 32) holds rows 16 kg .. 16 kg + 15 of
 // column c in registers.  Sums over rows go through LDS (8 partials a column),
-// sums over columns through lane shuffles within a 32-lane half.
+// sums over columns through LDS as well (one padded row of products per state
+// row, added up by one thread per row).  What a token reads from global memory
+// is requested one token ahead.
 #include "gdn.h"
 
 namespace pluto_hip {
@@ -69,35 +71,62 @@ struct TokenScalars {
   float alpha, softplus, rate, decay, sigmoid, beta;
 };
 
-__device__ inline TokenScalars token_scalars(const RecurrenceArgs& a, int t, int head) {
+// What a thread reads from global memory for one token.  It is requested one
+// token ahead, so that the sequential chain never waits for these loads.
+struct TokenInputs {
+  float q[2], k[2];   // wave 0: raw q and k channels lane and lane + 64
+  float a, b;         // the head's gate logits
+  float v, dy;        // this thread's value column and (backward) its gradient
+};
+
+__device__ inline TokenInputs fetch_token(const RecurrenceArgs& a, int t, int head, int key_head,
+                                          int column, bool column_ok, bool with_gradient) {
+  TokenInputs in;
+  const int channels = 2 * a.kh * a.kd + a.vh * a.vd;
+  const int tid = threadIdx.x;
+  in.q[0] = in.q[1] = in.k[0] = in.k[1] = 0.0f;
+  if (tid < 64) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int d = tid + 64 * j;
+      if (d < a.kd) {
+        in.q[j] = a.post[1LL * t * channels + key_head * a.kd + d];
+        in.k[j] = a.post[1LL * t * channels + (a.kh + key_head) * a.kd + d];
+      }
+    }
+  }
+  in.a = bf16_bits_to_float(a.a[1LL * t * a.vh + head]);
+  in.b = bf16_bits_to_float(a.b[1LL * t * a.vh + head]);
+  in.v = column_ok ? a.post[1LL * t * channels + 2 * a.kh * a.kd + head * a.vd + column] : 0.0f;
+  in.dy = (with_gradient && column_ok) ? a.dcore[(1LL * t * a.vh + head) * a.vd + column] : 0.0f;
+  return in;
+}
+
+__device__ inline TokenScalars token_scalars(const RecurrenceArgs& a, const TokenInputs& in,
+                                             int head) {
   TokenScalars s;
-  s.alpha = bf16_bits_to_float(a.a[1LL * t * a.vh + head]) + a.dt_bias[head];
+  s.alpha = in.a + a.dt_bias[head];
   s.softplus = fmaxf(s.alpha, 0.0f) + logf(1.0f + expf(-fabsf(s.alpha)));
   s.rate = expf(a.a_log[head]);
   s.decay = expf(-s.rate * s.softplus);
-  s.sigmoid = 1.0f / (1.0f + expf(-bf16_bits_to_float(a.b[1LL * t * a.vh + head])));
+  s.sigmoid = 1.0f / (1.0f + expf(-in.b));
   s.beta = round_if(s.sigmoid, a.round);
   return s;
 }
 
-// Raw q and k of one token into LDS together with 1/|q|, 1/|k| (1e-6 added to
+// Raw q and k of the token into LDS together with 1/|q|, 1/|k| (1e-6 added to
 // the sums of squares, sequence_delta_net.cc:84-85).
-__device__ inline void load_token_qk(const RecurrenceArgs& a, int t, int key_head, float* raw_q,
-                                     float* raw_k, float* inverses) {
-  const int channels = 2 * a.kh * a.kd + a.vh * a.vd;
+__device__ inline void publish_token_qk(const TokenInputs& in, float* raw_q, float* raw_k,
+                                        float* inverses) {
   const int tid = threadIdx.x;
   if (tid < 64) {
     float qq = 0.0f, kk = 0.0f;
-    for (int d = tid; d < kMaxKey; d += 64) {
-      float qv = 0.0f, kv = 0.0f;
-      if (d < a.kd) {
-        qv = a.post[1LL * t * channels + key_head * a.kd + d];
-        kv = a.post[1LL * t * channels + (a.kh + key_head) * a.kd + d];
-      }
-      raw_q[d] = qv;
-      raw_k[d] = kv;
-      qq += qv * qv;
-      kk += kv * kv;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      raw_q[tid + 64 * j] = in.q[j];
+      raw_k[tid + 64 * j] = in.k[j];
+      qq += in.q[j] * in.q[j];
+      kk += in.k[j] * in.k[j];
     }
     qq = wave_sum(qq);
     kk = wave_sum(kk);
@@ -117,12 +146,6 @@ __device__ inline float column_total(float partial, float (*scratch)[kColumns], 
   for (int g = 0; g < kGroups; ++g) total += scratch[g][c];
   __syncthreads();
   return total;
-}
-
-__device__ inline float half_wave_sum(float v) {
-#pragma unroll
-  for (int offset = 16; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, 64);
-  return v;
 }
 
 __global__ void __launch_bounds__(256)
@@ -145,10 +168,13 @@ recurrence_states_kernel(RecurrenceArgs a) {
     const int row = kg * kRows + r;
     if (row < a.kd && column_ok) a.states[(static_cast<size_t>(head) * a.kd + row) * a.vd + column] = 0.0f;
   }
+  TokenInputs next = fetch_token(a, 0, head, key_head, column, column_ok, false);
   for (int t = 0; t < a.length; ++t) {
-    load_token_qk(a, t, key_head, raw_q, raw_k, inverses);
+    const TokenInputs in = next;
+    if (t + 1 < a.length) next = fetch_token(a, t + 1, head, key_head, column, column_ok, false);
+    publish_token_qk(in, raw_q, raw_k, inverses);
     __syncthreads();
-    const TokenScalars s = token_scalars(a, t, head);
+    const TokenScalars s = token_scalars(a, in, head);
     const float iq = inverses[0], ik = inverses[1];
     float prediction = 0.0f;
 #pragma unroll
@@ -157,8 +183,7 @@ recurrence_states_kernel(RecurrenceArgs a) {
       prediction += m[r] * (raw_k[kg * kRows + r] * ik);
     }
     prediction = column_total(prediction, scratch, kg, c);
-    const float v = column_ok ? a.post[1LL * t * channels + 2 * a.kh * a.kd + head * a.vd + column] : 0.0f;
-    const float delta = (v - prediction) * s.beta;
+    const float delta = (in.v - prediction) * s.beta;
     float out = 0.0f;
 #pragma unroll
     for (int r = 0; r < kRows; ++r) {
@@ -179,6 +204,10 @@ recurrence_backward_kernel(RecurrenceArgs a) {
   __shared__ float scratch[kGroups][kColumns];
   __shared__ float dq_rows[kMaxKey], dk_rows[kMaxKey];
   __shared__ float block_sums[4][3];
+  // per-element products whose sums over the 32 columns give dq and dk: one
+  // padded row per state row, summed by one thread per row (a lane shuffle
+  // tree per row costs a multiple of this)
+  __shared__ float q_products[kMaxKey][kColumns + 1], k_products[kMaxKey][kColumns + 1];
   const int tiles = (a.vd + kColumns - 1) / kColumns;
   const int head = blockIdx.x / tiles, tile = blockIdx.x % tiles;
   const int key_head = head / (a.vh / a.kh);
@@ -202,8 +231,11 @@ recurrence_backward_kernel(RecurrenceArgs a) {
     after[r] = ok ? a.states[a.length * stride + at] : 0.0f;
     before[r] = ok ? a.states[(a.length - 1) * stride + at] : 0.0f;
   }
+  TokenInputs next = fetch_token(a, a.length - 1, head, key_head, column, column_ok, true);
   for (int t = a.length - 1; t >= 0; --t) {
-    load_token_qk(a, t, key_head, raw_q, raw_k, inverses);
+    const TokenInputs in = next;
+    if (t > 0) next = fetch_token(a, t - 1, head, key_head, column, column_ok, true);
+    publish_token_qk(in, raw_q, raw_k, inverses);
     float ahead[kRows];
 #pragma unroll
     for (int r = 0; r < kRows; ++r) {
@@ -213,11 +245,11 @@ recurrence_backward_kernel(RecurrenceArgs a) {
                     : 0.0f;
     }
     __syncthreads();
-    const TokenScalars s = token_scalars(a, t, head);
+    const TokenScalars s = token_scalars(a, in, head);
     const float iq = inverses[0], ik = inverses[1];
     float previous[kRows], decayed[kRows], q[kRows], k[kRows];
     float prediction = 0.0f;
-    const float dy = column_ok ? a.dcore[(1LL * t * a.vh + head) * a.vd + column] : 0.0f;
+    const float dy = in.dy;
 #pragma unroll
     for (int r = 0; r < kRows; ++r) {
       const int row = kg * kRows + r;
@@ -228,13 +260,17 @@ recurrence_backward_kernel(RecurrenceArgs a) {
       decayed[r] = previous[r] * s.decay;
       prediction += decayed[r] * k[r];
       // dq[row] = sum over columns of S_{t+1}[row, column] dy[column]
-      const float dq_row = half_wave_sum(matrix * dy);
-      if (c == 0) dq_rows[row] = dq_row;
+      q_products[row][c] = matrix * dy;
       dm[r] += q[r] * dy;
     }
     prediction = column_total(prediction, scratch, kg, c);
-    const float v = column_ok ? a.post[1LL * t * channels + 2 * a.kh * a.kd + head * a.vd + column] : 0.0f;
-    const float difference = v - prediction;
+    if (tid < kMaxKey) {
+      float sum = 0.0f;
+#pragma unroll
+      for (int j = 0; j < kColumns; ++j) sum += q_products[tid][j];
+      dq_rows[tid] = sum;
+    }
+    const float difference = in.v - prediction;
     const float delta = difference * s.beta;
     float ddelta = 0.0f;
 #pragma unroll
@@ -247,8 +283,7 @@ recurrence_backward_kernel(RecurrenceArgs a) {
 #pragma unroll
     for (int r = 0; r < kRows; ++r) {
       const int row = kg * kRows + r;
-      const float dk_row = half_wave_sum(dm[r] * delta - decayed[r] * dv);
-      if (c == 0) dk_rows[row] = dk_row;
+      k_products[row][c] = dm[r] * delta - decayed[r] * dv;
       const float ddecayed = dm[r] - k[r] * dv;
       dg += ddecayed * previous[r];
       dm[r] = ddecayed * s.decay;
@@ -262,6 +297,13 @@ recurrence_backward_kernel(RecurrenceArgs a) {
     if (tid % 64 == 0) {
       block_sums[wave][0] = dg;
       block_sums[wave][1] = db_partial;
+    }
+    __syncthreads();
+    if (tid < kMaxKey) {
+      float sum = 0.0f;
+#pragma unroll
+      for (int j = 0; j < kColumns; ++j) sum += k_products[tid][j];
+      dk_rows[tid] = sum;
     }
     __syncthreads();
     const long long partial = (1LL * t * a.vh + head) * tiles + tile;
