@@ -70,7 +70,7 @@ struct Config {
   static constexpr int kStageBytes = 2 * kTileBytes;
   static constexpr int kLoads = BN * KCH / kThreads;  // 16-byte loads per lane per tensor
   // waves per SIMD the register budget is sized for
-  static constexpr int kOccupancy = (D == 64 && G == 1) ? 3 : 2;
+  static constexpr int kOccupancy = (D == 64 && G == 1) ? 3 : (D == 256 ? 1 : 2);
 };
 
 template <int D, int G, int WAVES>
@@ -378,7 +378,7 @@ long long grid_blocks(const FlashForwardArgs& a, int block_rows, int sequences, 
 }  // namespace
 
 bool flash_forward_supported(const FlashForwardArgs& a, int head_dim) {
-  if (head_dim != 64 && head_dim != 128) return false;
+  if (head_dim != 64 && head_dim != 128 && head_dim != 256) return false;
   auto aligned = [](const void* p) {
     return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
   };
@@ -404,7 +404,9 @@ int launch_flash_forward(hipStream_t stream, const FlashForwardArgs& a,
   const long long blocks = grid_blocks(a, 128, sequences, head_dim == 64);
   if (blocks <= 0 || blocks > 0x7fffffffLL) return PLUTO_HIP_EINVAL;
   const dim3 grid(static_cast<unsigned>(blocks));
-  if (head_dim == 128)
+  if (head_dim == 256)
+    flash_forward_kernel<256, 1, 4><<<grid, 256, 0, stream>>>(a);
+  else if (head_dim == 128)
     flash_forward_kernel<128, 1, 4><<<grid, 256, 0, stream>>>(a);
   else
     flash_forward_kernel<64, 1, 4><<<grid, 256, 0, stream>>>(a);
