@@ -68,8 +68,34 @@ int launch_gdn_output(hipStream_t stream, const void* core, int core_dtype, cons
                       int z_dtype, const float* norm, long long rows, int value_dim,
                       float epsilon, bool round, void* out, int out_dtype);
 
+// Chunked form of the recurrence part of the backward for 128 x 128 heads
+// (gdn_backward_chunked.hip): `forward` leaves the outputs in `core`, `reverse`
+// (after `dcore` is known) leaves dv in `dpost` and the q/k and gate gradients
+// as one partial per (token, value head), in the layout the token-by-token
+// kernels use with a single column tile.
+struct GdnChunkedBackward {
+  const float* post = nullptr;   // [T, channels] convolved, activated q | k | v
+  const uint16_t* a = nullptr;   // bf16 [T, vh]
+  const uint16_t* b = nullptr;
+  const float* a_log = nullptr;
+  const float* dt_bias = nullptr;
+  const float* dcore = nullptr;  // [T, vh, 128]
+  float* core = nullptr;         // [T, vh, 128]
+  float* dpost = nullptr;
+  float* qk_partials = nullptr;      // [T, vh, 2, 128]
+  float* scalar_partials = nullptr;  // [T, vh, 3]
+  float* records = nullptr;          // gdn_backward_chunked_bytes(...)
+  int length = 0, key_heads = 0, value_heads = 0;
+  bool round = true;
+};
+bool gdn_backward_chunked_supported(const pluto_hip_delta_params* p);
+size_t gdn_backward_chunked_bytes(const pluto_hip_delta_params* p, int length);
+int launch_gdn_backward_chunked_forward(hipStream_t stream, const GdnChunkedBackward& c);
+int launch_gdn_backward_chunked_reverse(hipStream_t stream, const GdnChunkedBackward& c);
+
 // Backward of the whole layer for one sequence (gdn_backward.hip): the forward
-// pass is repeated with every per-token state kept in `workspace`.
+// pass is repeated with the states it needs kept in `workspace` (one per
+// 64-token chunk for 128 x 128 heads, one per token otherwise).
 constexpr int kGdnSumChunks = 128;
 size_t gdn_backward_workspace_bytes(const pluto_hip_delta_params* p, int length, bool norm_grad);
 int launch_gdn_backward(hipStream_t stream, const pluto_hip_delta_params* p, int length,

@@ -488,15 +488,25 @@ unsigned blocks_for(long long elements) { return static_cast<unsigned>((elements
 
 }  // namespace
 
+bool force_generic();  // mha_capi.hip
+
+namespace {
+bool use_chunks(const pluto_hip_delta_params* p) {
+  return !force_generic() && gdn_backward_chunked_supported(p);
+}
+}  // namespace
+
 size_t gdn_backward_workspace_bytes(const pluto_hip_delta_params* p, int length, bool norm_grad) {
   const size_t T = static_cast<size_t>(length);
   const size_t kh = p->key_heads, vh = p->value_heads, kd = p->key_head_dim, vd = p->value_head_dim;
   const size_t channels = 2 * kh * kd + vh * vd;
-  const size_t tiles = (vd + kColumns - 1) / kColumns;
+  const bool chunked = use_chunks(p);
+  const size_t tiles = chunked ? 1 : (vd + kColumns - 1) / kColumns;
   size_t bytes = 0;
   bytes += 4 * align_up(T * channels * 4, 256);          // pre, post, dpost, dpre
   bytes += 2 * align_up(T * vh * vd * 4, 256);           // core, dcore
-  bytes += align_up((T + 1) * vh * kd * vd * 4, 256);    // states
+  bytes += chunked ? gdn_backward_chunked_bytes(p, length)
+                   : align_up((T + 1) * vh * kd * vd * 4, 256);  // states
   bytes += align_up(T * vh * tiles * 2 * kd * 4, 256);   // q/k partials
   bytes += align_up(T * vh * tiles * 3 * 4, 256);        // scalar partials
   if (norm_grad) bytes += align_up(T * vh * vd * 4, 256) + align_up(kGdnSumChunks * vd * 4, 256);
@@ -512,7 +522,8 @@ int launch_gdn_backward(hipStream_t stream, const pluto_hip_delta_params* p, int
   const size_t T = static_cast<size_t>(length);
   const int kh = p->key_heads, vh = p->value_heads, kd = p->key_head_dim, vd = p->value_head_dim;
   const int channels = 2 * kh * kd + vh * vd, kernel = p->conv_kernel_dim;
-  const int tiles = (vd + kColumns - 1) / kColumns;
+  const bool chunked = use_chunks(p);
+  const int tiles = chunked ? 1 : (vd + kColumns - 1) / kColumns;
   const bool round = p->round_to_bfloat16 != 0;
   char* at = static_cast<char*>(workspace);
   auto take = [&](size_t bytes) {
@@ -526,7 +537,7 @@ int launch_gdn_backward(hipStream_t stream, const pluto_hip_delta_params* p, int
   float* dpre = take(T * channels * 4);
   float* core = take(T * vh * vd * 4);
   float* dcore = take(T * vh * vd * 4);
-  float* states = take((T + 1) * vh * kd * vd * 4);
+  float* states = take(chunked ? gdn_backward_chunked_bytes(p, length) : (T + 1) * vh * kd * vd * 4);
   float* qk_partials = take(T * vh * tiles * 2 * kd * 4);
   float* scalar_partials = take(T * vh * tiles * 3 * 4);
   float* norm_partials = d_norm ? take(T * vh * vd * 4) : nullptr;
@@ -555,8 +566,28 @@ int launch_gdn_backward(hipStream_t stream, const pluto_hip_delta_params* p, int
   r.kd = kd;
   r.vd = vd;
   r.round = round;
-  recurrence_states_kernel<<<vh * tiles, 256, 0, stream>>>(r);
-  status = launch_status();
+  GdnChunkedBackward c;
+  c.post = post;
+  c.a = r.a;
+  c.b = r.b;
+  c.a_log = a_log;
+  c.dt_bias = dt_bias;
+  c.dcore = dcore;
+  c.core = core;
+  c.dpost = dpost;
+  c.qk_partials = qk_partials;
+  c.scalar_partials = scalar_partials;
+  c.records = states;
+  c.length = length;
+  c.key_heads = kh;
+  c.value_heads = vh;
+  c.round = round;
+  if (chunked) {
+    status = launch_gdn_backward_chunked_forward(stream, c);
+  } else {
+    recurrence_states_kernel<<<vh * tiles, 256, 0, stream>>>(r);
+    status = launch_status();
+  }
   if (status != 0) return status;
   output_backward_kernel<<<static_cast<unsigned>(length) * vh, 64, 0, stream>>>(
       core, static_cast<const uint16_t*>(z), norm, dy, vd, p->rms_norm_epsilon, round, dcore, dz,
@@ -570,8 +601,12 @@ int launch_gdn_backward(hipStream_t stream, const pluto_hip_delta_params* p, int
     status = launch_status();
     if (status != 0) return status;
   }
-  recurrence_backward_kernel<<<vh * tiles, 256, 0, stream>>>(r);
-  status = launch_status();
+  if (chunked) {
+    status = launch_gdn_backward_chunked_reverse(stream, c);
+  } else {
+    recurrence_backward_kernel<<<vh * tiles, 256, 0, stream>>>(r);
+    status = launch_status();
+  }
   if (status != 0) return status;
   gather_qk_kernel<<<dim3(kh, length), 128, 0, stream>>>(qk_partials, kh, vh, kd, tiles, channels,
                                                          dpost);

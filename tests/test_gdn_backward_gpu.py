@@ -80,7 +80,11 @@ def run(capi, shape, rounding, seed=0, batch=1, with_parameters=True):
     return got, want, args, grads
 
 
-SHAPES = [(4, 1, 2, 3, 5, 3), (9, 2, 4, 5, 35, 4), (33, 2, 2, 16, 40, 4), (64, 1, 2, 128, 128, 4)]
+# (T, key heads, value heads, key width, value width, conv taps).  128 x 128
+# heads take the chunked kernels (64-token chunks: one full chunk, a ragged
+# tail, grouped heads over several chunks); the other widths go token by token.
+SHAPES = [(4, 1, 2, 3, 5, 3), (9, 2, 4, 5, 35, 4), (33, 2, 2, 16, 40, 4), (64, 1, 2, 128, 128, 4),
+          (37, 1, 1, 128, 128, 4), (200, 1, 2, 128, 128, 4), (130, 2, 4, 128, 128, 3)]
 
 
 @pytest.mark.parametrize("rounding", [False, True])
@@ -119,6 +123,42 @@ def test_batch_and_parameter_gradient_accumulation(capi):
     frozen, _, _, _ = run(capi, shape, False, seed=3, batch=3, with_parameters=False)
     for name in ("dqkv", "dz", "da", "db"):
         np.testing.assert_array_equal(frozen[name], got[name])
+
+
+def test_chunked_and_token_by_token_kernels_agree(capi):
+    """128 x 128 heads over 9 chunks: the chunked kernels against the
+    token-by-token kernels of the same library (FP32 both, different order of
+    summation), at a length the CPU oracle would take minutes for."""
+    import os
+    shape = (520, 2, 4, 128, 128, 4)
+    T, kh, vh, kd, vd, K = shape
+    kw = dict(key_heads=kh, value_heads=vh, key_head_dim=kd, value_head_dim=vd, conv_kernel_dim=K,
+              round_to_bfloat16=False)
+    p = capi.delta_params(**kw)
+    c = make_case(T, kh, vh, kd, vd, K, seed=11)
+    bf = torch.bfloat16
+    args = (p, dev(c["qkv"], bf), dev(c["z"], bf), dev(c["a"], bf), dev(c["b"], bf), dev(c["conv"]),
+            dev(c["a_log"]), dev(c["dt_bias"]), dev(c["norm"]), dev(c["dy"]))
+    channels = 2 * kh * kd + vh * vd
+
+    def once():
+        grads = dict(conv_weight=torch.zeros(channels, K, device="cuda"),
+                     a_log=torch.zeros(vh, device="cuda"), dt_bias=torch.zeros(vh, device="cuda"),
+                     norm=torch.zeros(vd, device="cuda"))
+        out = capi.gdn_layer_backward(*args, parameter_grads=grads)
+        torch.cuda.synchronize()
+        named = dict(zip(("dqkv", "dz", "da", "db"), out))
+        named.update(grads)
+        return {k: v.cpu().numpy() for k, v in named.items()}
+
+    chunked = once()
+    os.environ["PLUTO_HIP_FORCE_GENERIC"] = "1"
+    try:
+        sequential = once()
+    finally:
+        del os.environ["PLUTO_HIP_FORCE_GENERIC"]
+    for name in sequential:
+        assert_close(chunked[name], sequential[name], 2e-4, name)
 
 
 def test_rejects_bad_arguments(capi):
