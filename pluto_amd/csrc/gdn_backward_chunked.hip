@@ -16,17 +16,25 @@
 //   O   = diag(E) Q^ S + P Dl
 //   S'  = E_63 S + (diag(L) K^)^T Dl
 // which is the recurrence S <- decay S; delta = beta (v - S^T k^); S += k^ x
-// delta; o = S^T q^ unrolled over the chunk.  The backward differentiates
-// exactly these formulas:
-//   chunk_prepare_kernel           everything that depends on one chunk only
-//   chunk_states_forward_kernel    S entering every chunk, Dl, O (sequential in
-//                                  the chunks, one workgroup per 32 value columns)
-//   chunk_states_backward_kernel   dS leaving every chunk and dDl, in reverse
-//   chunk_gradients_kernel         dq, dk, dv, d beta, d log-decay of a chunk
-//                                  from S, dS, Dl, dDl (chunk-parallel)
-// Matrix products run on v_mfma_f32_32x32x2_f32; operands are read straight
-// from global memory (written by the kernel before in the order the consumer
-// contracts over) or from LDS.
+// delta; o = S^T q^ unrolled over the chunk.  Eliminating Dl, the state obeys
+// an affine recurrence whose matrices depend on one chunk only,
+//   S' = M S + B,     M = E_63 I - (diag(L) K^)^T W,    B = (diag(L) K^)^T U,
+// and so does its gradient:
+//   dS = M^T dS' + C,  C = Y^T dO,   Y = diag(E) Q^ - P W.
+// The kernels, in launch order:
+//   chunk_prepare_kernel           T, W, U, P of every chunk          (parallel)
+//   chunk_transfer_kernel          M, M^T, B, Y                       (parallel)
+//   chunk_states_forward_kernel    S entering every chunk             (sequential)
+//   chunk_outputs_kernel           Dl and O from S                    (parallel)
+//     -- the caller turns O into dO here --
+//   chunk_local_kernel             C                                  (parallel)
+//   chunk_states_backward_kernel   dS' leaving every chunk            (sequential)
+//   chunk_gradients_kernel         dDl, then dq, dk, dv, d beta and
+//                                  d log-decay of the chunk           (parallel)
+// The sequential kernels run one workgroup per (head, 32 value columns) and
+// do one 128 x 128 x 32 product a chunk, with the next chunk's matrix already
+// in registers.  Matrix products run on v_mfma_f32_32x32x2_f32; operands are
+// read straight from global memory or from LDS.
 #include "gdn.h"
 
 namespace pluto_hip {
@@ -41,17 +49,17 @@ constexpr int kState = kD * kD;    // elements of a state
 
 // Per (head, chunk) records in the workspace, in floats.
 struct Records {
-  float *qn, *qt, *kn, *kt;   // q^, k^ [64][128] and their transposes [128][64]
-  float *w, *wt, *u;          // W, W^T, U
-  float *p, *pt, *tm, *kkd;   // P, P^T, T, strict_lower((k^_i . k^_j) D_ij)   [64][64]
-  float *gates;               // [4][64]: G, beta, 1/|q|, 1/|k|
+  float *qn, *kn;             // q^, k^                                  [64][128]
+  float *w, *u, *y, *dl;      // W, U, Y, Dl                             [64][128]
+  float *p, *tm, *kkd;        // P, T, strict_lower((k^_i . k^_j) D_ij)  [64][64]
+  float *gates;               // [6][64]: G, beta, 1/|q|, 1/|k|, E, L
+  float *m, *mt, *bc, *cc;    // M, M^T, B, C                            [128][128]
   float *s0, *ds1;            // state entering the chunk, gradient of the state leaving it
-  float *dl, *ddl;            // Dl and its gradient [64][128]
 };
 
-constexpr size_t kRecordFloats =
-    7 * static_cast<size_t>(kWide) + 4 * kSquare + 4 * kC + 2 * static_cast<size_t>(kState) +
-    2 * kWide;
+constexpr int kGateRows = 6;
+constexpr size_t kRecordFloats = 6 * static_cast<size_t>(kWide) + 3 * kSquare + kGateRows * kC +
+                                 6 * static_cast<size_t>(kState);
 
 struct ChunkedArgs {
   const float* post = nullptr;     // [T, channels]
@@ -116,8 +124,18 @@ __device__ inline float4 scaled(float4 v, float s) {
   return make_float4(v.x * s, v.y * s, v.z * s, v.w * s);
 }
 
+__device__ inline float4 gather4(const float* p, int stride) {
+  return make_float4(p[0], p[stride], p[2 * stride], p[3 * stride]);
+}
+
+// Barrier for data exchanged through LDS only: pending global loads and
+// stores stay in flight across it.
+__device__ inline void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 // ---------------------------------------------------------------------------
-// Everything that depends on one chunk only.
+// T, W, U, P and the gates of one chunk.
 __global__ void __launch_bounds__(256)
 chunk_prepare_kernel(ChunkedArgs a) {
   __shared__ float qs[kC][kD + 1], ks[kC][kD + 1];
@@ -132,7 +150,7 @@ chunk_prepare_kernel(ChunkedArgs a) {
   const size_t rec = static_cast<size_t>(head) * a.chunks + chunk;
   const int t0 = chunk * kC;
   const float norm_scale = sqrtf(static_cast<float>(kD));
-  float* gates = a.r.gates + rec * 4 * kC;
+  float* gates = a.r.gates + rec * kGateRows * kC;
 
   // normalised rows (1e-6 added to the sums of squares, sequence_delta_net.cc:84-85)
   for (int r = 0; r < kC / 4; ++r) {
@@ -186,7 +204,11 @@ chunk_prepare_kernel(ChunkedArgs a) {
     }
   }
   __syncthreads();
-  if (tid < kC) gates[tid] = g_cum[tid];
+  if (tid < kC) {
+    gates[tid] = g_cum[tid];
+    gates[4 * kC + tid] = expf(g_cum[tid]);
+    gates[5 * kC + tid] = expf(g_cum[kC - 1] - g_cum[tid]);
+  }
 
   // k^ k^T and q^ k^T, one 32 x 32 tile a wave (tile (0, 1) is above the diagonal)
   {
@@ -200,22 +222,13 @@ chunk_prepare_kernel(ChunkedArgs a) {
     }
     const int col = 32 * tj + n;
 #pragma unroll
-    for (int i4 = 0; i4 < 4; ++i4) {
-      float4 transposed;
-      float* piece = &transposed.x;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int i = 4 * i4 + e, row = 32 * ti + tile_row(i, h);
-        const float d = row >= col ? expf(g_cum[row] - g_cum[col]) : 0.0f;
-        const float pv = row >= col ? qk[i] * d : 0.0f;
-        const float kv = row > col ? kk[i] * d : 0.0f;
-        a.r.p[rec * kSquare + row * kC + col] = pv;
-        a.r.kkd[rec * kSquare + row * kC + col] = kv;
-        am[row][col] = beta_s[row] * kv;
-        piece[e] = pv;
-      }
-      *reinterpret_cast<float4*>(a.r.pt + rec * kSquare + col * kC + 32 * ti + tile_row(4 * i4, h)) =
-          transposed;
+    for (int i = 0; i < 16; ++i) {
+      const int row = 32 * ti + tile_row(i, h);
+      const float d = row >= col ? expf(g_cum[row] - g_cum[col]) : 0.0f;
+      const float kv = row > col ? kk[i] * d : 0.0f;
+      a.r.p[rec * kSquare + row * kC + col] = row >= col ? qk[i] * d : 0.0f;
+      a.r.kkd[rec * kSquare + row * kC + col] = kv;
+      am[row][col] = beta_s[row] * kv;
     }
   }
   __syncthreads();
@@ -253,165 +266,213 @@ chunk_prepare_kernel(ChunkedArgs a) {
             return t < a.length ? a.post[static_cast<size_t>(t) * channels + value_offset + col] : 0.0f;
           });
 #pragma unroll
-      for (int i4 = 0; i4 < 4; ++i4) {
-        float4 transposed;
-        float* piece = &transposed.x;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int i = 4 * i4 + e, row = 32 * ti + tile_row(i, h);
-          a.r.w[rec * kWide + row * kD + col] = wacc[i];
-          a.r.u[rec * kWide + row * kD + col] = uacc[i];
-          piece[e] = wacc[i];
-        }
-        *reinterpret_cast<float4*>(a.r.wt + rec * kWide + col * kC + 32 * ti + tile_row(4 * i4, h)) =
-            transposed;
-      }
-    }
-  }
-  // transposed copies of q^ and k^
-  for (int idx = tid; idx < kWide; idx += 256) {
-    const int d = idx / kC, i = idx % kC;
-    a.r.qt[rec * kWide + idx] = qs[i][d];
-    a.r.kt[rec * kWide + idx] = ks[i][d];
-  }
-}
-
-// ---------------------------------------------------------------------------
-// States entering the chunks, the delta rows and the outputs.  One workgroup
-// per (head, 32 value columns); wave w keeps rows 32w..32w+31 of its state
-// slice in accumulator registers.
-__global__ void __launch_bounds__(256)
-chunk_states_forward_kernel(ChunkedArgs a) {
-  __shared__ float state[kD][kSlice];
-  __shared__ float delta[kC][kSlice], delta_decayed[kC][kSlice];
-  __shared__ float e_s[kC], l_s[kC];
-  const int head = blockIdx.x / (kD / kSlice), col0 = (blockIdx.x % (kD / kSlice)) * kSlice;
-  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
-  const int h = lane / 32, n = lane % 32;
-  floatx16 s_acc = zero_tile();
-  for (int chunk = 0; chunk < a.chunks; ++chunk) {
-    const size_t rec = static_cast<size_t>(head) * a.chunks + chunk;
-    const float* gates = a.r.gates + rec * 4 * kC;
-    if (tid < kC) {
-      const float g = gates[tid];
-      e_s[tid] = expf(g);
-      l_s[tid] = expf(gates[kC - 1] - g);
-    }
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int row = 32 * wave + tile_row(i, h);
-      state[row][n] = s_acc[i];
-      a.r.s0[rec * kState + row * kD + col0 + n] = s_acc[i];
-    }
-    __syncthreads();
-    floatx16 acc;
-    const int ti = wave % 2;
-    if (wave < 2) {
-      // Dl = U - W S
-#pragma unroll
-      for (int i = 0; i < 16; ++i)
-        acc[i] = a.r.u[rec * kWide + (32 * ti + tile_row(i, h)) * kD + col0 + n];
-      const float* wt = a.r.wt + rec * kWide + 32 * ti + n;
-      acc = product<kD>(acc, [&](int k) { return -wt[k * kC]; }, [&](int k) { return state[k][n]; });
-#pragma unroll
       for (int i = 0; i < 16; ++i) {
         const int row = 32 * ti + tile_row(i, h);
-        delta[row][n] = acc[i];
-        delta_decayed[row][n] = acc[i] * l_s[row];
-        a.r.dl[rec * kWide + row * kD + col0 + n] = acc[i];
-      }
-    } else {
-      // O = diag(E) Q^ S ...
-      const float e = e_s[32 * ti + n];
-      const float* qt = a.r.qt + rec * kWide + 32 * ti + n;
-      acc = product<kD>(zero_tile(), [&](int k) { return qt[k * kC] * e; },
-                        [&](int k) { return state[k][n]; });
-    }
-    __syncthreads();
-    if (wave >= 2) {
-      // ... + P Dl
-      const float* pt = a.r.pt + rec * kSquare + 32 * ti + n;
-      acc = product<kC>(acc, [&](int k) { return pt[k * kC]; }, [&](int k) { return delta[k][n]; });
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int t = chunk * kC + 32 * ti + tile_row(i, h);
-        if (t < a.length)
-          a.core[(static_cast<size_t>(t) * a.vh + head) * kD + col0 + n] = round_if(acc[i], a.round);
+        a.r.w[rec * kWide + row * kD + col] = wacc[i];
+        a.r.u[rec * kWide + row * kD + col] = uacc[i];
       }
     }
-    // S' = E_63 S + (diag(L) K^)^T Dl
-    const float e_last = e_s[kC - 1];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) s_acc[i] *= e_last;
-    const float* kn = a.r.kn + rec * kWide + 32 * wave + n;
-    s_acc = product<kC>(s_acc, [&](int k) { return kn[k * kD]; },
-                        [&](int k) { return delta_decayed[k][n]; });
-    __syncthreads();
   }
 }
 
 // ---------------------------------------------------------------------------
-// Gradients of the states leaving the chunks and of the delta rows, in
-// reverse.  Same decomposition as the forward kernel.
+// The matrices of the two affine recurrences that depend on the chunk alone:
+// M, M^T, B and Y.  Wave w owns columns 32w..32w+31 of each.
 __global__ void __launch_bounds__(256)
-chunk_states_backward_kernel(ChunkedArgs a) {
-  __shared__ float dstate[kD][kSlice];
-  __shared__ float dout[kC][kSlice], dout_decayed[kC][kSlice], ddelta[kC][kSlice];
+chunk_transfer_kernel(ChunkedArgs a) {
   __shared__ float e_s[kC], l_s[kC];
+  const int chunk = blockIdx.x, head = blockIdx.y;
+  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+  const int h = lane / 32, n = lane % 32;
+  const size_t rec = static_cast<size_t>(head) * a.chunks + chunk;
+  const float* gates = a.r.gates + rec * kGateRows * kC;
+  const float* Q = a.r.qn + rec * kWide;
+  const float* K = a.r.kn + rec * kWide;
+  const float* W = a.r.w + rec * kWide;
+  const float* U = a.r.u + rec * kWide;
+  const float* P = a.r.p + rec * kSquare;
+  if (tid < kC) {
+    e_s[tid] = gates[4 * kC + tid];
+    l_s[tid] = gates[5 * kC + tid];
+  }
+  __syncthreads();
+  const int col = 32 * wave + n;
+  // Y = diag(E) Q^ - P W
+#pragma unroll
+  for (int ti = 0; ti < 2; ++ti) {
+    floatx16 acc;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int row = 32 * ti + tile_row(i, h);
+      acc[i] = e_s[row] * Q[row * kD + col];
+    }
+    const int m = 32 * ti + n;
+    acc = product4<kC>(acc, [&](int k) { return scaled(load4(P + m * kC + k), -1.0f); },
+                       [&](int k) { return gather4(W + k * kD + col, kD); });
+#pragma unroll
+    for (int i = 0; i < 16; ++i) a.r.y[rec * kWide + (32 * ti + tile_row(i, h)) * kD + col] = acc[i];
+  }
+  // M = E_63 I - (diag(L) K^)^T W and B = (diag(L) K^)^T U
+  const float e_last = e_s[kC - 1];
+#pragma unroll
+  for (int td = 0; td < 4; ++td) {
+    const int m = 32 * td + n;
+    floatx16 macc;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) macc[i] = 32 * td + tile_row(i, h) == col ? e_last : 0.0f;
+    macc = product<kC>(macc, [&](int k) { return -l_s[k] * K[k * kD + m]; },
+                       [&](int k) { return W[k * kD + col]; });
+    const floatx16 bacc = product<kC>(zero_tile(), [&](int k) { return l_s[k] * K[k * kD + m]; },
+                                      [&](int k) { return U[k * kD + col]; });
+#pragma unroll
+    for (int i4 = 0; i4 < 4; ++i4) {
+      const int row = 32 * td + tile_row(4 * i4, h);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        a.r.m[rec * kState + (row + e) * kD + col] = macc[4 * i4 + e];
+        a.r.bc[rec * kState + (row + e) * kD + col] = bacc[4 * i4 + e];
+      }
+      *reinterpret_cast<float4*>(a.r.mt + rec * kState + col * kD + row) =
+          make_float4(macc[4 * i4], macc[4 * i4 + 1], macc[4 * i4 + 2], macc[4 * i4 + 3]);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// next = matrix . state + offset over the chunks of one (head, 32 value
+// columns): forward (REVERSE false) it stores the state entering every chunk,
+// with matrix M (read through its transpose) and offset B; in reverse it
+// stores the state gradient leaving every chunk, with matrix M^T (read through
+// M) and offset C.  Wave w keeps rows 32w..32w+31 of the slice; the matrix
+// column and the offset tile of the next chunk are requested while the
+// current product runs.
+template <bool REVERSE>
+__global__ void __launch_bounds__(256)
+chunk_states_kernel(ChunkedArgs a) {
+  __shared__ float state[2][kD][kSlice];
   const int head = blockIdx.x / (kD / kSlice), col0 = (blockIdx.x % (kD / kSlice)) * kSlice;
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
   const int h = lane / 32, n = lane % 32;
-  floatx16 ds_acc = zero_tile();
-  for (int chunk = a.chunks - 1; chunk >= 0; --chunk) {
-    const size_t rec = static_cast<size_t>(head) * a.chunks + chunk;
-    const float* gates = a.r.gates + rec * 4 * kC;
-    if (tid < kC) {
-      const float g = gates[tid];
-      e_s[tid] = expf(g);
-      l_s[tid] = expf(gates[kC - 1] - g);
-    }
+  const float* matrices = REVERSE ? a.r.m : a.r.mt;
+  const float* offsets = REVERSE ? a.r.cc : a.r.bc;
+  float* saved = REVERSE ? a.r.ds1 : a.r.s0;
+  auto record = [&](int step) {
+    return static_cast<size_t>(head) * a.chunks + (REVERSE ? a.chunks - 1 - step : step);
+  };
+  float matrix[kD / 2], next_matrix[kD / 2];
+  floatx16 offset, next_offset;
+  auto request = [&](int step, float* mat, floatx16& off) {
+    const size_t rec = record(step);
+    const float* source = matrices + rec * kState + 32 * wave + n;
+#pragma unroll
+    for (int s = 0; s < kD / 2; ++s) mat[s] = source[(2 * s + h) * kD];
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      off[i] = offsets[rec * kState + (32 * wave + tile_row(i, h)) * kD + col0 + n];
+  };
+  request(0, matrix, offset);
+  floatx16 acc = zero_tile();
+  for (int step = 0; step < a.chunks; ++step) {
+    const size_t rec = record(step);
+    float (*current)[kSlice] = state[step & 1];
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       const int row = 32 * wave + tile_row(i, h);
-      dstate[row][n] = ds_acc[i];
-      a.r.ds1[rec * kState + row * kD + col0 + n] = ds_acc[i];
+      current[row][n] = acc[i];
+      saved[rec * kState + row * kD + col0 + n] = acc[i];
     }
-    for (int idx = tid; idx < kC * kSlice; idx += 256) {
-      const int i = idx / kSlice, c = idx % kSlice, t = chunk * kC + i;
-      const float value =
-          t < a.length ? a.dcore[(static_cast<size_t>(t) * a.vh + head) * kD + col0 + c] : 0.0f;
-      dout[i][c] = value;
-      dout_decayed[i][c] = value * expf(gates[i]);
-    }
-    __syncthreads();
-    // dS = E_63 dS' + (diag(E) Q^)^T dO - W^T dDl, first two terms
-    const float e_last = e_s[kC - 1];
+    lds_barrier();
+    if (step + 1 < a.chunks) request(step + 1, next_matrix, next_offset);
+    acc = offset;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) ds_acc[i] *= e_last;
-    const float* qn = a.r.qn + rec * kWide + 32 * wave + n;
-    ds_acc = product<kC>(ds_acc, [&](int k) { return qn[k * kD]; },
-                         [&](int k) { return dout_decayed[k][n]; });
-    if (wave < 2) {
-      // dDl = P^T dO + diag(L) K^ dS'
-      const float* p = a.r.p + rec * kSquare + 32 * wave + n;
-      floatx16 acc = product<kC>(zero_tile(), [&](int k) { return p[k * kC]; },
-                                 [&](int k) { return dout[k][n]; });
-      const float l = l_s[32 * wave + n];
-      const float* kt = a.r.kt + rec * kWide + 32 * wave + n;
-      acc = product<kD>(acc, [&](int k) { return kt[k * kC] * l; },
-                        [&](int k) { return dstate[k][n]; });
+    for (int s = 0; s < kD / 2; ++s)
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(matrix[s], current[2 * s + h][n], acc, 0, 0, 0);
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int row = 32 * wave + tile_row(i, h);
-        ddelta[row][n] = acc[i];
-        a.r.ddl[rec * kWide + row * kD + col0 + n] = acc[i];
-      }
+    for (int s = 0; s < kD / 2; ++s) matrix[s] = next_matrix[s];
+    offset = next_offset;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Dl = U - W S and O = diag(E) Q^ S + P Dl of one chunk.  Wave w owns value
+// columns 32w..32w+31.
+__global__ void __launch_bounds__(256)
+chunk_outputs_kernel(ChunkedArgs a) {
+  __shared__ float delta[kC][kD];
+  __shared__ float e_s[kC];
+  const int chunk = blockIdx.x, head = blockIdx.y;
+  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+  const int h = lane / 32, n = lane % 32;
+  const size_t rec = static_cast<size_t>(head) * a.chunks + chunk;
+  const float* gates = a.r.gates + rec * kGateRows * kC;
+  const float* S0 = a.r.s0 + rec * kState;
+  const float* Q = a.r.qn + rec * kWide;
+  const float* W = a.r.w + rec * kWide;
+  const float* U = a.r.u + rec * kWide;
+  const float* P = a.r.p + rec * kSquare;
+  if (tid < kC) e_s[tid] = gates[4 * kC + tid];
+  const int col = 32 * wave + n;
+  floatx16 out[2];
+#pragma unroll
+  for (int ti = 0; ti < 2; ++ti) {
+    const int m = 32 * ti + n;
+    floatx16 acc;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = U[(32 * ti + tile_row(i, h)) * kD + col];
+    acc = product4<kD>(acc, [&](int k) { return scaled(load4(W + m * kD + k), -1.0f); },
+                       [&](int k) { return gather4(S0 + k * kD + col, kD); });
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int row = 32 * ti + tile_row(i, h);
+      delta[row][col] = acc[i];
+      a.r.dl[rec * kWide + row * kD + col] = acc[i];
     }
-    __syncthreads();
-    const float* w = a.r.w + rec * kWide + 32 * wave + n;
-    ds_acc = product<kC>(ds_acc, [&](int k) { return -w[k * kD]; },
-                         [&](int k) { return ddelta[k][n]; });
-    __syncthreads();
+    out[ti] = product4<kD>(zero_tile(), [&](int k) { return load4(Q + m * kD + k); },
+                           [&](int k) { return gather4(S0 + k * kD + col, kD); });
+  }
+  __syncthreads();
+#pragma unroll
+  for (int ti = 0; ti < 2; ++ti) {
+    const int m = 32 * ti + n;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) out[ti][i] *= e_s[32 * ti + tile_row(i, h)];
+    // only columns j <= i of P are set: the second row tile needs all 64
+    out[ti] = product4<kC>(out[ti], [&](int k) { return load4(P + m * kC + k); },
+                           [&](int k) {
+                             return make_float4(delta[k][col], delta[k + 1][col], delta[k + 2][col],
+                                                delta[k + 3][col]);
+                           });
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int t = chunk * kC + 32 * ti + tile_row(i, h);
+      if (t < a.length)
+        a.core[(static_cast<size_t>(t) * a.vh + head) * kD + col] = round_if(out[ti][i], a.round);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// C = Y^T dO of one chunk.
+__global__ void __launch_bounds__(256)
+chunk_local_kernel(ChunkedArgs a) {
+  const int chunk = blockIdx.x, head = blockIdx.y;
+  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+  const int h = lane / 32, n = lane % 32;
+  const size_t rec = static_cast<size_t>(head) * a.chunks + chunk;
+  const float* Y = a.r.y + rec * kWide;
+  const int col = 32 * wave + n, t0 = chunk * kC;
+#pragma unroll
+  for (int td = 0; td < 4; ++td) {
+    const int m = 32 * td + n;
+    const floatx16 acc = product<kC>(
+        zero_tile(), [&](int k) { return Y[k * kD + m]; },
+        [&](int k) {
+          const int t = t0 + k;
+          return t < a.length ? a.dcore[(static_cast<size_t>(t) * a.vh + head) * kD + col] : 0.0f;
+        });
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      a.r.cc[rec * kState + (32 * td + tile_row(i, h)) * kD + col] = acc[i];
   }
 }
 
@@ -420,12 +481,14 @@ chunk_states_backward_kernel(ChunkedArgs a) {
 // every other lane of it).
 __device__ inline float half_sum(float v) { return wave_half_sum(v); }
 
-// Gradients of one chunk.  Wave w owns columns 32w..32w+31 of the three
-// [64, 128] outputs (two 32-row tiles each) and one 32 x 32 tile of every
-// [64, 64] intermediate.
+// Gradients of one chunk: dDl = P^T dO + diag(L) K^ dS', then everything
+// the chunk's formulas feed.  Wave w owns columns 32w..32w+31 of the [64, 128]
+// matrices (two 32-row tiles each) and one 32 x 32 tile of every [64, 64]
+// intermediate.
 __global__ void __launch_bounds__(256)
 chunk_gradients_kernel(ChunkedArgs a) {
   __shared__ float dw[kC][kD + 1];
+  __shared__ __attribute__((aligned(16))) float ddl[kC][kD + 4];
   __shared__ float mx[kC][kC + 1], my[kC][kC + 1], mz[kC][kC + 1], mu[kC][kC + 1];
   __shared__ float g_s[kC], e_s[kC], l_s[kC], beta_s[kC], dg_s[kC];
   __shared__ float row_parts[6][kC][4];
@@ -440,11 +503,10 @@ chunk_gradients_kernel(ChunkedArgs a) {
   const size_t value_offset = 2 * static_cast<size_t>(a.kh) * kD + static_cast<size_t>(head) * kD;
   const size_t rec = static_cast<size_t>(head) * a.chunks + chunk;
   const int t0 = chunk * kC;
-  const float* gates = a.r.gates + rec * 4 * kC;
+  const float* gates = a.r.gates + rec * kGateRows * kC;
   const float* S0 = a.r.s0 + rec * kState;
   const float* dS1 = a.r.ds1 + rec * kState;
   const float* Dl = a.r.dl + rec * kWide;
-  const float* dDl = a.r.ddl + rec * kWide;
   const float* Q = a.r.qn + rec * kWide;
   const float* K = a.r.kn + rec * kWide;
   const float* Tm = a.r.tm + rec * kSquare;
@@ -455,6 +517,10 @@ chunk_gradients_kernel(ChunkedArgs a) {
     const int t = t0 + i;
     return t < a.length ? load4(a.dcore + (static_cast<size_t>(t) * a.vh + head) * kD + c)
                         : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+  };
+  auto dO1 = [&](int i, int c) {
+    const int t = t0 + i;
+    return t < a.length ? a.dcore[(static_cast<size_t>(t) * a.vh + head) * kD + c] : 0.0f;
   };
   auto V4 = [&](int j, int c) {
     const int t = t0 + j;
@@ -468,12 +534,26 @@ chunk_gradients_kernel(ChunkedArgs a) {
   if (tid < kC) {
     const float g = gates[tid];
     g_s[tid] = g;
-    e_s[tid] = expf(g);
-    l_s[tid] = expf(gates[kC - 1] - g);
+    e_s[tid] = gates[4 * kC + tid];
+    l_s[tid] = gates[5 * kC + tid];
     beta_s[tid] = gates[kC + tid];
   }
   __syncthreads();
   const int dcol = 32 * wave + n;
+
+  // ---- dDl = P^T dO + diag(L) K^ dS' ----------------------------------------
+#pragma unroll
+  for (int ti = 0; ti < 2; ++ti) {
+    const int m = 32 * ti + n;
+    floatx16 acc = product<kC>(zero_tile(), [&](int k) { return P[k * kC + m]; },
+                               [&](int k) { return dO1(k, dcol); });
+    const float l = l_s[m];
+    acc = product4<kD>(acc, [&](int k) { return scaled(load4(K + m * kD + k), l); },
+                       [&](int k) { return gather4(dS1 + k * kD + dcol, kD); });
+#pragma unroll
+    for (int i = 0; i < 16; ++i) ddl[32 * ti + tile_row(i, h)][dcol] = acc[i];
+  }
+  __syncthreads();
 
   // ---- products against the two states ------------------------------------
   floatx16 dq[2], dk[2];
@@ -482,7 +562,7 @@ chunk_gradients_kernel(ChunkedArgs a) {
     const int m = 32 * ti + n;
     // dW = -dDl S^T
     const floatx16 dwt = product4<kD>(
-        zero_tile(), [&](int k) { return scaled(load4(dDl + m * kD + k), -1.0f); },
+        zero_tile(), [&](int k) { return scaled(load4(&ddl[m][k]), -1.0f); },
         [&](int k) { return load4(S0 + dcol * kD + k); });
 #pragma unroll
     for (int i = 0; i < 16; ++i) dw[32 * ti + tile_row(i, h)][dcol] = dwt[i];
@@ -536,7 +616,7 @@ chunk_gradients_kernel(ChunkedArgs a) {
     const float fv = beta_s[j], fk = fv * e_s[j];
     floatx16 acc = product<kD>(zero_tile(), [&](int k) { return dw[32 * ti + n][k]; },
                                [&](int k) { return K[j * kD + k] * fk; });
-    acc = product4<kD>(acc, [&](int k) { return load4(dDl + (32 * ti + n) * kD + k); },
+    acc = product4<kD>(acc, [&](int k) { return load4(&ddl[32 * ti + n][k]); },
                        [&](int k) { return scaled(V4(j, k), fv); });
 #pragma unroll
     for (int i = 0; i < 16; ++i) mx[32 * ti + tile_row(i, h)][j] = acc[i];
@@ -607,7 +687,7 @@ chunk_gradients_kernel(ChunkedArgs a) {
                          [&](int k) { return Q[k * kD + dcol]; });
     // dv = diag(beta) T^T dDl
     const floatx16 tu = product<kC>(zero_tile(), [&](int k) { return Tm[k * kC + m]; },
-                                    [&](int k) { return dDl[k * kD + dcol]; });
+                                    [&](int k) { return ddl[k][dcol]; });
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       const int row = 32 * t2 + tile_row(i, h), t = t0 + row;
@@ -701,21 +781,21 @@ ChunkedArgs make_args(const GdnChunkedBackward& c) {
     return result;
   };
   a.r.qn = take(kWide);
-  a.r.qt = take(kWide);
   a.r.kn = take(kWide);
-  a.r.kt = take(kWide);
   a.r.w = take(kWide);
-  a.r.wt = take(kWide);
   a.r.u = take(kWide);
+  a.r.y = take(kWide);
+  a.r.dl = take(kWide);
   a.r.p = take(kSquare);
-  a.r.pt = take(kSquare);
   a.r.tm = take(kSquare);
   a.r.kkd = take(kSquare);
-  a.r.gates = take(4 * kC);
+  a.r.gates = take(kGateRows * kC);
+  a.r.m = take(kState);
+  a.r.mt = take(kState);
+  a.r.bc = take(kState);
+  a.r.cc = take(kState);
   a.r.s0 = take(kState);
   a.r.ds1 = take(kState);
-  a.r.dl = take(kWide);
-  a.r.ddl = take(kWide);
   return a;
 }
 
@@ -733,19 +813,30 @@ size_t gdn_backward_chunked_bytes(const pluto_hip_delta_params* p, int length) {
 
 int launch_gdn_backward_chunked_forward(hipStream_t stream, const GdnChunkedBackward& c) {
   const ChunkedArgs a = make_args(c);
-  chunk_prepare_kernel<<<dim3(a.chunks, a.vh), 256, 0, stream>>>(a);
+  const dim3 per_chunk(a.chunks, a.vh);
+  chunk_prepare_kernel<<<per_chunk, 256, 0, stream>>>(a);
   int status = launch_status();
   if (status != 0) return status;
-  chunk_states_forward_kernel<<<a.vh * (kD / kSlice), 256, 0, stream>>>(a);
+  chunk_transfer_kernel<<<per_chunk, 256, 0, stream>>>(a);
+  status = launch_status();
+  if (status != 0) return status;
+  chunk_states_kernel<false><<<a.vh * (kD / kSlice), 256, 0, stream>>>(a);
+  status = launch_status();
+  if (status != 0) return status;
+  chunk_outputs_kernel<<<per_chunk, 256, 0, stream>>>(a);
   return launch_status();
 }
 
 int launch_gdn_backward_chunked_reverse(hipStream_t stream, const GdnChunkedBackward& c) {
   const ChunkedArgs a = make_args(c);
-  chunk_states_backward_kernel<<<a.vh * (kD / kSlice), 256, 0, stream>>>(a);
+  const dim3 per_chunk(a.chunks, a.vh);
+  chunk_local_kernel<<<per_chunk, 256, 0, stream>>>(a);
   int status = launch_status();
   if (status != 0) return status;
-  chunk_gradients_kernel<<<dim3(a.chunks, a.vh), 256, 0, stream>>>(a);
+  chunk_states_kernel<true><<<a.vh * (kD / kSlice), 256, 0, stream>>>(a);
+  status = launch_status();
+  if (status != 0) return status;
+  chunk_gradients_kernel<<<per_chunk, 256, 0, stream>>>(a);
   return launch_status();
 }
 
