@@ -29,8 +29,11 @@
 //     -- the caller turns O into dO here --
 //   chunk_local_kernel             C                                  (parallel)
 //   chunk_states_backward_kernel   dS' leaving every chunk            (sequential)
-//   chunk_gradients_kernel         dDl, then dq, dk, dv, d beta and
-//                                  d log-decay of the chunk           (parallel)
+//   chunk_delta_gradient_kernel    dDl from dO and dS'                (parallel)
+//   chunk_state_products_kernel    dW and the state terms of dq^, dk^ (parallel)
+//   chunk_triangle_kernel          dP, dT, dA: the [64, 64] matrices  (parallel)
+//   chunk_finish_kernel            dq, dk, dv                         (parallel)
+//   chunk_gates_kernel             d beta, d log-decay -> da, db      (parallel)
 // The sequential kernels run one workgroup per (head, 32 value columns) and
 // do one 128 x 128 x 32 product a chunk, with the next chunk's matrix already
 // in registers.  Matrix products run on v_mfma_f32_32x32x2_f32; operands are
@@ -51,15 +54,19 @@ constexpr int kState = kD * kD;    // elements of a state
 struct Records {
   float *qn, *kn;             // q^, k^                                  [64][128]
   float *w, *u, *y, *dl;      // W, U, Y, Dl                             [64][128]
+  float *ddl, *dwm;           // dDl, dW                                 [64][128]
+  float *dqp, *dkp;           // the parts of dq^ and dk^ that come from the states
   float *p, *tm, *kkd;        // P, T, strict_lower((k^_i . k^_j) D_ij)  [64][64]
+  float *pd, *rr;             // dP D, diag(beta) dA D                   [64][64]
   float *gates;               // [6][64]: G, beta, 1/|q|, 1/|k|, E, L
+  float *sums;                // [9][64]: row and column sums for d beta and d log-decay
   float *m, *mt, *bc, *cc;    // M, M^T, B, C                            [128][128]
   float *s0, *ds1;            // state entering the chunk, gradient of the state leaving it
 };
 
-constexpr int kGateRows = 6;
-constexpr size_t kRecordFloats = 6 * static_cast<size_t>(kWide) + 3 * kSquare + kGateRows * kC +
-                                 6 * static_cast<size_t>(kState);
+constexpr int kGateRows = 6, kSumRows = 9;
+constexpr size_t kRecordFloats = 10 * static_cast<size_t>(kWide) + 5 * kSquare +
+                                 (kGateRows + kSumRows) * kC + 6 * static_cast<size_t>(kState);
 
 struct ChunkedArgs {
   const float* post = nullptr;     // [T, channels]
@@ -91,30 +98,68 @@ __device__ inline floatx16 zero_tile() {
 __device__ inline int tile_row(int i, int h) { return 8 * (i / 4) + 4 * h + i % 4; }
 
 // acc[m][n] += sum over k < K of A[m][k] B[k][n] for the lane's operand row m
-// and column n: a(k) returns A[m][k], b(k) returns B[k][n].
-template <int K, class AF, class BF>
+// and column n: a(k) returns A[m][k], b(k) returns B[k][n].  Every operand of
+// the product is requested before the first multiplication (one memory
+// latency a product instead of one every few steps) unless STREAM is set:
+// kernels whose registers allow many resident waves do better with the loads
+// spread between the multiplications.
+template <int K, bool STREAM = false, class AF, class BF>
 __device__ inline floatx16 product(floatx16 acc, AF a, BF b) {
   const int h = (threadIdx.x % 64) / 32;
+  if constexpr (STREAM) {
 #pragma unroll 8
-  for (int k = 0; k < K; k += 2)
-    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a(k + h), b(k + h), acc, 0, 0, 0);
+    for (int k = 0; k < K; k += 2)
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a(k + h), b(k + h), acc, 0, 0, 0);
+    return acc;
+  }
+  float av[K / 2], bv[K / 2];
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int s = 0; s < K / 2; ++s) {
+    av[s] = a(2 * s + h);
+    bv[s] = b(2 * s + h);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int s = 0; s < K / 2; ++s)
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[s], bv[s], acc, 0, 0, 0);
+  __builtin_amdgcn_sched_barrier(0);
   return acc;
 }
 
 // The same sum for operands that are contiguous along k: a4(k) returns
 // A[m][k..k+3], b4(k) returns B[k..k+3][n], k a multiple of 4.  The two lane
 // halves take alternate groups of four (the order of a contraction is free).
-template <int K, class AF, class BF>
+template <int K, bool STREAM = false, class AF, class BF>
 __device__ inline floatx16 product4(floatx16 acc, AF a4, BF b4) {
   const int h = (threadIdx.x % 64) / 32;
+  if constexpr (STREAM) {
 #pragma unroll 4
-  for (int k = 0; k < K; k += 8) {
-    const float4 x = a4(k + 4 * h), y = b4(k + 4 * h);
-    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.x, y.x, acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.y, y.y, acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.z, y.z, acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.w, y.w, acc, 0, 0, 0);
+    for (int k = 0; k < K; k += 8) {
+      const float4 x = a4(k + 4 * h), y = b4(k + 4 * h);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.x, y.x, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.y, y.y, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.z, y.z, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.w, y.w, acc, 0, 0, 0);
+    }
+    return acc;
   }
+  float4 av[K / 8], bv[K / 8];
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int s = 0; s < K / 8; ++s) {
+    av[s] = a4(8 * s + 4 * h);
+    bv[s] = b4(8 * s + 4 * h);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int s = 0; s < K / 8; ++s) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[s].x, bv[s].x, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[s].y, bv[s].y, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[s].z, bv[s].z, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[s].w, bv[s].w, acc, 0, 0, 0);
+  }
+  __builtin_amdgcn_sched_barrier(0);
   return acc;
 }
 
@@ -122,6 +167,13 @@ __device__ inline float4 load4(const float* p) { return *reinterpret_cast<const 
 
 __device__ inline float4 scaled(float4 v, float s) {
   return make_float4(v.x * s, v.y * s, v.z * s, v.w * s);
+}
+
+// Rows of tokens beyond the sequence read as zero: the load itself is always
+// made (from the last row), so that it needs no branch.
+__device__ inline float keep(bool ok, float v) { return ok ? v : 0.0f; }
+__device__ inline float4 keep(bool ok, float4 v) {
+  return make_float4(ok ? v.x : 0.0f, ok ? v.y : 0.0f, ok ? v.z : 0.0f, ok ? v.w : 0.0f);
 }
 
 __device__ inline float4 gather4(const float* p, int stride) {
@@ -262,8 +314,8 @@ chunk_prepare_kernel(ChunkedArgs a) {
       const floatx16 uacc = product<kC>(
           zero_tile(), [&](int k) { return tv[32 * ti + n][k]; },
           [&](int k) {
-            const int t = t0 + k;
-            return t < a.length ? a.post[static_cast<size_t>(t) * channels + value_offset + col] : 0.0f;
+            const int t = t0 + k, row = min(t, a.length - 1);
+            return keep(t < a.length, a.post[static_cast<size_t>(row) * channels + value_offset + col]);
           });
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
@@ -419,7 +471,7 @@ chunk_outputs_kernel(ChunkedArgs a) {
     floatx16 acc;
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[i] = U[(32 * ti + tile_row(i, h)) * kD + col];
-    acc = product4<kD>(acc, [&](int k) { return scaled(load4(W + m * kD + k), -1.0f); },
+    acc = product4<kD, true>(acc, [&](int k) { return scaled(load4(W + m * kD + k), -1.0f); },
                        [&](int k) { return gather4(S0 + k * kD + col, kD); });
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
@@ -427,7 +479,7 @@ chunk_outputs_kernel(ChunkedArgs a) {
       delta[row][col] = acc[i];
       a.r.dl[rec * kWide + row * kD + col] = acc[i];
     }
-    out[ti] = product4<kD>(zero_tile(), [&](int k) { return load4(Q + m * kD + k); },
+    out[ti] = product4<kD, true>(zero_tile(), [&](int k) { return load4(Q + m * kD + k); },
                            [&](int k) { return gather4(S0 + k * kD + col, kD); });
   }
   __syncthreads();
@@ -437,7 +489,7 @@ chunk_outputs_kernel(ChunkedArgs a) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) out[ti][i] *= e_s[32 * ti + tile_row(i, h)];
     // only columns j <= i of P are set: the second row tile needs all 64
-    out[ti] = product4<kC>(out[ti], [&](int k) { return load4(P + m * kC + k); },
+    out[ti] = product4<kC, true>(out[ti], [&](int k) { return load4(P + m * kC + k); },
                            [&](int k) {
                              return make_float4(delta[k][col], delta[k + 1][col], delta[k + 2][col],
                                                 delta[k + 3][col]);
@@ -467,8 +519,8 @@ chunk_local_kernel(ChunkedArgs a) {
     const floatx16 acc = product<kC>(
         zero_tile(), [&](int k) { return Y[k * kD + m]; },
         [&](int k) {
-          const int t = t0 + k;
-          return t < a.length ? a.dcore[(static_cast<size_t>(t) * a.vh + head) * kD + col] : 0.0f;
+          const int t = t0 + k, row = min(t, a.length - 1);
+          return keep(t < a.length, a.dcore[(static_cast<size_t>(row) * a.vh + head) * kD + col]);
         });
 #pragma unroll
     for (int i = 0; i < 16; ++i)
@@ -477,174 +529,200 @@ chunk_local_kernel(ChunkedArgs a) {
 }
 
 // ---------------------------------------------------------------------------
-// Sum over the 32 lanes of a half wave, into lane n == 0 of the half (and
-// every other lane of it).
-__device__ inline float half_sum(float v) { return wave_half_sum(v); }
+// The gradients of one chunk, in four kernels that exchange [64, 128] and
+// [64, 64] matrices through the records.  In each, wave w owns columns
+// 32w..32w+31 of the [64, 128] matrices (two 32-row tiles) or one 32 x 32 tile
+// of a [64, 64] matrix.
 
-// Gradients of one chunk: dDl = P^T dO + diag(L) K^ dS', then everything
-// the chunk's formulas feed.  Wave w owns columns 32w..32w+31 of the [64, 128]
-// matrices (two 32-row tiles each) and one 32 x 32 tile of every [64, 64]
-// intermediate.
+// Sums over the four waves of per-row partial sums left in parts[row][wave].
+__device__ inline float across_waves(const float (*parts)[4], int row) {
+  return (parts[row][0] + parts[row][1]) + (parts[row][2] + parts[row][3]);
+}
+
+struct ChunkView {
+  size_t rec;
+  int t0, head, channels;
+  size_t value_offset;
+  const float *gates, *S0, *dS1, *Dl, *Q, *K, *Tm, *P, *KKD;
+};
+
+__device__ inline ChunkView chunk_view(const ChunkedArgs& a, int chunk, int head) {
+  ChunkView v;
+  v.rec = static_cast<size_t>(head) * a.chunks + chunk;
+  v.t0 = chunk * kC;
+  v.head = head;
+  v.channels = 2 * a.kh * kD + a.vh * kD;
+  v.value_offset = 2 * static_cast<size_t>(a.kh) * kD + static_cast<size_t>(head) * kD;
+  v.gates = a.r.gates + v.rec * kGateRows * kC;
+  v.S0 = a.r.s0 + v.rec * kState;
+  v.dS1 = a.r.ds1 + v.rec * kState;
+  v.Dl = a.r.dl + v.rec * kWide;
+  v.Q = a.r.qn + v.rec * kWide;
+  v.K = a.r.kn + v.rec * kWide;
+  v.Tm = a.r.tm + v.rec * kSquare;
+  v.P = a.r.p + v.rec * kSquare;
+  v.KKD = a.r.kkd + v.rec * kSquare;
+  return v;
+}
+
+// Rows of dO and V; tokens beyond the sequence read as zero.
+__device__ inline float4 d_out4(const ChunkedArgs& a, const ChunkView& v, int i, int c) {
+  const int t = v.t0 + i, row = min(t, a.length - 1);
+  return keep(t < a.length, load4(a.dcore + (static_cast<size_t>(row) * a.vh + v.head) * kD + c));
+}
+__device__ inline float d_out1(const ChunkedArgs& a, const ChunkView& v, int i, int c) {
+  const int t = v.t0 + i, row = min(t, a.length - 1);
+  return keep(t < a.length, a.dcore[(static_cast<size_t>(row) * a.vh + v.head) * kD + c]);
+}
+__device__ inline float4 value4(const ChunkedArgs& a, const ChunkView& v, int j, int c) {
+  const int t = v.t0 + j, row = min(t, a.length - 1);
+  return keep(t < a.length, load4(a.post + static_cast<size_t>(row) * v.channels + v.value_offset + c));
+}
+__device__ inline float value1(const ChunkedArgs& a, const ChunkView& v, int j, int c) {
+  const int t = v.t0 + j, row = min(t, a.length - 1);
+  return keep(t < a.length, a.post[static_cast<size_t>(row) * v.channels + v.value_offset + c]);
+}
+
+// dDl = P^T dO + diag(L) K^ dS'
 __global__ void __launch_bounds__(256)
-chunk_gradients_kernel(ChunkedArgs a) {
-  __shared__ float dw[kC][kD + 1];
-  __shared__ __attribute__((aligned(16))) float ddl[kC][kD + 4];
-  __shared__ float mx[kC][kC + 1], my[kC][kC + 1], mz[kC][kC + 1], mu[kC][kC + 1];
-  __shared__ float g_s[kC], e_s[kC], l_s[kC], beta_s[kC], dg_s[kC];
-  __shared__ float row_parts[6][kC][4];
-  __shared__ float row_sums[4][kC];
+chunk_delta_gradient_kernel(ChunkedArgs a) {
+  const ChunkView v = chunk_view(a, blockIdx.x, blockIdx.y);
+  const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+  const int h = lane / 32, n = lane % 32, col = 32 * wave + n;
+#pragma unroll
+  for (int ti = 0; ti < 2; ++ti) {
+    const int m = 32 * ti + n;
+    floatx16 acc = product<kC, true>(zero_tile(), [&](int k) { return v.P[k * kC + m]; },
+                               [&](int k) { return d_out1(a, v, k, col); });
+    const float l = v.gates[5 * kC + m];
+    acc = product4<kD, true>(acc, [&](int k) { return scaled(load4(v.K + m * kD + k), l); },
+                       [&](int k) { return gather4(v.dS1 + k * kD + col, kD); });
+#pragma unroll
+    for (int i = 0; i < 16; ++i) a.r.ddl[v.rec * kWide + (32 * ti + tile_row(i, h)) * kD + col] = acc[i];
+  }
+}
+
+// Products against the two states, one per blockIdx.z:
+//   0: dW = -dDl S^T
+//   1: diag(E) dO S^T (the first part of dq^) and its row sums against q^
+//   2: diag(L) Dl dS'^T (the first part of dk^), its row sums against k^, <dS', S>
+__global__ void __launch_bounds__(256)
+chunk_state_products_kernel(ChunkedArgs a) {
+  __shared__ float parts[kC][4];
   __shared__ float reduce[256];
-  const int chunk = blockIdx.x, head = blockIdx.y;
-  const int key_head = head / (a.vh / a.kh);
-  (void)key_head;
-  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
-  const int h = lane / 32, n = lane % 32;
-  const int channels = 2 * a.kh * kD + a.vh * kD;
-  const size_t value_offset = 2 * static_cast<size_t>(a.kh) * kD + static_cast<size_t>(head) * kD;
-  const size_t rec = static_cast<size_t>(head) * a.chunks + chunk;
-  const int t0 = chunk * kC;
-  const float* gates = a.r.gates + rec * kGateRows * kC;
-  const float* S0 = a.r.s0 + rec * kState;
-  const float* dS1 = a.r.ds1 + rec * kState;
-  const float* Dl = a.r.dl + rec * kWide;
-  const float* Q = a.r.qn + rec * kWide;
-  const float* K = a.r.kn + rec * kWide;
-  const float* Tm = a.r.tm + rec * kSquare;
-  const float* P = a.r.p + rec * kSquare;
-  const float* KKD = a.r.kkd + rec * kSquare;
-  // rows of dO and V of tokens beyond the sequence are zero
-  auto dO4 = [&](int i, int c) {
-    const int t = t0 + i;
-    return t < a.length ? load4(a.dcore + (static_cast<size_t>(t) * a.vh + head) * kD + c)
-                        : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-  };
-  auto dO1 = [&](int i, int c) {
-    const int t = t0 + i;
-    return t < a.length ? a.dcore[(static_cast<size_t>(t) * a.vh + head) * kD + c] : 0.0f;
-  };
-  auto V4 = [&](int j, int c) {
-    const int t = t0 + j;
-    return t < a.length ? load4(a.post + static_cast<size_t>(t) * channels + value_offset + c)
-                        : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-  };
-  auto V1 = [&](int j, int c) {
-    const int t = t0 + j;
-    return t < a.length ? a.post[static_cast<size_t>(t) * channels + value_offset + c] : 0.0f;
-  };
-  if (tid < kC) {
-    const float g = gates[tid];
-    g_s[tid] = g;
-    e_s[tid] = gates[4 * kC + tid];
-    l_s[tid] = gates[5 * kC + tid];
-    beta_s[tid] = gates[kC + tid];
-  }
-  __syncthreads();
-  const int dcol = 32 * wave + n;
-
-  // ---- dDl = P^T dO + diag(L) K^ dS' ----------------------------------------
+  const ChunkView v = chunk_view(a, blockIdx.x, blockIdx.y);
+  const int which = blockIdx.z;
+  const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+  const int h = lane / 32, n = lane % 32, col = 32 * wave + n;
+  const float* dDl = a.r.ddl + v.rec * kWide;
+  float* sums = a.r.sums + v.rec * kSumRows * kC;
+  const float* state = which == 2 ? v.dS1 : v.S0;
+  float* target = (which == 0 ? a.r.dwm : which == 1 ? a.r.dqp : a.r.dkp) + v.rec * kWide;
+  const float* against = which == 1 ? v.Q : v.K;
 #pragma unroll
   for (int ti = 0; ti < 2; ++ti) {
     const int m = 32 * ti + n;
-    floatx16 acc = product<kC>(zero_tile(), [&](int k) { return P[k * kC + m]; },
-                               [&](int k) { return dO1(k, dcol); });
-    const float l = l_s[m];
-    acc = product4<kD>(acc, [&](int k) { return scaled(load4(K + m * kD + k), l); },
-                       [&](int k) { return gather4(dS1 + k * kD + dcol, kD); });
-#pragma unroll
-    for (int i = 0; i < 16; ++i) ddl[32 * ti + tile_row(i, h)][dcol] = acc[i];
-  }
-  __syncthreads();
-
-  // ---- products against the two states ------------------------------------
-  floatx16 dq[2], dk[2];
-#pragma unroll
-  for (int ti = 0; ti < 2; ++ti) {
-    const int m = 32 * ti + n;
-    // dW = -dDl S^T
-    const floatx16 dwt = product4<kD>(
-        zero_tile(), [&](int k) { return scaled(load4(&ddl[m][k]), -1.0f); },
-        [&](int k) { return load4(S0 + dcol * kD + k); });
-#pragma unroll
-    for (int i = 0; i < 16; ++i) dw[32 * ti + tile_row(i, h)][dcol] = dwt[i];
-    // d(diag(E) Q^) = dO S^T, times E
-    const float e = e_s[m];
-    dq[ti] = product4<kD>(zero_tile(), [&](int k) { return scaled(dO4(m, k), e); },
-                          [&](int k) { return load4(S0 + dcol * kD + k); });
-    // d(diag(L) K^) = Dl dS'^T, times L
-    const float l = l_s[m];
-    dk[ti] = product4<kD>(zero_tile(), [&](int k) { return scaled(load4(Dl + m * kD + k), l); },
-                          [&](int k) { return load4(dS1 + dcol * kD + k); });
+    const float factor = which == 0 ? -1.0f : v.gates[(which == 1 ? 4 : 5) * kC + m];
+    const floatx16 acc = product4<kD, true>(
+        zero_tile(),
+        [&](int k) {
+          const float4 row = which == 0   ? load4(dDl + m * kD + k)
+                             : which == 1 ? d_out4(a, v, m, k)
+                                          : load4(v.Dl + m * kD + k);
+          return scaled(row, factor);
+        },
+        [&](int k) { return load4(state + col * kD + k); });
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       const int row = 32 * ti + tile_row(i, h);
-      const float gq = half_sum(dq[ti][i] * Q[row * kD + dcol]);
-      const float g1 = half_sum(dk[ti][i] * K[row * kD + dcol]);
-      if (n == 0) {
-        row_parts[0][row][wave] = gq;
-        row_parts[1][row][wave] = g1;
+      target[row * kD + col] = acc[i];
+      if (which != 0) {
+        const float sum = wave_half_sum(acc[i] * against[row * kD + col]);
+        if (n == 0) parts[row][wave] = sum;
       }
     }
   }
-  // dP = lower(dO Dl^T): Pd = dP D and dP P
-  const int ti = wave / 2, tj = wave % 2;
-  {
-    floatx16 dp = zero_tile();
-    if (ti >= tj)
-      dp = product4<kD>(dp, [&](int k) { return dO4(32 * ti + n, k); },
-                        [&](int k) { return load4(Dl + (32 * tj + n) * kD + k); });
-    const int col = 32 * tj + n;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int row = 32 * ti + tile_row(i, h);
-      const bool keep = row >= col;
-      const float value = keep ? dp[i] : 0.0f;
-      my[row][col] = keep ? value * expf(g_s[row] - g_s[col]) : 0.0f;
-      mu[row][col] = value * P[row * kC + col];
-    }
-  }
-  // <dS', S>
-  {
+  if (which == 0) return;
+  if (which == 2) {
     float dot = 0.0f;
-    for (int idx = tid; idx < kState; idx += 256) dot += S0[idx] * dS1[idx];
+    for (int idx = tid; idx < kState; idx += 256) dot += v.S0[idx] * v.dS1[idx];
     reduce[tid] = dot;
   }
   __syncthreads();
+  if (tid < kC) sums[(which - 1) * kC + tid] = across_waves(parts, tid);
+  if (which == 2 && tid == 0) {
+    float dot = 0.0f;
+    for (int j = 0; j < 256; ++j) dot += reduce[j];
+    sums[6 * kC] = dot;
+  }
+}
 
-  // ---- dT = dW (diag(beta E) K^)^T + dDl (diag(beta) V)^T ------------------
-  {
-    const int j = 32 * tj + n;
-    const float fv = beta_s[j], fk = fv * e_s[j];
-    floatx16 acc = product<kD>(zero_tile(), [&](int k) { return dw[32 * ti + n][k]; },
-                               [&](int k) { return K[j * kD + k] * fk; });
-    acc = product4<kD>(acc, [&](int k) { return load4(&ddl[32 * ti + n][k]); },
-                       [&](int k) { return scaled(V4(j, k), fv); });
-#pragma unroll
-    for (int i = 0; i < 16; ++i) mx[32 * ti + tile_row(i, h)][j] = acc[i];
+// The [64, 64] part: dP = lower(dO Dl^T), dT = dW (diag(beta E) K^)^T +
+// dDl (diag(beta) V)^T, dA = -strict_lower(T^T dT T^T); leaves Pd = dP D and
+// R = diag(beta) dA D in the records, and the row and column sums that feed
+// d beta and d log-decay.
+__global__ void __launch_bounds__(256)
+chunk_triangle_kernel(ChunkedArgs a) {
+  __shared__ float mx[kC][kC + 1], mz[kC][kC + 1], mu[kC][kC + 1];
+  __shared__ float g_s[kC], beta_s[kC];
+  const ChunkView v = chunk_view(a, blockIdx.x, blockIdx.y);
+  const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+  const int h = lane / 32, n = lane % 32;
+  const int ti = wave / 2, tj = wave % 2;
+  const float* dDl = a.r.ddl + v.rec * kWide;
+  const float* dW = a.r.dwm + v.rec * kWide;
+  float* sums = a.r.sums + v.rec * kSumRows * kC;
+  if (tid < kC) {
+    g_s[tid] = v.gates[tid];
+    beta_s[tid] = v.gates[kC + tid];
   }
   __syncthreads();
-  // ---- X = T^T dT ----------------------------------------------------------
+  const int col = 32 * tj + n;
   {
-    const floatx16 acc = product<kC>(zero_tile(), [&](int k) { return Tm[k * kC + 32 * ti + n]; },
-                                     [&](int k) { return mx[k][32 * tj + n]; });
+    floatx16 dp = zero_tile();
+    if (ti >= tj)
+      dp = product4<kD>(dp, [&](int k) { return d_out4(a, v, 32 * ti + n, k); },
+                        [&](int k) { return load4(v.Dl + col * kD + k); });
 #pragma unroll
-    for (int i = 0; i < 16; ++i) mz[32 * ti + tile_row(i, h)][32 * tj + n] = acc[i];
+    for (int i = 0; i < 16; ++i) {
+      const int row = 32 * ti + tile_row(i, h);
+      const bool lower = row >= col;
+      const float value = lower ? dp[i] : 0.0f;
+      a.r.pd[v.rec * kSquare + row * kC + col] = lower ? value * expf(g_s[row] - g_s[col]) : 0.0f;
+      mu[row][col] = value * v.P[row * kC + col];
+    }
+  }
+  {
+    const float fv = beta_s[col], fk = fv * v.gates[4 * kC + col];
+    floatx16 acc = product4<kD>(zero_tile(), [&](int k) { return load4(dW + (32 * ti + n) * kD + k); },
+                                [&](int k) { return scaled(load4(v.K + col * kD + k), fk); });
+    acc = product4<kD>(acc, [&](int k) { return load4(dDl + (32 * ti + n) * kD + k); },
+                       [&](int k) { return scaled(value4(a, v, col, k), fv); });
+#pragma unroll
+    for (int i = 0; i < 16; ++i) mx[32 * ti + tile_row(i, h)][col] = acc[i];
   }
   __syncthreads();
-  // ---- dA = -strict_lower(X T^T) ------------------------------------------
+  {
+    const floatx16 acc = product<kC>(zero_tile(), [&](int k) { return v.Tm[k * kC + 32 * ti + n]; },
+                                     [&](int k) { return mx[k][col]; });
+#pragma unroll
+    for (int i = 0; i < 16; ++i) mz[32 * ti + tile_row(i, h)][col] = acc[i];
+  }
+  __syncthreads();
   {
     floatx16 acc = zero_tile();
     if (ti >= tj)
       acc = product<kC>(acc, [&](int k) { return -mz[32 * ti + n][k]; },
-                        [&](int k) { return Tm[(32 * tj + n) * kC + k]; });
+                        [&](int k) { return v.Tm[col * kC + k]; });
     __syncthreads();  // X has been read by every wave
-    const int col = 32 * tj + n;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       const int row = 32 * ti + tile_row(i, h);
-      const bool keep = row > col;
-      const float da = keep ? acc[i] : 0.0f;
-      mz[row][col] = da * KKD[row * kC + col];                                         // N
-      mx[row][col] = keep ? da * beta_s[row] * expf(g_s[row] - g_s[col]) : 0.0f;     // R
+      const bool lower = row > col;
+      const float da = lower ? acc[i] : 0.0f;
+      mz[row][col] = da * v.KKD[row * kC + col];  // N
+      a.r.rr[v.rec * kSquare + row * kC + col] =
+          lower ? da * beta_s[row] * expf(g_s[row] - g_s[col]) : 0.0f;
     }
   }
   __syncthreads();
@@ -657,103 +735,133 @@ chunk_gradients_kernel(ChunkedArgs a) {
       row_p += mu[tid][j];
       col_p += mu[j][tid];
     }
-    row_sums[0][tid] = row_n;
-    row_sums[1][tid] = col_m;
-    row_sums[2][tid] = row_p;
-    row_sums[3][tid] = col_p;
+    sums[2 * kC + tid] = row_n;
+    sums[3 * kC + tid] = col_m;
+    sums[4 * kC + tid] = row_p;
+    sums[5 * kC + tid] = col_p;
   }
+}
 
-  // ---- the three outputs ----------------------------------------------------
-#pragma unroll
-  for (int t2 = 0; t2 < 2; ++t2) {
-    const int m = 32 * t2 + n;
-    // dq^ += Pd K^
-    dq[t2] = product<kC>(dq[t2], [&](int k) { return my[m][k]; },
-                         [&](int k) { return K[k * kD + dcol]; });
-    // T^T dW: d(diag(beta E) K^)
-    const floatx16 tw = product<kC>(zero_tile(), [&](int k) { return Tm[k * kC + m]; },
-                                    [&](int k) { return dw[k][dcol]; });
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int row = 32 * t2 + tile_row(i, h);
-      const float r = half_sum(tw[i] * K[row * kD + dcol]) * e_s[row];
-      if (n == 0) row_parts[2][row][wave] = r;
-      dk[t2][i] += beta_s[row] * e_s[row] * tw[i];
-    }
-    // dk^ += (R + R^T) K^ + Pd^T Q^
-    dk[t2] = product<kC>(dk[t2], [&](int k) { return mx[m][k] + mx[k][m]; },
-                         [&](int k) { return K[k * kD + dcol]; });
-    dk[t2] = product<kC>(dk[t2], [&](int k) { return my[k][m]; },
-                         [&](int k) { return Q[k * kD + dcol]; });
-    // dv = diag(beta) T^T dDl
-    const floatx16 tu = product<kC>(zero_tile(), [&](int k) { return Tm[k * kC + m]; },
-                                    [&](int k) { return ddl[k][dcol]; });
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int row = 32 * t2 + tile_row(i, h), t = t0 + row;
-      const float rv = half_sum(tu[i] * V1(row, dcol));
-      const float q_dot = half_sum(dq[t2][i] * Q[row * kD + dcol]);
-      const float k_dot = half_sum(dk[t2][i] * K[row * kD + dcol]);
-      if (n == 0) {
-        row_parts[3][row][wave] = rv;
-        row_parts[4][row][wave] = q_dot;
-        row_parts[5][row][wave] = k_dot;
-      }
-      if (t < a.length) a.dpost[static_cast<size_t>(t) * channels + value_offset + dcol] = beta_s[row] * tu[i];
-    }
+// dq and dk (back through the normalisations) and dv of 32 rows of a chunk
+// (blockIdx.z picks the row tile), and the row sums of those rows that the
+// gate gradients need.
+__global__ void __launch_bounds__(256)
+chunk_finish_kernel(ChunkedArgs a) {
+  __shared__ float parts[4][kC / 2][4];
+  __shared__ float e_s[kC], beta_s[kC];
+  const ChunkView v = chunk_view(a, blockIdx.x, blockIdx.y);
+  const int ti = blockIdx.z;
+  const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+  const int h = lane / 32, n = lane % 32, col = 32 * wave + n;
+  const float* dDl = a.r.ddl + v.rec * kWide;
+  const float* dW = a.r.dwm + v.rec * kWide;
+  const float* Pd = a.r.pd + v.rec * kSquare;
+  const float* R = a.r.rr + v.rec * kSquare;
+  float* sums = a.r.sums + v.rec * kSumRows * kC;
+  if (tid < kC) {
+    e_s[tid] = v.gates[4 * kC + tid];
+    beta_s[tid] = v.gates[kC + tid];
   }
   __syncthreads();
-  auto parts = [&](int which, int row) {
-    return (row_parts[which][row][0] + row_parts[which][row][1]) +
-           (row_parts[which][row][2] + row_parts[which][row][3]);
-  };
+  const int m = 32 * ti + n;
+  floatx16 dq, dk;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int row = 32 * ti + tile_row(i, h);
+    dq[i] = a.r.dqp[v.rec * kWide + row * kD + col];
+    dk[i] = a.r.dkp[v.rec * kWide + row * kD + col];
+  }
+  // dq^ += Pd K^
+  dq = product4<kC>(dq, [&](int k) { return load4(Pd + m * kC + k); },
+                    [&](int k) { return gather4(v.K + k * kD + col, kD); });
+  // T^T dW = d(diag(beta E) K^)
+  const floatx16 tw = product<kC>(zero_tile(), [&](int k) { return v.Tm[k * kC + m]; },
+                                  [&](int k) { return dW[k * kD + col]; });
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int local = tile_row(i, h), row = 32 * ti + local;
+    const float r = wave_half_sum(tw[i] * v.K[row * kD + col]) * e_s[row];
+    if (n == 0) parts[0][local][wave] = r;
+    dk[i] += beta_s[row] * e_s[row] * tw[i];
+  }
+  // dk^ += (R + R^T) K^ + Pd^T Q^
+  dk = product4<kC>(dk, [&](int k) { return load4(R + m * kC + k); },
+                    [&](int k) { return gather4(v.K + k * kD + col, kD); });
+  dk = product<kC>(dk, [&](int k) { return R[k * kC + m]; },
+                   [&](int k) { return v.K[k * kD + col]; });
+  dk = product<kC>(dk, [&](int k) { return Pd[k * kC + m]; },
+                   [&](int k) { return v.Q[k * kD + col]; });
+  // dv = diag(beta) T^T dDl
+  const floatx16 tu = product<kC>(zero_tile(), [&](int k) { return v.Tm[k * kC + m]; },
+                                  [&](int k) { return dDl[k * kD + col]; });
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int local = tile_row(i, h), row = 32 * ti + local, t = v.t0 + row;
+    const float rv = wave_half_sum(tu[i] * value1(a, v, row, col));
+    const float q_dot = wave_half_sum(dq[i] * v.Q[row * kD + col]);
+    const float k_dot = wave_half_sum(dk[i] * v.K[row * kD + col]);
+    if (n == 0) {
+      parts[1][local][wave] = rv;
+      parts[2][local][wave] = q_dot;
+      parts[3][local][wave] = k_dot;
+    }
+    if (t < a.length)
+      a.dpost[static_cast<size_t>(t) * v.channels + v.value_offset + col] = beta_s[row] * tu[i];
+  }
+  __syncthreads();
   // back through the L2 normalisations (and the 1/sqrt(d) of q)
   const float norm_scale = sqrtf(static_cast<float>(kD));
 #pragma unroll
-  for (int t2 = 0; t2 < 2; ++t2)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int row = 32 * t2 + tile_row(i, h), t = t0 + row;
-      if (t >= a.length) continue;
-      const float iq = gates[2 * kC + row], ik = gates[3 * kC + row];
-      const float qv = Q[row * kD + dcol], kv = K[row * kD + dcol];
-      float* out = a.qk_partials + (static_cast<size_t>(t) * a.vh + head) * 2 * kD;
-      out[dcol] = iq / norm_scale * (dq[t2][i] - static_cast<float>(kD) * qv * parts(4, row));
-      out[kD + dcol] = ik * (dk[t2][i] - kv * parts(5, row));
-    }
-  // d log-decay and d beta
-  if (tid < kC) {
-    const float beta = beta_s[tid];
-    const float g1 = parts(1, tid), r = parts(2, tid);
-    float dG = parts(0, tid) + beta * r + (beta * row_sums[0][tid] - row_sums[1][tid]) +
-               (row_sums[2][tid] - row_sums[3][tid]) - g1;
-    if (tid == kC - 1) {
-      float total = 0.0f;
-      for (int j = 0; j < kC; ++j) total += parts(1, j);
-      float dot = 0.0f;
-      for (int j = 0; j < 256; ++j) dot += reduce[j];
-      dG += total + dot * e_s[kC - 1];
-    }
-    dg_s[tid] = dG;
+  for (int i = 0; i < 16; ++i) {
+    const int local = tile_row(i, h), row = 32 * ti + local, t = v.t0 + row;
+    if (t >= a.length) continue;
+    const float iq = v.gates[2 * kC + row], ik = v.gates[3 * kC + row];
+    const float qv = v.Q[row * kD + col], kv = v.K[row * kD + col];
+    float* out = a.qk_partials + (static_cast<size_t>(t) * a.vh + v.head) * 2 * kD;
+    out[col] = iq / norm_scale *
+               (dq[i] - static_cast<float>(kD) * qv * across_waves(parts[2], local));
+    out[kD + col] = ik * (dk[i] - kv * across_waves(parts[3], local));
   }
+  if (tid < kC / 2) {
+    sums[7 * kC + 32 * ti + tid] = across_waves(parts[0], tid);
+    sums[8 * kC + 32 * ti + tid] = across_waves(parts[1], tid);
+  }
+}
+
+// d log-decay and d beta of the 64 tokens of a chunk from the row and column
+// sums the other kernels left, then through the gates to da, db and the
+// contribution to d A_log.
+__global__ void __launch_bounds__(64)
+chunk_gates_kernel(ChunkedArgs a) {
+  __shared__ float dg_s[kC];
+  const ChunkView v = chunk_view(a, blockIdx.x, blockIdx.y);
+  const float* sums = a.r.sums + v.rec * kSumRows * kC;
+  const int tid = threadIdx.x;
+  const float beta = v.gates[kC + tid];
+  const float r = sums[7 * kC + tid];
+  float dG = sums[tid] + beta * r + (beta * sums[2 * kC + tid] - sums[3 * kC + tid]) +
+             (sums[4 * kC + tid] - sums[5 * kC + tid]) - sums[kC + tid];
+  if (tid == kC - 1) {
+    float total = 0.0f;
+    for (int j = 0; j < kC; ++j) total += sums[kC + j];
+    dG += total + sums[6 * kC] * v.gates[4 * kC + kC - 1];
+  }
+  dg_s[tid] = dG;
   __syncthreads();
-  if (tid < kC) {
-    const int t = t0 + tid;
-    if (t < a.length) {
-      float dg = 0.0f;
-      for (int i = kC - 1; i >= tid; --i) dg += dg_s[i];
-      const float dbeta = row_sums[0][tid] + parts(2, tid) + parts(3, tid);
-      const float alpha = bf16_bits_to_float(a.a[static_cast<size_t>(t) * a.vh + head]) + a.dt_bias[head];
-      const float softplus = fmaxf(alpha, 0.0f) + logf(1.0f + expf(-fabsf(alpha)));
-      const float rate = expf(a.a_log[head]);
-      const float bv = bf16_bits_to_float(a.b[static_cast<size_t>(t) * a.vh + head]);
-      const float sigmoid = 1.0f / (1.0f + expf(-bv));
-      float* out = a.scalar_partials + (static_cast<size_t>(t) * a.vh + head) * 3;
-      out[0] = -dg * rate / (1.0f + expf(-alpha));
-      out[1] = dbeta * sigmoid * (1.0f - sigmoid);
-      out[2] = -dg * rate * softplus;
-    }
-  }
+  const int t = v.t0 + tid;
+  if (t >= a.length) return;
+  float dg = 0.0f;
+  for (int i = kC - 1; i >= tid; --i) dg += dg_s[i];
+  const float dbeta = sums[2 * kC + tid] + r + sums[8 * kC + tid];
+  const float alpha = bf16_bits_to_float(a.a[static_cast<size_t>(t) * a.vh + v.head]) + a.dt_bias[v.head];
+  const float softplus = fmaxf(alpha, 0.0f) + logf(1.0f + expf(-fabsf(alpha)));
+  const float rate = expf(a.a_log[v.head]);
+  const float bv = bf16_bits_to_float(a.b[static_cast<size_t>(t) * a.vh + v.head]);
+  const float sigmoid = 1.0f / (1.0f + expf(-bv));
+  float* out = a.scalar_partials + (static_cast<size_t>(t) * a.vh + v.head) * 3;
+  out[0] = -dg * rate / (1.0f + expf(-alpha));
+  out[1] = dbeta * sigmoid * (1.0f - sigmoid);
+  out[2] = -dg * rate * softplus;
 }
 
 ChunkedArgs make_args(const GdnChunkedBackward& c) {
@@ -786,9 +894,16 @@ ChunkedArgs make_args(const GdnChunkedBackward& c) {
   a.r.u = take(kWide);
   a.r.y = take(kWide);
   a.r.dl = take(kWide);
+  a.r.ddl = take(kWide);
+  a.r.dwm = take(kWide);
+  a.r.dqp = take(kWide);
+  a.r.dkp = take(kWide);
   a.r.p = take(kSquare);
   a.r.tm = take(kSquare);
   a.r.kkd = take(kSquare);
+  a.r.pd = take(kSquare);
+  a.r.rr = take(kSquare);
+  a.r.sums = take(kSumRows * kC);
   a.r.gates = take(kGateRows * kC);
   a.r.m = take(kState);
   a.r.mt = take(kState);
@@ -836,7 +951,19 @@ int launch_gdn_backward_chunked_reverse(hipStream_t stream, const GdnChunkedBack
   chunk_states_kernel<true><<<a.vh * (kD / kSlice), 256, 0, stream>>>(a);
   status = launch_status();
   if (status != 0) return status;
-  chunk_gradients_kernel<<<per_chunk, 256, 0, stream>>>(a);
+  chunk_delta_gradient_kernel<<<per_chunk, 256, 0, stream>>>(a);
+  status = launch_status();
+  if (status != 0) return status;
+  chunk_state_products_kernel<<<dim3(a.chunks, a.vh, 3), 256, 0, stream>>>(a);
+  status = launch_status();
+  if (status != 0) return status;
+  chunk_triangle_kernel<<<per_chunk, 256, 0, stream>>>(a);
+  status = launch_status();
+  if (status != 0) return status;
+  chunk_finish_kernel<<<dim3(a.chunks, a.vh, 2), 256, 0, stream>>>(a);
+  status = launch_status();
+  if (status != 0) return status;
+  chunk_gates_kernel<<<per_chunk, kC, 0, stream>>>(a);
   return launch_status();
 }
 
