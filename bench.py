@@ -178,8 +178,9 @@ def gqa_prefill_bwd(torch, capi):
 
 
 def gdn_layer_bwd(torch, capi):
-    """Backward of the gated delta-net layer (token-serial FP32 kernels that keep
-    one state per token): a row after the headline ones, not part of --workload all."""
+    """Backward of the gated delta-net layer (FP32; 128 x 128 heads run in
+    64-token chunks on the FP32 matrix cores): a row after the headline ones, not
+    part of --workload all."""
     import numpy as np
     B, T, H, dk, dv, K = 1, 2048, 16, 128, 128, 4
     p = capi.delta_params(H, H, dk, dv, K)
@@ -199,14 +200,15 @@ def gdn_layer_bwd(torch, capi):
     def step():
         capi.gdn_layer_backward(p, qkv, z, a, b, conv, a_log, dt_bias, norm, dy)
 
-    # every per-token state is written once and read twice (as S_t and as S_{t+1})
-    work = 3.0 * B * (T + 1) * H * dk * dv * 4
+    # recurrence form, per token, head and state element: 7 FLOPs to repeat the
+    # forward (decay, prediction, update, output) and 15 for the reverse sweep
+    work = 22.0 * B * T * H * dk * dv
     return dict(step=step, parts=[("backward", step, work)], work=work,
-                metric="gdn_layer_backward_hbm_gbs", unit="GB/s", dtype="f32", bound="hbm",
-                peak=PEAK_HBM_GBS,
+                metric="gdn_layer_backward_tflops", unit="TFLOP/s", dtype="f32", bound="mfma",
+                peak=PEAK_FP32_TFLOPS,
                 config={"workload": "gated_delta_net_layer_backward", "batch": B, "seq_len": T,
                         "heads": H, "d_k": dk, "d_v": dv, "conv_kernel": K,
-                        "counted": "per-token state traffic (1 write + 2 reads)"},
+                        "counted": "22 dk dv FLOPs per token and head (recurrence form)"},
                 cpu=None)
 
 

@@ -34,8 +34,8 @@
 //   chunk_triangle_kernel          dP, dT, dA: the [64, 64] matrices  (parallel)
 //   chunk_finish_kernel            dq, dk, dv                         (parallel)
 //   chunk_gates_kernel             d beta, d log-decay -> da, db      (parallel)
-// The sequential kernels run one workgroup per (head, 32 value columns) and
-// do one 128 x 128 x 32 product a chunk, with the next chunk's matrix already
+// The sequential kernels run one workgroup per (head, 16 value columns) and
+// do one 128 x 128 x 16 product a chunk, with the next chunk's matrix already
 // in registers.  Matrix products run on v_mfma_f32_32x32x2_f32; operands are
 // read straight from global memory or from LDS.
 #include "gdn.h"
@@ -45,7 +45,7 @@ namespace {
 
 constexpr int kC = 64;       // tokens per chunk
 constexpr int kD = 128;      // key and value channels per head
-constexpr int kSlice = 32;   // value columns per workgroup of the sequential kernels
+constexpr int kSlice = 16;   // value columns per workgroup of the sequential kernels
 constexpr int kWide = kC * kD;     // elements of a [64, 128] record
 constexpr int kSquare = kC * kC;   // elements of a [64, 64] record
 constexpr int kState = kD * kD;    // elements of a state
@@ -391,7 +391,7 @@ chunk_transfer_kernel(ChunkedArgs a) {
 }
 
 // ---------------------------------------------------------------------------
-// next = matrix . state + offset over the chunks of one (head, 32 value
+// next = matrix . state + offset over the chunks of one (head, 16 value
 // columns): forward (REVERSE false) it stores the state entering every chunk,
 // with matrix M (read through its transpose) and offset B; in reverse it
 // stores the state gradient leaving every chunk, with matrix M^T (read through
@@ -404,44 +404,94 @@ chunk_states_kernel(ChunkedArgs a) {
   __shared__ float state[2][kD][kSlice];
   const int head = blockIdx.x / (kD / kSlice), col0 = (blockIdx.x % (kD / kSlice)) * kSlice;
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
-  const int h = lane / 32, n = lane % 32;
+  const int quarter = lane / 16, n = lane % 16;
   const float* matrices = REVERSE ? a.r.m : a.r.mt;
   const float* offsets = REVERSE ? a.r.cc : a.r.bc;
   float* saved = REVERSE ? a.r.ds1 : a.r.s0;
   auto record = [&](int step) {
     return static_cast<size_t>(head) * a.chunks + (REVERSE ? a.chunks - 1 - step : step);
   };
-  float matrix[kD / 2], next_matrix[kD / 2];
-  floatx16 offset, next_offset;
-  auto request = [&](int step, float* mat, floatx16& off) {
-    const size_t rec = record(step);
-    const float* source = matrices + rec * kState + 32 * wave + n;
-#pragma unroll
-    for (int s = 0; s < kD / 2; ++s) mat[s] = source[(2 * s + h) * kD];
-#pragma unroll
-    for (int i = 0; i < 16; ++i)
-      off[i] = offsets[rec * kState + (32 * wave + tile_row(i, h)) * kD + col0 + n];
+  // v_mfma_f32_16x16x4_f32: lane (quarter, n) supplies A[n][quarter] and
+  // B[quarter][n] and receives C[4 quarter + e][n], e = 0..3.  The wave's 32
+  // rows are two such tiles, interleaved (tile t holds rows 2i + t) so that a
+  // lane's two matrix elements of a step are neighbours in memory.
+  constexpr int kSteps = kD / 4;
+  struct Operands {
+    float2 matrix[kSteps];
+    floatx4 offset[2];
   };
-  request(0, matrix, offset);
-  floatx16 acc = zero_tile();
-  for (int step = 0; step < a.chunks; ++step) {
-    const size_t rec = record(step);
+  auto row_of = [&](int tile, int e) { return 32 * wave + 8 * quarter + 2 * e + tile; };
+  auto matrix_of = [&](int step) {
+    return matrices + record(min(step, a.chunks - 1)) * kState + 32 * wave + 2 * n + quarter * kD;
+  };
+  auto request_matrix = [&](const float* source, Operands& o, int s) {
+    o.matrix[s] = *reinterpret_cast<const float2*>(source + 4 * s * kD);
+  };
+  auto request_offset = [&](int step, Operands& o) {
+    const size_t rec = record(min(step, a.chunks - 1));
+#pragma unroll
+    for (int tile = 0; tile < 2; ++tile)
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        o.offset[tile][e] = offsets[rec * kState + row_of(tile, e) * kD + col0 + n];
+  };
+  auto request = [&](int step, Operands& o) {
+    const float* source = matrix_of(step);
+#pragma unroll
+    for (int s = 0; s < kSteps; ++s) request_matrix(source, o, s);
+    request_offset(step, o);
+  };
+  floatx4 acc[2];
+#pragma unroll
+  for (int tile = 0; tile < 2; ++tile)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) acc[tile][e] = 0.0f;
+  // One chunk: publish the state, multiply with the operands requested two
+  // chunks ago, request those of the chunk after next.  Three register sets
+  // take turns.  The requests are spread between the multiplications (their
+  // address arithmetic runs while the matrix pipe is busy) and come after the
+  // first of them in program order: the wait for this chunk's operands then
+  // has fewer than 64 younger memory operations behind it, which is as far as
+  // the counter reaches.  Requests are unconditional (past the end they repeat
+  // the last chunk's) so that the number in flight is the same on every path.
+  auto advance = [&](int step, const Operands& now, Operands& later) {
     float (*current)[kSlice] = state[step & 1];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int row = 32 * wave + tile_row(i, h);
-      current[row][n] = acc[i];
-      saved[rec * kState + row * kD + col0 + n] = acc[i];
+    for (int tile = 0; tile < 2; ++tile)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) current[row_of(tile, e)][n] = acc[tile][e];
+    if (step < a.chunks) {
+      const size_t rec = record(step);
+#pragma unroll
+      for (int tile = 0; tile < 2; ++tile)
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          saved[rec * kState + row_of(tile, e) * kD + col0 + n] = acc[tile][e];
     }
     lds_barrier();
-    if (step + 1 < a.chunks) request(step + 1, next_matrix, next_offset);
-    acc = offset;
+    acc[0] = now.offset[0];
+    acc[1] = now.offset[1];
+    const float* source = matrix_of(step + 2);
+    float b[kSteps];
 #pragma unroll
-    for (int s = 0; s < kD / 2; ++s)
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(matrix[s], current[2 * s + h][n], acc, 0, 0, 0);
+    for (int s = 0; s < kSteps; ++s) b[s] = current[4 * s + quarter][n];
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int s = 0; s < kD / 2; ++s) matrix[s] = next_matrix[s];
-    offset = next_offset;
+    for (int s = 0; s < kSteps; ++s) {
+      acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(now.matrix[s].x, b[s], acc[0], 0, 0, 0);
+      acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(now.matrix[s].y, b[s], acc[1], 0, 0, 0);
+      request_matrix(source, later, s);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    request_offset(step + 2, later);
+  };
+  Operands set0, set1, set2;
+  request(0, set0);
+  request(1, set1);
+  for (int step = 0; step < a.chunks; step += 3) {
+    advance(step, set0, set2);
+    advance(step + 1, set1, set0);
+    advance(step + 2, set2, set1);
   }
 }
 
