@@ -344,10 +344,12 @@ int pluto_hip_gdn_layer_forward(void* stream, const pluto_hip_delta_params* p,
  * (sequence_delta_net.cc:482-561; kernels OutputBackward :125-155,
  * RecurrenceBackward :171-253, the two gathers :255-305, the convolution
  * backward kernels :307-355).  Self-contained: it takes the layer's inputs and
- * repeats the forward pass, keeping the recurrent state after every token in
- * the workspace ((length + 1) * vh * kd * vd floats, as the reference's saved
- * state does), so it is meant for training-length sequences (length <= 65535
- * and as far as that scratch fits).  FP32 arithmetic, token by token.
+ * repeats the forward pass.  128 x 128 heads run in 64-token chunks on the
+ * FP32 matrix cores and keep one state per chunk (about 0.8 MB of workspace
+ * per chunk and value head); other head widths go token by token and keep the
+ * recurrent state after every token ((length + 1) * vh * kd * vd floats, as
+ * the reference's saved state does).  length <= 65535 and as far as the
+ * workspace fits.  FP32 arithmetic throughout.
  *   dy    fp32 [batch, length, vh*vd]
  *   dqkv  fp32 [batch, length, channels];  dz fp32 [batch, length, vh*vd]
  *   da, db  fp32 [batch, length, vh]

@@ -99,9 +99,10 @@ StatusOr<FwdResult> SequenceDeltaNetLayer::fwd_impl(hip::Executor& executor,
 }
 
 // src/llm/layers/sequence_delta_net.cc:482-561.  The library's backward entry
-// repeats the forward pass itself (keeping every per-token state in its
-// workspace, as the reference's saved state does), so the saved state only
-// supplies the four input handles.
+// repeats the forward pass itself (keeping the states it needs in its
+// workspace: one per 64-token chunk for 128 x 128 heads, one per token
+// otherwise, where the reference saves every per-token state), so the saved
+// state only supplies the four input handles.
 StatusOr<BufferVec> SequenceDeltaNetLayer::bwd_impl(hip::Executor& executor,
                                                     Span<const Buffer> gradients,
                                                     BackwardState state, LayerHooks*) {

@@ -7,7 +7,7 @@
 // sequence length up to kMaximumSequenceLength is accepted (the reference
 // stops at 128).  The per-token state snapshots the reference keeps for its
 // backward pass are not produced by forward: backward repeats the forward pass
-// token by token and keeps them in its own scratch.
+// and keeps the states it needs in its own scratch.
 #pragma once
 
 #include <memory>
