@@ -188,15 +188,25 @@ int pluto_hip_attention_params_validate(const pluto_hip_attention_params* p);
  *   q_norm, k_norm  fp32 [d], zero centred (multiplier 1 + w)
  *   out  bf16 [length, qh, d] = bf16(bf16(core) * bf16(sigmoid(gate)))
  *   lse  optional fp32 [length, qh]: max + log(normalizer) of each row
+ *   saved  optional, pluto_hip_gqa_prefill_saved_bytes(...) bytes: what
+ *        pluto_hip_gqa_prefill_backward would otherwise recompute (the
+ *        attention output before the gate and the row statistics; the
+ *        counterpart of the state SequenceForward hands to SequenceBackward,
+ *        qwen_attention.cc:445-447, without its quadratic tensors).  Only for
+ *        start_position 0 and where that size is not 0: round_to_bfloat16, a
+ *        BF16 cache and head_dim 64 or 128; PLUTO_HIP_EUNSUPPORTED otherwise.
  * The quadratic probability tensor of the reference is not produced. */
 size_t pluto_hip_gqa_prefill_workspace_bytes(const pluto_hip_attention_params* p,
                                              int length);
+size_t pluto_hip_gqa_prefill_saved_bytes(const pluto_hip_attention_params* p,
+                                         int length, int cache_dtype);
 int pluto_hip_gqa_prefill(void* stream, const pluto_hip_attention_params* p,
                           int length, int start_position, const void* qg,
                           const void* k, const void* v, const float* q_norm,
                           const float* k_norm,
                           const pluto_hip_kv_cache_view* cache, void* out,
-                          float* lse, void* workspace, size_t workspace_bytes);
+                          float* lse, void* saved, void* workspace,
+                          size_t workspace_bytes);
 
 /* Backward of the whole-sequence layer
  * (QwenAttentionLayer::SequenceBackward, qwen_attention.cc:450-499; kernels
@@ -206,6 +216,9 @@ int pluto_hip_gqa_prefill(void* stream, const pluto_hip_attention_params* p,
  * nothing quadratic (the reference saves probabilities and score gradients,
  * [qh, length, length] each) is kept between the passes.
  *   dy       fp32 [length, qh, d]     gradient of the layer output
+ *   saved    optional: the block pluto_hip_gqa_prefill filled for the same
+ *            inputs and parameters; the attention forward is then not repeated
+ *            (a quarter of the call at length 8192).  NULL recomputes.
  *   dqg      fp32 [length, qh, 2, d]  query gradients at [..,0,:], gate at [..,1,:]
  *   dk, dv   fp32 [length, kh, d]
  *   dq_norm, dk_norm  optional fp32 [d]: the norm weights' gradients are ADDED
@@ -221,10 +234,10 @@ size_t pluto_hip_gqa_prefill_backward_workspace_bytes(const pluto_hip_attention_
 int pluto_hip_gqa_prefill_backward(void* stream, const pluto_hip_attention_params* p,
                                    int length, const void* qg, const void* k,
                                    const void* v, const float* q_norm,
-                                   const float* k_norm, const float* dy, float* dqg,
-                                   float* dk, float* dv, float* dq_norm,
-                                   float* dk_norm, void* workspace,
-                                   size_t workspace_bytes);
+                                   const float* k_norm, const float* dy,
+                                   const void* saved, float* dqg, float* dk,
+                                   float* dv, float* dq_norm, float* dk_norm,
+                                   void* workspace, size_t workspace_bytes);
 
 /* The FP32 probabilities tensor of the same ForwardKernel
  * (qwen_attention.cc:68-119, reported to attention_probabilities_hook at

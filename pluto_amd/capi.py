@@ -91,15 +91,16 @@ SIGNATURES = {
                                     _VP, _VP, _SZ]),
     "pluto_hip_attention_params_validate": (_I, [ctypes.POINTER(AttentionParams)]),
     "pluto_hip_gqa_prefill_workspace_bytes": (_SZ, [ctypes.POINTER(AttentionParams), _I]),
+    "pluto_hip_gqa_prefill_saved_bytes": (_SZ, [ctypes.POINTER(AttentionParams), _I, _I]),
     "pluto_hip_gqa_prefill": (_I, [_VP, ctypes.POINTER(AttentionParams), _I, _I, _VP,
                                    _VP, _VP, _VP, _VP, ctypes.POINTER(KvCacheView),
-                                   _VP, _VP, _VP, _SZ]),
+                                   _VP, _VP, _VP, _VP, _SZ]),
     "pluto_hip_gqa_prefill_probabilities": (_I, [_VP, ctypes.POINTER(AttentionParams), _I, _I,
                                                  ctypes.POINTER(KvCacheView), _VP, _SZ, _VP]),
     "pluto_hip_gqa_prefill_backward_workspace_bytes": (_SZ, [ctypes.POINTER(AttentionParams), _I,
                                                              _I, _I]),
     "pluto_hip_gqa_prefill_backward": (_I, [_VP, ctypes.POINTER(AttentionParams), _I] +
-                                       [_VP] * 11 + [_VP, _SZ]),
+                                       [_VP] * 12 + [_VP, _SZ]),
     "pluto_hip_gqa_decode_workspace_bytes": (_SZ, [ctypes.POINTER(AttentionParams), _I,
                                                    ctypes.POINTER(_I), _I]),
     "pluto_hip_gqa_decode": (_I, [_VP, ctypes.POINTER(AttentionParams), _I, _I, _VP,
@@ -256,11 +257,19 @@ class KvCache:
         return (t.permute(1, 0, 2) if self.layout == "head_major" else t).contiguous().numpy()
 
 
+def gqa_prefill_saved(p, length, cache, device="cuda"):
+    """Buffer for the state gqa_prefill can leave for gqa_prefill_backward, or
+    None where the library keeps none (it then recomputes)."""
+    size = lib().pluto_hip_gqa_prefill_saved_bytes(ctypes.byref(p), length, cache.view().dtype)
+    return torch.empty(size, dtype=torch.uint8, device=device) if size else None
+
+
 def gqa_prefill(p, qg, k, v, q_norm, k_norm, cache, start_position=0, want_lse=False,
-                stream=None, want_probabilities=False):
+                stream=None, want_probabilities=False, saved=None):
     """qg bf16 [T, qh, 2, d]; k, v bf16 [T, kh, d]; norms fp32 [d].
 
-    want_probabilities appends fp32 [qh, T, start_position + T] to the result."""
+    want_probabilities appends fp32 [qh, T, start_position + T] to the result.
+    saved: a gqa_prefill_saved(...) buffer to fill for the backward pass."""
     T = qg.shape[0]
     out = torch.empty((T, p.query_heads, p.head_dim), dtype=torch.bfloat16, device=qg.device)
     lse = (torch.empty((T, p.query_heads), dtype=torch.float32, device=qg.device)
@@ -271,7 +280,7 @@ def gqa_prefill(p, qg, k, v, q_norm, k_norm, cache, start_position=0, want_lse=F
     check(lib().pluto_hip_gqa_prefill(stream or current_stream(), ctypes.byref(p), T,
                                       start_position, ptr(qg), ptr(k), ptr(v), ptr(q_norm),
                                       ptr(k_norm), ctypes.byref(view), ptr(out), ptr(lse),
-                                      ptr(workspace), size))
+                                      ptr(saved), ptr(workspace), size))
     cache.position = start_position + T
     result = (out, lse) if want_lse else out
     if want_probabilities:
@@ -285,10 +294,11 @@ def gqa_prefill(p, qg, k, v, q_norm, k_norm, cache, start_position=0, want_lse=F
 
 
 def gqa_prefill_backward(p, qg, k, v, q_norm, k_norm, dy, dq_norm=None, dk_norm=None,
-                         stream=None):
+                         stream=None, saved=None):
     """Gradients of the whole-sequence layer: (dqg fp32 [T, qh, 2, d], dk, dv fp32 [T, kh, d]).
 
-    dq_norm / dk_norm: optional fp32 [d] accumulators the norm-weight gradients are added to."""
+    dq_norm / dk_norm: optional fp32 [d] accumulators the norm-weight gradients are added to.
+    saved: the buffer gqa_prefill filled for the same inputs (skips the forward recomputation)."""
     T = qg.shape[0]
     dqg = torch.empty((T, p.query_heads, 2, p.head_dim), dtype=torch.float32, device=qg.device)
     dk = torch.empty((T, p.key_value_heads, p.head_dim), dtype=torch.float32, device=qg.device)
@@ -298,8 +308,8 @@ def gqa_prefill_backward(p, qg, k, v, q_norm, k_norm, dy, dq_norm=None, dk_norm=
     workspace = torch.empty(max(size, 1), dtype=torch.uint8, device=qg.device)
     check(lib().pluto_hip_gqa_prefill_backward(
         stream or current_stream(), ctypes.byref(p), T, ptr(qg), ptr(k), ptr(v), ptr(q_norm),
-        ptr(k_norm), ptr(dy), ptr(dqg), ptr(dk), ptr(dv), ptr(dq_norm), ptr(dk_norm),
-        ptr(workspace), size))
+        ptr(k_norm), ptr(dy), ptr(saved), ptr(dqg), ptr(dk), ptr(dv), ptr(dq_norm),
+        ptr(dk_norm), ptr(workspace), size))
     return dqg, dk, dv
 
 

@@ -17,6 +17,7 @@ struct FlashForwardArgs {
   long long v_seq_stride = 0, v_row_stride = 0, v_head_stride = 0;
   uint16_t* out = nullptr;
   long long o_seq_stride = 0, o_row_stride = 0, o_head_stride = 0;
+  uint16_t* core = nullptr;        // optional: the output before the gate, laid out like out
   const uint16_t* gate = nullptr;  // optional sigmoid gate logits
   long long gate_seq_stride = 0, gate_row_stride = 0, gate_head_stride = 0;
   float* maxima = nullptr;       // [(seq*QH + head)*q_rows + row]

@@ -324,6 +324,7 @@ flash_forward_kernel(FlashForwardArgs a) {
       const int row = q_row[g];
       if (row < a.q_rows) {
         uint16_t* o_row = o_base + static_cast<long long>(row) * a.o_row_stride;
+        uint16_t* core_row = a.core ? a.core + (o_row - a.out) : nullptr;
         const uint16_t* gate_row =
             gate_base ? gate_base + static_cast<long long>(row) * a.gate_row_stride : nullptr;
 #pragma unroll
@@ -334,6 +335,12 @@ flash_forward_kernel(FlashForwardArgs a) {
             float c[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) c[e] = o_acc[g][db][4 * j + e] * inverse;
+            if (core_row) {
+              uint2 plain;
+              plain.x = pack_bf16(c[0], c[1]);
+              plain.y = pack_bf16(c[2], c[3]);
+              *reinterpret_cast<uint2*>(core_row + d) = plain;
+            }
             if (gate_row) {
               // out = bf16(bf16(core) * bf16(sigmoid(gate))): qwen_attention.cc:103-108
               const uint2 gate_bits = *reinterpret_cast<const uint2*>(gate_row + d);

@@ -109,6 +109,26 @@ long long decode_blocks(int batch, const int* positions, int split) {
   return blocks;
 }
 
+// What the forward pass can leave for the backward pass: the attention output
+// before the gate (bf16 [length, qh * d]) and the two row statistics (fp32
+// [qh, length] each), as the matrix-core backward kernels read them.
+struct SavedLayout {
+  size_t core, maxima, normalizers, total;
+};
+SavedLayout saved_layout(const pluto_hip_attention_params* p, int length) {
+  SavedLayout l{};
+  const size_t rows = static_cast<size_t>(length) * p->query_heads;
+  l.core = 0;
+  l.maxima = align_up(rows * p->head_dim * 2, 256);
+  l.normalizers = l.maxima + align_up(rows * 4, 256);
+  l.total = l.normalizers + align_up(rows * 4, 256);
+  return l;
+}
+bool saved_supported(const pluto_hip_attention_params* p, int cache_dtype) {
+  return p->round_to_bfloat16 && cache_dtype == PLUTO_HIP_BF16 &&
+         (p->head_dim == 64 || p->head_dim == 128) && !force_generic();
+}
+
 }  // namespace
 }  // namespace pluto_hip
 
@@ -125,11 +145,17 @@ size_t pluto_hip_gqa_prefill_workspace_bytes(const pluto_hip_attention_params* p
   return prefill_layout(p, length).total;
 }
 
+size_t pluto_hip_gqa_prefill_saved_bytes(const pluto_hip_attention_params* p, int length,
+                                         int cache_dtype) {
+  if (validate_params(p) != 0 || length <= 0 || !saved_supported(p, cache_dtype)) return 0;
+  return saved_layout(p, length).total;
+}
+
 int pluto_hip_gqa_prefill(void* stream, const pluto_hip_attention_params* p, int length,
                           int start_position, const void* qg, const void* k, const void* v,
                           const float* q_norm, const float* k_norm,
                           const pluto_hip_kv_cache_view* cache, void* out, float* lse,
-                          void* workspace, size_t workspace_bytes) {
+                          void* saved, void* workspace, size_t workspace_bytes) {
   int status = validate_params(p);
   if (status != 0) return status;
   if (length <= 0 || start_position < 0) return PLUTO_HIP_EINVAL;
@@ -138,6 +164,9 @@ int pluto_hip_gqa_prefill(void* stream, const pluto_hip_attention_params* p, int
   if (status != 0) return status;
   // cached_attention_ops.cc:318-320: appending beyond capacity fails first.
   if (static_cast<long long>(start_position) + length > p->capacity) return PLUTO_HIP_ERANGE;
+  // the saved state describes a whole sequence attended from position 0
+  if (saved && (start_position != 0 || !saved_supported(p, cache->dtype)))
+    return PLUTO_HIP_EUNSUPPORTED;
   const PrefillLayout layout = prefill_layout(p, length);
   if (!workspace || workspace_bytes < layout.total) return PLUTO_HIP_EWORKSPACE;
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -192,6 +221,12 @@ int pluto_hip_gqa_prefill(void* stream, const pluto_hip_attention_params* p, int
     f.gate_row_stride = 2LL * qh * d;
     f.gate_head_stride = 2LL * d;
     f.lse = lse;
+    if (saved) {
+      const SavedLayout sl = saved_layout(p, length);
+      f.core = reinterpret_cast<uint16_t*>(static_cast<char*>(saved) + sl.core);
+      f.maxima = reinterpret_cast<float*>(static_cast<char*>(saved) + sl.maxima);
+      f.normalizers = reinterpret_cast<float*>(static_cast<char*>(saved) + sl.normalizers);
+    }
     f.q_rows = length;
     f.kv_rows = start_position + length;
     f.start_position = start_position;
@@ -199,6 +234,7 @@ int pluto_hip_gqa_prefill(void* stream, const pluto_hip_attention_params* p, int
     f.group = qh / kh;
     f.scale = scale;
     if (flash_forward_supported(f, d)) return launch_flash_forward(s, f, d, 1);
+    if (saved) return PLUTO_HIP_EUNSUPPORTED;
   }
   GenericForwardArgs a;
   a.q = {queries, 0, 1LL * qh * d, d, prep.q_out_dtype};
@@ -231,8 +267,9 @@ size_t pluto_hip_gqa_prefill_backward_workspace_bytes(const pluto_hip_attention_
 int pluto_hip_gqa_prefill_backward(void* stream, const pluto_hip_attention_params* p, int length,
                                    const void* qg, const void* k, const void* v,
                                    const float* q_norm, const float* k_norm, const float* dy,
-                                   float* dqg, float* dk, float* dv, float* dq_norm,
-                                   float* dk_norm, void* workspace, size_t workspace_bytes) {
+                                   const void* saved, float* dqg, float* dk, float* dv,
+                                   float* dq_norm, float* dk_norm, void* workspace,
+                                   size_t workspace_bytes) {
   int status = validate_params(p);
   if (status != 0) return status;
   if (length <= 0) return PLUTO_HIP_EINVAL;
@@ -241,6 +278,7 @@ int pluto_hip_gqa_prefill_backward(void* stream, const pluto_hip_attention_param
                                                           dk_norm != nullptr);
   if (l.attention_bytes == 0) return PLUTO_HIP_EINVAL;
   if (!workspace || workspace_bytes < l.total) return PLUTO_HIP_EWORKSPACE;
+  if (saved && l.dtype != PLUTO_HIP_BF16) return PLUTO_HIP_EUNSUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
   char* scratch = static_cast<char*>(workspace);
   float* cosines = reinterpret_cast<float*>(scratch + l.cosines);
@@ -250,8 +288,8 @@ int pluto_hip_gqa_prefill_backward(void* stream, const pluto_hip_attention_param
   const int E = qh * d;
 
   // Recompute what the forward pass derived from the inputs: normalised,
-  // rotated q and k (PrepareKernel, qwen_attention.cc:30-63), then the
-  // attention core with its row statistics.
+  // rotated q and k (PrepareKernel, qwen_attention.cc:30-63), then -- unless
+  // the forward pass saved them -- the attention core with its row statistics.
   status = launch_rope_table(s, 0, length, p->rotary_dim, p->rope_theta, round, cosines, sines);
   if (status != 0) return status;
   PrefillPrepareArgs prep;
@@ -278,17 +316,28 @@ int pluto_hip_gqa_prefill_backward(void* stream, const pluto_hip_attention_param
   status = launch_pack_heads(s, scratch + l.queries, scratch + l.keys, scratch + l.values, l.dtype,
                              length, qh, kh, d, scratch + l.packed);
   if (status != 0) return status;
-  float* maxima = reinterpret_cast<float*>(scratch + l.maxima);
-  float* normalizers = reinterpret_cast<float*>(scratch + l.normalizers);
-  status = pluto_hip_mha_forward(stream, l.dtype, scratch + l.packed, length, length, qh, E,
-                                 scratch + l.core, maxima, normalizers);
-  if (status != 0) return status;
+  const void* core = scratch + l.core;
+  const float* maxima = reinterpret_cast<const float*>(scratch + l.maxima);
+  const float* normalizers = reinterpret_cast<const float*>(scratch + l.normalizers);
+  if (saved) {
+    const SavedLayout sl = saved_layout(p, length);
+    const char* base = static_cast<const char*>(saved);
+    core = base + sl.core;
+    maxima = reinterpret_cast<const float*>(base + sl.maxima);
+    normalizers = reinterpret_cast<const float*>(base + sl.normalizers);
+  } else {
+    status = pluto_hip_mha_forward(stream, l.dtype, scratch + l.packed, length, length, qh, E,
+                                   scratch + l.core,
+                                   reinterpret_cast<float*>(scratch + l.maxima),
+                                   reinterpret_cast<float*>(scratch + l.normalizers));
+    if (status != 0) return status;
+  }
 
   float* dc = reinterpret_cast<float*>(scratch + l.dc);
-  status = launch_gate_backward(s, qg, scratch + l.core, l.dtype, dy, length, qh, d, round, dc, dqg);
+  status = launch_gate_backward(s, qg, core, l.dtype, dy, length, qh, d, round, dc, dqg);
   if (status != 0) return status;
   float* d_packed = reinterpret_cast<float*>(scratch + l.d_packed);
-  status = pluto_hip_mha_backward(stream, l.dtype, scratch + l.packed, scratch + l.core, dc, maxima,
+  status = pluto_hip_mha_backward(stream, l.dtype, scratch + l.packed, core, dc, maxima,
                                   normalizers, length, length, qh, E, d_packed,
                                   scratch + l.attention, l.attention_bytes);
   if (status != 0) return status;

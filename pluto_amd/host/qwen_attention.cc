@@ -174,11 +174,18 @@ StatusOr<FwdResult> QwenAttentionLayer::SequenceForward(hip::Executor& executor,
   ASSIGN_OR_RETURN(auto workspace, Buffer::Allocate(executor, workspace_bytes));
   ASSIGN_OR_RETURN(auto output, Buffer::Allocate(executor, 2 * qn));
   ASSIGN_OR_RETURN(auto lse, Buffer::Allocate(executor, static_cast<size_t>(t) * qh * 4));
+  // What the backward pass would otherwise recompute (the attention output
+  // before the gate and its row statistics), where the library keeps it; an
+  // empty buffer stands for "recompute".
+  const size_t saved_bytes = pluto_hip_gqa_prefill_saved_bytes(&abi, t, view.dtype);
+  ASSIGN_OR_RETURN(auto saved, Buffer::Allocate(executor, saved_bytes));
   RETURN_IF_ERROR(hip::HipStatus(
       pluto_hip_gqa_prefill(executor.stream(), &abi, t, 0, inputs[0].data(), inputs[1].data(),
                             inputs[2].data(), static_cast<const float*>(weights_[0].data()),
                             static_cast<const float*>(weights_[1].data()), &view, output.data(),
-                            static_cast<float*>(lse.data()), workspace.data(), workspace_bytes),
+                            static_cast<float*>(lse.data()),
+                            saved_bytes ? saved.data() : nullptr, workspace.data(),
+                            workspace_bytes),
       "sequence full attention forward"));
   if (hooks && hooks->attention_probabilities_hook) {
     ASSIGN_OR_RETURN(auto probabilities,
@@ -193,17 +200,19 @@ StatusOr<FwdResult> QwenAttentionLayer::SequenceForward(hip::Executor& executor,
   }
   BackwardState state;
   state.intermediates = {inputs[0], inputs[1], inputs[2], std::move(keys), std::move(values),
-                         std::move(lse)};
+                         std::move(lse), std::move(saved)};
   return FwdResult{{std::move(output)}, std::move(state)};
 }
 
-// src/llm/layers/qwen_attention.cc:450-499.  The library's backward entry is
-// self-contained (it recomputes what the forward pass derived from the
-// inputs), so only the three input handles of the saved state are used.
+// src/llm/layers/qwen_attention.cc:450-499.  The library's backward entry
+// recomputes what the forward pass derived from the inputs except for the
+// attention output and its row statistics, which it takes from the saved
+// block when forward could fill one: the three input handles and that block
+// are what is used of the saved state.
 StatusOr<BufferVec> QwenAttentionLayer::SequenceBackward(hip::Executor& executor,
                                                          Span<const Buffer> gradients,
                                                          BackwardState state) {
-  if (&executor != &executor_ || state.intermediates.size() != 6)
+  if (&executor != &executor_ || state.intermediates.size() != 7)
     return InvalidArgumentError("sequence attention backward Executor/state mismatch");
   const auto& p = parameters_;
   const int t = sequence_length_, d = p.head_dim, qh = p.query_heads, kh = p.key_value_heads;
@@ -226,7 +235,8 @@ StatusOr<BufferVec> QwenAttentionLayer::SequenceBackward(hip::Executor& executor
           executor.stream(), &abi, t, s[0].data(), s[1].data(), s[2].data(),
           static_cast<const float*>(weights_[0].data()),
           static_cast<const float*>(weights_[1].data()),
-          static_cast<const float*>(gradients[0].data()), static_cast<float*>(dqg.data()),
+          static_cast<const float*>(gradients[0].data()),
+          s[6].size_bytes() ? s[6].data() : nullptr, static_cast<float*>(dqg.data()),
           static_cast<float*>(dk.data()), static_cast<float*>(dv.data()),
           q_active ? static_cast<float*>(q_norm_->gradient().data()) : nullptr,
           k_active ? static_cast<float*>(k_norm_->gradient().data()) : nullptr, workspace.data(),

@@ -96,6 +96,58 @@ def test_matrix_core_kernels_match_oracle(capi, shape):
         assert_close_bf16(got[name], want[name], "%s T%d d%d" % (name, T, d))
 
 
+@pytest.mark.parametrize("shape", [(200, 8, 2, 64, 32), (333, 6, 2, 128, 64)])
+def test_state_saved_by_forward_gives_the_recomputed_gradients(capi, shape):
+    """pluto_hip_gqa_prefill can leave the attention output before the gate and
+    the row statistics for the backward pass (the role of the state
+    SequenceForward hands to SequenceBackward, qwen_attention.cc:445-447); the
+    gradients must be those of the self-contained call."""
+    T, qh, kh, d, rot = shape
+    got, want, args, _ = run_case(capi, T, qh, kh, d, rot, True, seed=T)
+    p, qg, k, v, qw, kw_, dy = args
+    cache = capi.KvCache(T, kh, d)
+    saved = capi.gqa_prefill_saved(p, T, cache)
+    assert saved is not None and saved.numel() >= T * qh * (2 * d + 8)
+    capi.gqa_prefill(p, qg, k, v, qw, kw_, cache, saved=saved)
+    dq_norm, dk_norm = torch.zeros(d, device="cuda"), torch.zeros(d, device="cuda")
+    dqg, dk, dv = capi.gqa_prefill_backward(p, qg, k, v, qw, kw_, dy, dq_norm=dq_norm,
+                                            dk_norm=dk_norm, saved=saved)
+    torch.cuda.synchronize()
+    with_saved = dict(dqg=dqg, dk=dk, dv=dv, dq_norm=dq_norm, dk_norm=dk_norm)
+    for name, value in with_saved.items():
+        # same kernels, same operands: the forward pass of the two calls differs
+        # only in where K and V are read from
+        np.testing.assert_allclose(value.cpu().numpy(), got[name], rtol=1e-5, atol=1e-6,
+                                   err_msg=name)
+        assert_close_bf16(value.cpu().numpy(), want[name], "%s T%d d%d" % (name, T, d))
+
+
+def test_saved_state_is_refused_where_none_is_kept(capi):
+    T, qh, kh, d, rot = 16, 2, 1, 32, 8
+    kw = dict(query_heads=qh, key_value_heads=kh, head_dim=d, rotary_dim=rot, capacity=T,
+              round_to_bfloat16=True)
+    p = capi.attention_params(**kw)
+    cache = capi.KvCache(T, kh, d)
+    assert capi.gqa_prefill_saved(p, T, cache) is None  # head width without matrix-core backward
+    lib = capi.lib()
+    import ctypes
+    fp32 = capi.attention_params(**dict(kw, head_dim=64, rotary_dim=16, round_to_bfloat16=False))
+    assert lib.pluto_hip_gqa_prefill_saved_bytes(ctypes.byref(fp32), T, capi.BF16) == 0
+    wide = capi.attention_params(**dict(kw, head_dim=64, rotary_dim=16))
+    assert lib.pluto_hip_gqa_prefill_saved_bytes(ctypes.byref(wide), T, capi.F32) == 0
+    assert lib.pluto_hip_gqa_prefill_saved_bytes(ctypes.byref(wide), T, capi.BF16) > 0
+    # a block offered where none can be filled is an error, not silently ignored
+    qg = torch.zeros((T, qh, 2, d), dtype=torch.bfloat16, device="cuda")
+    k = torch.zeros((T, kh, d), dtype=torch.bfloat16, device="cuda")
+    w = torch.zeros(d, device="cuda")
+    bogus = torch.empty(1 << 16, dtype=torch.uint8, device="cuda")
+    with pytest.raises(capi.PlutoHipError):
+        capi.gqa_prefill(p, qg, k, k, w, w, cache, saved=bogus)
+    dy = torch.zeros((T, qh, d), device="cuda")
+    with pytest.raises(capi.PlutoHipError):
+        capi.gqa_prefill_backward(p, qg, k, k, w, w, dy, saved=bogus)
+
+
 def test_weight_gradients_accumulate_and_are_optional(capi):
     T, qh, kh, d, rot = 5, 2, 1, 8, 4
     got, want, args, (dq_norm, dk_norm) = run_case(capi, T, qh, kh, d, rot, True)
@@ -140,11 +192,11 @@ def test_rejects_bad_arguments_before_touching_outputs(capi):
     x = torch.zeros(1024, device="cuda")
     rc = lib.pluto_hip_gqa_prefill_backward(capi.current_stream(), ctypes.byref(p), 3, capi.ptr(x),
                                             capi.ptr(x), capi.ptr(x), capi.ptr(x), capi.ptr(x),
-                                            capi.ptr(x), capi.ptr(x), capi.ptr(x), capi.ptr(x),
+                                            capi.ptr(x), None, capi.ptr(x), capi.ptr(x), capi.ptr(x),
                                             None, None, capi.ptr(x), 16)
     assert rc == capi.EWORKSPACE if hasattr(capi, "EWORKSPACE") else rc != 0
     rc = lib.pluto_hip_gqa_prefill_backward(capi.current_stream(), ctypes.byref(p), 3, None,
                                             capi.ptr(x), capi.ptr(x), capi.ptr(x), capi.ptr(x),
-                                            capi.ptr(x), capi.ptr(x), capi.ptr(x), capi.ptr(x),
+                                            capi.ptr(x), None, capi.ptr(x), capi.ptr(x), capi.ptr(x),
                                             None, None, capi.ptr(x), size)
     assert rc != 0
