@@ -204,8 +204,13 @@ def gdn_layer_bwd(torch, capi):
     norm = torch.ones(dv, device="cuda")
     dy = torch.randn((B, T, H * dv), generator=gen, device="cuda")
 
+    # every parameter trains: the four parameter gradients are part of the call
+    grads = dict(conv_weight=torch.zeros_like(conv), a_log=torch.zeros_like(a_log),
+                 dt_bias=torch.zeros_like(dt_bias), norm=torch.zeros_like(norm))
+
     def step():
-        capi.gdn_layer_backward(p, qkv, z, a, b, conv, a_log, dt_bias, norm, dy)
+        capi.gdn_layer_backward(p, qkv, z, a, b, conv, a_log, dt_bias, norm, dy,
+                                parameter_grads=grads)
 
     # recurrence form, per token, head and state element: 7 FLOPs to repeat the
     # forward (decay, prediction, update, output) and 15 for the reverse sweep

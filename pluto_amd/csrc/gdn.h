@@ -96,7 +96,7 @@ int launch_gdn_backward_chunked_reverse(hipStream_t stream, const GdnChunkedBack
 // Backward of the whole layer for one sequence (gdn_backward.hip): the forward
 // pass is repeated with the states it needs kept in `workspace` (one per
 // 64-token chunk for 128 x 128 heads, one per token otherwise).
-constexpr int kGdnSumChunks = 128;
+constexpr int kGdnSumChunks = 512;
 size_t gdn_backward_workspace_bytes(const pluto_hip_delta_params* p, int length, bool norm_grad);
 int launch_gdn_backward(hipStream_t stream, const pluto_hip_delta_params* p, int length,
                         const void* qkv, const void* z, const void* a, const void* b,

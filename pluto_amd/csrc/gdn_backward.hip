@@ -11,7 +11,7 @@
 //   gather_scalar_kernel         GatherScalarGradient   (:278-305)
 //   conv_silu_backward_kernel    ConvSiluBackward       (:307-318)
 //   conv_input_backward_kernel   ConvInputBackward      (:320-336)
-//   conv_weight_backward_kernel  ConvWeightBackward     (:338-355)
+//   conv_weight_*_kernel         ConvWeightBackward     (:338-355), two levels
 //   sum_rows_*_kernel            SumNormGradient        (:157-166), two levels
 //
 // The two recurrence kernels share one layout: a workgroup owns the
@@ -30,25 +30,75 @@ constexpr int kRows = 16;        // state rows per thread
 constexpr int kGroups = 8;       // row groups per workgroup
 constexpr int kColumns = 32;     // state columns per workgroup
 constexpr int kMaxKey = kRows * kGroups;  // 128
+constexpr int kConvSlices = 64;  // token slices of the convolution weight gradient
 
 __device__ inline float round_if(float x, bool round) { return round ? round_to_bf16(x) : x; }
 
+// VEC consecutive elements of a row as one access (VEC is 1 or 4).
+template <int VEC>
+struct Pack {
+  float e[VEC];
+};
+template <int VEC>
+__device__ inline Pack<VEC> load_floats(const float* p) {
+  Pack<VEC> r;
+  if constexpr (VEC == 4) {
+    const float4 v = *reinterpret_cast<const float4*>(p);
+    r.e[0] = v.x; r.e[1] = v.y; r.e[2] = v.z; r.e[3] = v.w;
+  } else {
+    r.e[0] = p[0];
+  }
+  return r;
+}
+template <int VEC>
+__device__ inline void store_floats(float* p, const Pack<VEC>& v) {
+  if constexpr (VEC == 4)
+    *reinterpret_cast<float4*>(p) = make_float4(v.e[0], v.e[1], v.e[2], v.e[3]);
+  else
+    p[0] = v.e[0];
+}
+template <int VEC>
+__device__ inline Pack<VEC> load_bf16s(const uint16_t* p) {
+  Pack<VEC> r;
+  if constexpr (VEC == 4) {
+    const uint2 bits = *reinterpret_cast<const uint2*>(p);
+    r.e[0] = __uint_as_float(bits.x << 16);
+    r.e[1] = __uint_as_float(bits.x & 0xffff0000u);
+    r.e[2] = __uint_as_float(bits.y << 16);
+    r.e[3] = __uint_as_float(bits.y & 0xffff0000u);
+  } else {
+    r.e[0] = bf16_bits_to_float(p[0]);
+  }
+  return r;
+}
+
+// One thread per VEC channels of a token (channels % VEC == 0).
+template <int VEC>
 __global__ void __launch_bounds__(256)
 conv_train_kernel(const uint16_t* input, const float* __restrict__ weight, int length,
                   int channels, int kernel, bool round, float* pre, float* post) {
-  const long long total = 1LL * length * channels;
+  const int groups = channels / VEC;
   const long long i = blockIdx.x * 256LL + threadIdx.x;
-  if (i >= total) return;
-  const int c = static_cast<int>(i % channels), t = static_cast<int>(i / channels);
-  float sum = 0.0f;
+  if (i >= 1LL * length * groups) return;
+  const int c = static_cast<int>(i % groups) * VEC, t = static_cast<int>(i / groups);
+  Pack<VEC> sum;
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) sum.e[e] = 0.0f;
   for (int tap = 0; tap < kernel; ++tap) {
     const int source = t + tap - kernel + 1;
-    if (source >= 0)
-      sum += bf16_bits_to_float(input[1LL * source * channels + c]) * weight[1LL * c * kernel + tap];
+    if (source < 0) continue;
+    const Pack<VEC> x = load_bf16s<VEC>(input + 1LL * source * channels + c);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) sum.e[e] += x.e[e] * weight[1LL * (c + e) * kernel + tap];
   }
-  sum = round_if(sum, round);
-  pre[i] = sum;
-  post[i] = round_if(sum / (1.0f + expf(-sum)), round);
+  Pack<VEC> activated;
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) {
+    sum.e[e] = round_if(sum.e[e], round);
+    activated.e[e] = round_if(sum.e[e] / (1.0f + expf(-sum.e[e])), round);
+  }
+  store_floats<VEC>(pre + 1LL * t * channels + c, sum);
+  store_floats<VEC>(post + 1LL * t * channels + c, activated);
 }
 
 struct RecurrenceArgs {
@@ -427,61 +477,103 @@ gather_scalar_kernel(const float* partials, int length, int vh, int tiles, float
   }
 }
 
+template <int VEC>
 __global__ void __launch_bounds__(256)
 conv_silu_backward_kernel(const float* pre, const float* dpost, long long elements, float* dpre) {
-  const long long i = blockIdx.x * 256LL + threadIdx.x;
+  const long long i = (blockIdx.x * 256LL + threadIdx.x) * VEC;
   if (i >= elements) return;
-  const float x = pre[i];
-  const float sigmoid = 1.0f / (1.0f + expf(-x));
-  dpre[i] = dpost[i] * sigmoid * (1.0f + x * (1.0f - sigmoid));
+  const Pack<VEC> x = load_floats<VEC>(pre + i), g = load_floats<VEC>(dpost + i);
+  Pack<VEC> r;
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) {
+    const float sigmoid = 1.0f / (1.0f + expf(-x.e[e]));
+    r.e[e] = g.e[e] * sigmoid * (1.0f + x.e[e] * (1.0f - sigmoid));
+  }
+  store_floats<VEC>(dpre + i, r);
 }
 
+template <int VEC>
 __global__ void __launch_bounds__(256)
 conv_input_backward_kernel(const float* dpre, const float* __restrict__ weight, int length,
                            int channels, int kernel, float* dx) {
+  const int groups = channels / VEC;
   const long long i = blockIdx.x * 256LL + threadIdx.x;
-  if (i >= 1LL * length * channels) return;
-  const int c = static_cast<int>(i % channels), t = static_cast<int>(i / channels);
-  float sum = 0.0f;
+  if (i >= 1LL * length * groups) return;
+  const int c = static_cast<int>(i % groups) * VEC, t = static_cast<int>(i / groups);
+  Pack<VEC> sum;
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) sum.e[e] = 0.0f;
   for (int tap = 0; tap < kernel; ++tap) {
     const int future = t + kernel - 1 - tap;
-    if (future < length) sum += dpre[1LL * future * channels + c] * weight[1LL * c * kernel + tap];
+    if (future >= length) continue;
+    const Pack<VEC> g = load_floats<VEC>(dpre + 1LL * future * channels + c);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) sum.e[e] += g.e[e] * weight[1LL * (c + e) * kernel + tap];
   }
-  dx[i] = sum;
+  store_floats<VEC>(dx + 1LL * t * channels + c, sum);
+}
+
+// dw[c, tap] += sum over t of dpre[t, c] x[t + tap - kernel + 1, c], in two
+// levels with a fixed order: blockIdx.z sums one slice of the tokens.
+__global__ void __launch_bounds__(256)
+conv_weight_partial_kernel(const uint16_t* input, const float* dpre, int length, int channels,
+                           int kernel, int slices, float* partial) {
+  const int c = blockIdx.x * 256 + threadIdx.x, tap = blockIdx.y, slice = blockIdx.z;
+  if (c >= channels) return;
+  const int per = (length + slices - 1) / slices;
+  const int first = max(slice * per, kernel - 1 - tap), last = min((slice + 1) * per, length);
+  float sum = 0.0f;
+  for (int t = first; t < last; ++t)
+    sum += dpre[1LL * t * channels + c] *
+           bf16_bits_to_float(input[1LL * (t + tap - kernel + 1) * channels + c]);
+  partial[(1LL * slice * channels + c) * kernel + tap] = sum;
 }
 
 __global__ void __launch_bounds__(256)
-conv_weight_backward_kernel(const uint16_t* input, const float* dpre, int length, int channels,
-                            int kernel, float* dw) {
-  const int c = blockIdx.x * 256 + threadIdx.x, tap = blockIdx.y;
-  if (c >= channels) return;
+conv_weight_final_kernel(const float* partial, long long elements, int slices, float* dw) {
+  const long long i = blockIdx.x * 256LL + threadIdx.x;
+  if (i >= elements) return;
   float sum = 0.0f;
-  for (int t = kernel - 1 - tap; t < length; ++t)
-    sum += dpre[1LL * t * channels + c] *
-           bf16_bits_to_float(input[1LL * (t + tap - kernel + 1) * channels + c]);
-  dw[1LL * c * kernel + tap] += sum;
+  for (int slice = 0; slice < slices; ++slice) sum += partial[slice * elements + i];
+  dw[i] += sum;
 }
 
 // gradient[c] += sum over rows of partials[row, c], two levels, fixed order.
+// Sum of rows first..last-1 of a [rows, width] matrix (width <= 256), per
+// column.  The 256 threads form up to 8 groups of `width`; group g takes rows
+// first + g, first + g + groups, ...; the groups' sums are added in ascending
+// order.  Returns the column's total in the threads of group 0.
+__device__ inline float sum_block_rows(const float* parts, long long first, long long last,
+                                       int width) {
+  __shared__ float scratch[8][256];
+  const int fit = 256 / width, groups = fit < 8 ? fit : 8;
+  const int c = threadIdx.x % width, g = threadIdx.x / width;
+  if (g < groups) {
+    float sum = 0.0f;
+#pragma unroll 8
+    for (long long row = first + g; row < last; row += groups) sum += parts[row * width + c];
+    scratch[g][c] = sum;
+  }
+  __syncthreads();
+  float total = 0.0f;
+  if (g == 0)
+    for (int j = 0; j < groups; ++j) total += scratch[j][c];
+  return total;
+}
+
 __global__ void __launch_bounds__(256)
 sum_rows_partial_kernel(const float* parts, long long rows, int width, int chunks, float* partial) {
-  const int c = threadIdx.x;
-  if (c >= width) return;
   const long long per = (rows + chunks - 1) / chunks;
   const long long first = blockIdx.x * per;
   const long long last = first + per < rows ? first + per : rows;
-  float sum = 0.0f;
-  for (long long row = first; row < last; ++row) sum += parts[row * width + c];
-  partial[1LL * blockIdx.x * width + c] = sum;
+  const float total = sum_block_rows(parts, first, last, width);
+  if (threadIdx.x < width) partial[1LL * blockIdx.x * width + threadIdx.x] = total;
 }
 
 __global__ void __launch_bounds__(256)
 sum_rows_final_kernel(const float* partial, int chunks, int width, float* gradient) {
-  const int c = threadIdx.x;
-  if (c >= width) return;
-  float sum = 0.0f;
-  for (int chunk = 0; chunk < chunks; ++chunk) sum += partial[1LL * chunk * width + c];
-  gradient[c] += sum;
+  const float total = sum_block_rows(partial, 0, chunks, width);
+  if (threadIdx.x < width) gradient[threadIdx.x] += total;
 }
 
 unsigned blocks_for(long long elements) { return static_cast<unsigned>((elements + 255) / 256); }
@@ -510,6 +602,7 @@ size_t gdn_backward_workspace_bytes(const pluto_hip_delta_params* p, int length,
   bytes += align_up(T * vh * tiles * 2 * kd * 4, 256);   // q/k partials
   bytes += align_up(T * vh * tiles * 3 * 4, 256);        // scalar partials
   if (norm_grad) bytes += align_up(T * vh * vd * 4, 256) + align_up(kGdnSumChunks * vd * 4, 256);
+  bytes += align_up(kConvSlices * channels * p->conv_kernel_dim * 4, 256);  // conv weight partials
   return bytes;
 }
 
@@ -542,9 +635,12 @@ int launch_gdn_backward(hipStream_t stream, const pluto_hip_delta_params* p, int
   float* scalar_partials = take(T * vh * tiles * 3 * 4);
   float* norm_partials = d_norm ? take(T * vh * vd * 4) : nullptr;
   float* norm_chunks = d_norm ? take(static_cast<size_t>(kGdnSumChunks) * vd * 4) : nullptr;
+  float* conv_partials = take(static_cast<size_t>(kConvSlices) * channels * kernel * 4);
 
   const long long elements = 1LL * length * channels;
-  conv_train_kernel<<<blocks_for(elements), 256, 0, stream>>>(
+  // one channel a thread: four a thread (one wide access instead of four) was
+  // measured slower for the two kernels that also read the weights
+  conv_train_kernel<1><<<blocks_for(elements), 256, 0, stream>>>(
       static_cast<const uint16_t*>(qkv), conv_weight, length, channels, kernel, round, pre, post);
   int status = launch_status();
   if (status != 0) return status;
@@ -612,12 +708,22 @@ int launch_gdn_backward(hipStream_t stream, const pluto_hip_delta_params* p, int
                                                          dpost);
   gather_scalar_kernel<<<vh, 256, 0, stream>>>(scalar_partials, length, vh, tiles, da, db, d_a_log,
                                                d_dt_bias);
-  conv_silu_backward_kernel<<<blocks_for(elements), 256, 0, stream>>>(pre, dpost, elements, dpre);
-  conv_input_backward_kernel<<<blocks_for(elements), 256, 0, stream>>>(dpre, conv_weight, length,
-                                                                      channels, kernel, dqkv);
-  if (d_conv_weight)
-    conv_weight_backward_kernel<<<dim3((channels + 255) / 256, kernel), 256, 0, stream>>>(
-        static_cast<const uint16_t*>(qkv), dpre, length, channels, kernel, d_conv_weight);
+  if (elements % 4 == 0)
+    conv_silu_backward_kernel<4><<<blocks_for(elements / 4), 256, 0, stream>>>(pre, dpost, elements,
+                                                                               dpre);
+  else
+    conv_silu_backward_kernel<1><<<blocks_for(elements), 256, 0, stream>>>(pre, dpost, elements,
+                                                                           dpre);
+  conv_input_backward_kernel<1><<<blocks_for(elements), 256, 0, stream>>>(
+      dpre, conv_weight, length, channels, kernel, dqkv);
+  if (d_conv_weight) {
+    conv_weight_partial_kernel<<<dim3((channels + 255) / 256, kernel, kConvSlices), 256, 0, stream>>>(
+        static_cast<const uint16_t*>(qkv), dpre, length, channels, kernel, kConvSlices,
+        conv_partials);
+    const long long weights = 1LL * channels * kernel;
+    conv_weight_final_kernel<<<blocks_for(weights), 256, 0, stream>>>(conv_partials, weights,
+                                                                      kConvSlices, d_conv_weight);
+  }
   return launch_status();
 }
 
