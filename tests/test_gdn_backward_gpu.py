@@ -82,9 +82,12 @@ def run(capi, shape, rounding, seed=0, batch=1, with_parameters=True):
 
 # (T, key heads, value heads, key width, value width, conv taps).  128 x 128
 # heads take the chunked kernels (64-token chunks: one full chunk, a ragged
-# tail, grouped heads over several chunks); the other widths go token by token.
+# tail, grouped heads over several chunks, and 1, 2, 3, 4 and 5 chunks for the
+# three operand sets the sequential kernels rotate); the other widths go token
+# by token.
 SHAPES = [(4, 1, 2, 3, 5, 3), (9, 2, 4, 5, 35, 4), (33, 2, 2, 16, 40, 4), (64, 1, 2, 128, 128, 4),
-          (37, 1, 1, 128, 128, 4), (200, 1, 2, 128, 128, 4), (130, 2, 4, 128, 128, 3)]
+          (37, 1, 1, 128, 128, 4), (200, 1, 2, 128, 128, 4), (130, 2, 4, 128, 128, 3),
+          (100, 1, 1, 128, 128, 2), (300, 1, 1, 128, 128, 4)]
 
 
 @pytest.mark.parametrize("rounding", [False, True])
