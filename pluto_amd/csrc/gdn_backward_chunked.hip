@@ -584,6 +584,21 @@ chunk_local_kernel(ChunkedArgs a) {
 // 32w..32w+31 of the [64, 128] matrices (two 32-row tiles) or one 32 x 32 tile
 // of a [64, 64] matrix.
 
+// Sums over the 32 lanes of a half wave of sixteen values at once: the five
+// exchange stages are the outer loop, so that the sixteen exchanges of a stage
+// are in flight together (one value at a time, each stage waits for the one
+// before and the sums cost ten times as much).
+__device__ inline void half_sums(float (&v)[16]) {
+#pragma unroll
+  for (int offset = 16; offset > 0; offset >>= 1) {
+    float other[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) other[i] = __shfl_xor(v[i], offset, 64);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) v[i] += other[i];
+  }
+}
+
 // Sums over the four waves of per-row partial sums left in parts[row][wave].
 __device__ inline float across_waves(const float (*parts)[4], int row) {
   return (parts[row][0] + parts[row][1]) + (parts[row][2] + parts[row][3]);
@@ -656,6 +671,9 @@ chunk_delta_gradient_kernel(ChunkedArgs a) {
 //   0: dW = -dDl S^T
 //   1: diag(E) dO S^T (the first part of dq^) and its row sums against q^
 //   2: diag(L) Dl dS'^T (the first part of dk^), its row sums against k^, <dS', S>
+// Both operands are contiguous along the contraction and are read in 16-byte
+// pieces, one row a lane.  (Staging them in LDS with coalesced loads first
+// measured the same 88 us: the kernel moves 270 MB.)
 __global__ void __launch_bounds__(256)
 chunk_state_products_kernel(ChunkedArgs a) {
   __shared__ float parts[kC][4];
@@ -669,6 +687,17 @@ chunk_state_products_kernel(ChunkedArgs a) {
   const float* state = which == 2 ? v.dS1 : v.S0;
   float* target = (which == 0 ? a.r.dwm : which == 1 ? a.r.dqp : a.r.dkp) + v.rec * kWide;
   const float* against = which == 1 ? v.Q : v.K;
+  float dot = 0.0f;
+  if (which == 2) {
+    const int c4 = 4 * (tid % 32);
+#pragma unroll
+    for (int j = 0; j < kD / 8; ++j) {
+      const int row = tid / 32 + 8 * j;
+      const float4 x = load4(v.S0 + row * kD + c4), y = load4(v.dS1 + row * kD + c4);
+      dot += (x.x * y.x + x.y * y.y) + (x.z * y.z + x.w * y.w);
+    }
+  }
+  reduce[tid] = dot;
 #pragma unroll
   for (int ti = 0; ti < 2; ++ti) {
     const int m = 32 * ti + n;
@@ -682,28 +711,28 @@ chunk_state_products_kernel(ChunkedArgs a) {
           return scaled(row, factor);
         },
         [&](int k) { return load4(state + col * kD + k); });
+    float weighted[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       const int row = 32 * ti + tile_row(i, h);
       target[row * kD + col] = acc[i];
-      if (which != 0) {
-        const float sum = wave_half_sum(acc[i] * against[row * kD + col]);
-        if (n == 0) parts[row][wave] = sum;
+      weighted[i] = which != 0 ? acc[i] * against[row * kD + col] : 0.0f;
+    }
+    if (which != 0) {
+      half_sums(weighted);
+      if (n == 0) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) parts[32 * ti + tile_row(i, h)][wave] = weighted[i];
       }
     }
   }
   if (which == 0) return;
-  if (which == 2) {
-    float dot = 0.0f;
-    for (int idx = tid; idx < kState; idx += 256) dot += v.S0[idx] * v.dS1[idx];
-    reduce[tid] = dot;
-  }
   __syncthreads();
   if (tid < kC) sums[(which - 1) * kC + tid] = across_waves(parts, tid);
   if (which == 2 && tid == 0) {
-    float dot = 0.0f;
-    for (int j = 0; j < 256; ++j) dot += reduce[j];
-    sums[6 * kC] = dot;
+    float total = 0.0f;
+    for (int j = 0; j < 256; ++j) total += reduce[j];
+    sums[6 * kC] = total;
   }
 }
 
@@ -827,12 +856,19 @@ chunk_finish_kernel(ChunkedArgs a) {
   // T^T dW = d(diag(beta E) K^)
   const floatx16 tw = product<kC>(zero_tile(), [&](int k) { return v.Tm[k * kC + m]; },
                                   [&](int k) { return dW[k * kD + col]; });
+  {
+    float weighted[16];
 #pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    const int local = tile_row(i, h), row = 32 * ti + local;
-    const float r = wave_half_sum(tw[i] * v.K[row * kD + col]) * e_s[row];
-    if (n == 0) parts[0][local][wave] = r;
-    dk[i] += beta_s[row] * e_s[row] * tw[i];
+    for (int i = 0; i < 16; ++i) {
+      const int row = 32 * ti + tile_row(i, h);
+      weighted[i] = tw[i] * v.K[row * kD + col] * e_s[row];
+      dk[i] += beta_s[row] * e_s[row] * tw[i];
+    }
+    half_sums(weighted);
+    if (n == 0) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) parts[0][tile_row(i, h)][wave] = weighted[i];
+    }
   }
   // dk^ += (R + R^T) K^ + Pd^T Q^
   dk = product4<kC>(dk, [&](int k) { return load4(R + m * kC + k); },
@@ -844,19 +880,29 @@ chunk_finish_kernel(ChunkedArgs a) {
   // dv = diag(beta) T^T dDl
   const floatx16 tu = product<kC>(zero_tile(), [&](int k) { return v.Tm[k * kC + m]; },
                                   [&](int k) { return dDl[k * kD + col]; });
+  {
+    float rv[16], q_dot[16], k_dot[16];
 #pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    const int local = tile_row(i, h), row = 32 * ti + local, t = v.t0 + row;
-    const float rv = wave_half_sum(tu[i] * value1(a, v, row, col));
-    const float q_dot = wave_half_sum(dq[i] * v.Q[row * kD + col]);
-    const float k_dot = wave_half_sum(dk[i] * v.K[row * kD + col]);
-    if (n == 0) {
-      parts[1][local][wave] = rv;
-      parts[2][local][wave] = q_dot;
-      parts[3][local][wave] = k_dot;
+    for (int i = 0; i < 16; ++i) {
+      const int row = 32 * ti + tile_row(i, h), t = v.t0 + row;
+      rv[i] = tu[i] * value1(a, v, row, col);
+      q_dot[i] = dq[i] * v.Q[row * kD + col];
+      k_dot[i] = dk[i] * v.K[row * kD + col];
+      if (t < a.length)
+        a.dpost[static_cast<size_t>(t) * v.channels + v.value_offset + col] = beta_s[row] * tu[i];
     }
-    if (t < a.length)
-      a.dpost[static_cast<size_t>(t) * v.channels + v.value_offset + col] = beta_s[row] * tu[i];
+    half_sums(rv);
+    half_sums(q_dot);
+    half_sums(k_dot);
+    if (n == 0) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int local = tile_row(i, h);
+        parts[1][local][wave] = rv[i];
+        parts[2][local][wave] = q_dot[i];
+        parts[3][local][wave] = k_dot[i];
+      }
+    }
   }
   __syncthreads();
   // back through the L2 normalisations (and the 1/sqrt(d) of q)
