@@ -186,16 +186,19 @@ decode_split_kernel(DecodeArgs a, DecodeBatch batch) {
         for (int e = 0; e < 8; ++e) acc[hh][e] += p[hh] * v[e];
     }
   }
+  // exchange stages outermost: the exchanges of a stage are in flight together
 #pragma unroll
-  for (int hh = 0; hh < GROUP; ++hh)
+  for (int offset = LANES_PER_ROW; offset < 64; offset <<= 1) {
+    float other[GROUP][8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      float x = acc[hh][e];
+    for (int hh = 0; hh < GROUP; ++hh)
 #pragma unroll
-      for (int offset = LANES_PER_ROW; offset < 64; offset <<= 1)
-        x += __shfl_xor(x, offset, 64);
-      acc[hh][e] = x;
-    }
+      for (int e = 0; e < 8; ++e) other[hh][e] = __shfl_xor(acc[hh][e], offset, 64);
+#pragma unroll
+    for (int hh = 0; hh < GROUP; ++hh)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[hh][e] += other[hh][e];
+  }
   __syncthreads();  // every wave is done with the probabilities
   if (sub == 0) {
 #pragma unroll
