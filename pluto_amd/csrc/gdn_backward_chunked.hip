@@ -402,7 +402,17 @@ template <bool REVERSE>
 __global__ void __launch_bounds__(256)
 chunk_states_kernel(ChunkedArgs a) {
   __shared__ float state[2][kD][kSlice];
-  const int head = blockIdx.x / (kD / kSlice), col0 = (blockIdx.x % (kD / kSlice)) * kSlice;
+  // The eight column slices of a head read the same matrices: they are given
+  // block numbers with the same remainder mod 8, which the hardware places on
+  // one XCD, so that seven of the eight reads are served by that XCD's L2.
+  constexpr int kSlices = kD / kSlice;
+  static_assert(kSlices == 8, "one slice of a head per block of an XCD's share");
+  int head = blockIdx.x / kSlices, slice = blockIdx.x % kSlices;
+  if (a.vh % 8 == 0) {
+    head = (blockIdx.x % 8) * (a.vh / 8) + blockIdx.x / 64;
+    slice = (blockIdx.x / 8) % kSlices;
+  }
+  const int col0 = slice * kSlice;
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
   const int quarter = lane / 16, n = lane % 16;
   const float* matrices = REVERSE ? a.r.m : a.r.mt;
@@ -630,6 +640,22 @@ __device__ inline ChunkView chunk_view(const ChunkedArgs& a, int chunk, int head
   return v;
 }
 
+// A 1-D grid of `parts` workgroups per (head, chunk) unit that read the same
+// records: the parts of a unit get block numbers with the same remainder mod 8
+// (one XCD, hence one L2) and next to each other in launch order.
+struct UnitPart {
+  int chunk, head, part;
+};
+__device__ inline UnitPart unit_part(const ChunkedArgs& a, int parts) {
+  const int units = a.chunks * a.vh, b = blockIdx.x;
+  int unit = b / parts, part = b % parts;
+  if (units % 8 == 0) {
+    part = (b / 8) % parts;
+    unit = (b / (8 * parts)) * 8 + b % 8;
+  }
+  return {unit % a.chunks, unit / a.chunks, part};
+}
+
 // Rows of dO and V; tokens beyond the sequence read as zero.
 __device__ inline float4 d_out4(const ChunkedArgs& a, const ChunkView& v, int i, int c) {
   const int t = v.t0 + i, row = min(t, a.length - 1);
@@ -667,7 +693,7 @@ chunk_delta_gradient_kernel(ChunkedArgs a) {
   }
 }
 
-// Products against the two states, one per blockIdx.z:
+// Products against the two states, one per part of a unit:
 //   0: dW = -dDl S^T
 //   1: diag(E) dO S^T (the first part of dq^) and its row sums against q^
 //   2: diag(L) Dl dS'^T (the first part of dk^), its row sums against k^, <dS', S>
@@ -678,8 +704,9 @@ __global__ void __launch_bounds__(256)
 chunk_state_products_kernel(ChunkedArgs a) {
   __shared__ float parts[kC][4];
   __shared__ float reduce[256];
-  const ChunkView v = chunk_view(a, blockIdx.x, blockIdx.y);
-  const int which = blockIdx.z;
+  const UnitPart u = unit_part(a, 3);
+  const ChunkView v = chunk_view(a, u.chunk, u.head);
+  const int which = u.part;
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int h = lane / 32, n = lane % 32, col = 32 * wave + n;
   const float* dDl = a.r.ddl + v.rec * kWide;
@@ -822,14 +849,15 @@ chunk_triangle_kernel(ChunkedArgs a) {
 }
 
 // dq and dk (back through the normalisations) and dv of 32 rows of a chunk
-// (blockIdx.z picks the row tile), and the row sums of those rows that the
+// (the unit's part picks the row tile), and the row sums of those rows that the
 // gate gradients need.
 __global__ void __launch_bounds__(256)
 chunk_finish_kernel(ChunkedArgs a) {
   __shared__ float parts[4][kC / 2][4];
   __shared__ float e_s[kC], beta_s[kC];
-  const ChunkView v = chunk_view(a, blockIdx.x, blockIdx.y);
-  const int ti = blockIdx.z;
+  const UnitPart u = unit_part(a, 2);
+  const ChunkView v = chunk_view(a, u.chunk, u.head);
+  const int ti = u.part;
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int h = lane / 32, n = lane % 32, col = 32 * wave + n;
   const float* dDl = a.r.ddl + v.rec * kWide;
@@ -1050,13 +1078,13 @@ int launch_gdn_backward_chunked_reverse(hipStream_t stream, const GdnChunkedBack
   chunk_delta_gradient_kernel<<<per_chunk, 256, 0, stream>>>(a);
   status = launch_status();
   if (status != 0) return status;
-  chunk_state_products_kernel<<<dim3(a.chunks, a.vh, 3), 256, 0, stream>>>(a);
+  chunk_state_products_kernel<<<a.chunks * a.vh * 3, 256, 0, stream>>>(a);
   status = launch_status();
   if (status != 0) return status;
   chunk_triangle_kernel<<<per_chunk, 256, 0, stream>>>(a);
   status = launch_status();
   if (status != 0) return status;
-  chunk_finish_kernel<<<dim3(a.chunks, a.vh, 2), 256, 0, stream>>>(a);
+  chunk_finish_kernel<<<a.chunks * a.vh * 2, 256, 0, stream>>>(a);
   status = launch_status();
   if (status != 0) return status;
   chunk_gates_kernel<<<per_chunk, kC, 0, stream>>>(a);
