@@ -46,7 +46,7 @@ NAMES = ["mha_train_bf16", "mha_fwd_fp32", "gqa_prefill", "gqa_decode", "gdn_sca
 # "copy" is a plain device copy of known size: the calibration case for the
 # FETCH_SIZE / WRITE_SIZE counters that `roofline.traffic` is derived from.
 # "gqa_prefill_bwd" and "gdn_layer_bwd" time the two sequence backward passes.
-EXTRA = ["copy", "gqa_prefill_bwd", "gdn_layer_bwd"]
+EXTRA = ["copy", "gqa_prefill_bwd", "gdn_layer_bwd", "gdn_decode"]
 
 
 def parse_args():
@@ -291,6 +291,37 @@ def gdn_scan(torch, capi):
                 cpu=None)
 
 
+def gdn_decode(torch, capi):
+    """One token of the gated delta-net layer for 32 sequences with their own
+    states (the delta-net half of a batched decoder step): a row after the
+    headline ones, not part of --workload all."""
+    batch, H, dk, dv, K = 32, 16, 128, 128, 4
+    p = capi.delta_params(H, H, dk, dv, K)
+    channels = 2 * H * dk + H * dv
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    states = capi.DeltaNetStep(p, batch=batch)
+    qkv = torch.randn((batch, channels), generator=gen, device="cuda")
+    z = torch.randn((batch, H * dv), generator=gen, device="cuda")
+    a = torch.randn((batch, H), generator=gen, device="cuda")
+    b = torch.randn((batch, H), generator=gen, device="cuda")
+    conv = 0.5 * torch.randn((channels, K), generator=gen, device="cuda")
+    a_log = torch.zeros(H, device="cuda")
+    dt_bias = torch.zeros(H, device="cuda")
+    norm = torch.ones(dv, device="cuda")
+
+    def step():
+        states.step(qkv, z, a, b, conv, a_log, dt_bias, norm)
+
+    # every recurrent state is read and written once; so is every convolution state
+    work = 2.0 * batch * (H * dk * dv + channels * K) * 4
+    return dict(step=step, parts=[("step", step, work)], work=work,
+                metric="gdn_decode_step_hbm_gbs", unit="GB/s", dtype="f32", bound="hbm",
+                peak=PEAK_HBM_GBS,
+                config={"workload": "gated_delta_net_decode_step", "batch": batch, "heads": H,
+                        "d_k": dk, "d_v": dv, "conv_kernel": K, "state": "fp32, one per sequence"},
+                cpu=None)
+
+
 def copy(torch, capi):
     n = 256 * 2 ** 20   # 1 GiB read + 1 GiB written per step
     src = torch.ones(n, dtype=torch.float32, device="cuda")
@@ -306,7 +337,7 @@ def copy(torch, capi):
                         "bytes_written": n * 4}, cpu=None)
 
 
-WORKLOADS = {"copy": copy, "mha_train_bf16": mha_train_bf16, "mha_fwd_fp32": mha_fwd_fp32,
+WORKLOADS = {"copy": copy, "gdn_decode": gdn_decode, "mha_train_bf16": mha_train_bf16, "mha_fwd_fp32": mha_fwd_fp32,
              "gqa_prefill": gqa_prefill, "gqa_prefill_bwd": gqa_prefill_bwd, "gdn_layer_bwd": gdn_layer_bwd,
              "gqa_decode": gqa_decode,
              "gdn_scan": gdn_scan}

@@ -386,6 +386,8 @@ int pluto_hip_gdn_layer_backward(void* stream, const pluto_hip_delta_params* p,
  *   conv_state fp32 [channels, kernel] and recurrent_state fp32 [vh, kd, vd]
  *   are updated in place (DeltaNetState::Reset = zero both). */
 size_t pluto_hip_gdn_step_workspace_bytes(const pluto_hip_delta_params* p);
+size_t pluto_hip_gdn_step_batch_workspace_bytes(const pluto_hip_delta_params* p,
+                                                int batch);
 int pluto_hip_gdn_step(void* stream, const pluto_hip_delta_params* p,
                        float* conv_state, float* recurrent_state,
                        const float* qkv, const float* z, const float* a,
@@ -393,6 +395,24 @@ int pluto_hip_gdn_step(void* stream, const pluto_hip_delta_params* p,
                        const float* a_log, const float* dt_bias,
                        const float* norm, float* output, void* workspace,
                        size_t workspace_bytes);
+
+/* The same step for `batch` independent sequences in one set of launches: the
+ * delta-net half of a decoder step lifted from batch one (Model::Step,
+ * src/llm/qwen/model.cc:405-428, drives one DeltaNetState::Step per layer and
+ * token) to the batch the cached attention entry point already takes.
+ * Sequence s owns conv_states[s] ([batch, channels, kernel]) and
+ * recurrent_states[s] ([batch, vh, kd, vd]); qkv [batch, channels], z and
+ * output [batch, vh*vd], a and b [batch, vh]; the weights are shared.  Row s
+ * of the result is bit for bit what pluto_hip_gdn_step gives for sequence s
+ * alone. */
+int pluto_hip_gdn_step_batch(void* stream, const pluto_hip_delta_params* p,
+                             int batch, float* conv_states,
+                             float* recurrent_states, const float* qkv,
+                             const float* z, const float* a, const float* b,
+                             const float* conv_weight, const float* a_log,
+                             const float* dt_bias, const float* norm,
+                             float* output, void* workspace,
+                             size_t workspace_bytes);
 
 #ifdef __cplusplus
 }

@@ -118,6 +118,9 @@ SIGNATURES = {
                                      [_VP, _SZ]),
     "pluto_hip_gdn_step_workspace_bytes": (_SZ, [ctypes.POINTER(DeltaParams)]),
     "pluto_hip_gdn_step": (_I, [_VP, ctypes.POINTER(DeltaParams)] + [_VP] * 11 + [_VP, _SZ]),
+    "pluto_hip_gdn_step_batch_workspace_bytes": (_SZ, [ctypes.POINTER(DeltaParams), _I]),
+    "pluto_hip_gdn_step_batch": (_I, [_VP, ctypes.POINTER(DeltaParams), _I] + [_VP] * 11 +
+                                 [_VP, _SZ]),
     "pluto_hip_gdn_recurrence": (_I, [_VP, ctypes.POINTER(DeltaParams), _I, _I, _VP, _VP,
                                       _VP, _VP, _VP, _I, ctypes.c_float, _VP, _VP, _I]),
 }
@@ -426,14 +429,19 @@ def gdn_layer_backward(p, qkv, z, a, b, conv_weight, a_log, dt_bias, norm, dy,
 
 
 class DeltaNetStep:
-    """Single-token delta-net state (DeltaNetState of the reference): fp32 arrays."""
+    """Single-token delta-net state (DeltaNetState of the reference): fp32 arrays.
+    With batch > 1 it holds that many independent sequences (leading axis of
+    every state and activation) advanced by one set of launches."""
 
-    def __init__(self, p, device="cuda"):
+    def __init__(self, p, device="cuda", batch=None):
         self.p = p
+        self.batch = batch
+        lead = () if batch is None else (batch,)
         channels = 2 * p.key_heads * p.key_head_dim + p.value_heads * p.value_head_dim
-        self.conv = torch.zeros((channels, p.conv_kernel_dim), device=device)
-        self.state = torch.zeros((p.value_heads, p.key_head_dim, p.value_head_dim), device=device)
-        size = lib().pluto_hip_gdn_step_workspace_bytes(ctypes.byref(p))
+        self.conv = torch.zeros(lead + (channels, p.conv_kernel_dim), device=device)
+        self.state = torch.zeros(lead + (p.value_heads, p.key_head_dim, p.value_head_dim),
+                                 device=device)
+        size = lib().pluto_hip_gdn_step_batch_workspace_bytes(ctypes.byref(p), batch or 1)
         self.workspace = torch.empty(max(size, 16), dtype=torch.uint8, device=device)
 
     def reset(self):
@@ -442,9 +450,17 @@ class DeltaNetStep:
 
     def step(self, qkv, z, a, b, conv_weight, a_log, dt_bias, norm, stream=None):
         p = self.p
-        out = torch.empty(p.value_heads * p.value_head_dim, device=qkv.device)
-        check(lib().pluto_hip_gdn_step(stream or current_stream(), ctypes.byref(p), ptr(self.conv),
-                                       ptr(self.state), ptr(qkv), ptr(z), ptr(a), ptr(b),
-                                       ptr(conv_weight), ptr(a_log), ptr(dt_bias), ptr(norm),
-                                       ptr(out), ptr(self.workspace), self.workspace.numel()))
+        width = p.value_heads * p.value_head_dim
+        if self.batch is None:
+            out = torch.empty(width, device=qkv.device)
+            check(lib().pluto_hip_gdn_step(
+                stream or current_stream(), ctypes.byref(p), ptr(self.conv), ptr(self.state),
+                ptr(qkv), ptr(z), ptr(a), ptr(b), ptr(conv_weight), ptr(a_log), ptr(dt_bias),
+                ptr(norm), ptr(out), ptr(self.workspace), self.workspace.numel()))
+            return out
+        out = torch.empty((self.batch, width), device=qkv.device)
+        check(lib().pluto_hip_gdn_step_batch(
+            stream or current_stream(), ctypes.byref(p), self.batch, ptr(self.conv),
+            ptr(self.state), ptr(qkv), ptr(z), ptr(a), ptr(b), ptr(conv_weight), ptr(a_log),
+            ptr(dt_bias), ptr(norm), ptr(out), ptr(self.workspace), self.workspace.numel()))
         return out

@@ -229,43 +229,55 @@ int pluto_hip_gdn_layer_backward(void* stream, const pluto_hip_delta_params* p, 
   return 0;
 }
 
-size_t pluto_hip_gdn_step_workspace_bytes(const pluto_hip_delta_params* p) {
-  if (validate_delta(p) != 0) return 0;
+size_t pluto_hip_gdn_step_batch_workspace_bytes(const pluto_hip_delta_params* p, int batch) {
+  if (validate_delta(p) != 0 || batch <= 0) return 0;
+  const size_t n = static_cast<size_t>(batch);
   const size_t channels = 2 * static_cast<size_t>(p->key_heads) * p->key_head_dim +
                           static_cast<size_t>(p->value_heads) * p->value_head_dim;
-  return align_up(channels * 4, 256) + 2 * align_up(static_cast<size_t>(p->value_heads) * 4, 256) +
-         align_up(static_cast<size_t>(p->value_heads) * p->value_head_dim * 4, 256);
+  return align_up(n * channels * 4, 256) + 2 * align_up(n * p->value_heads * 4, 256) +
+         align_up(n * p->value_heads * p->value_head_dim * 4, 256);
 }
 
-int pluto_hip_gdn_step(void* stream, const pluto_hip_delta_params* p, float* conv_state,
-                       float* recurrent_state, const float* qkv, const float* z,
-                       const float* a, const float* b, const float* conv_weight,
-                       const float* a_log, const float* dt_bias, const float* norm,
-                       float* output, void* workspace, size_t workspace_bytes) {
+size_t pluto_hip_gdn_step_workspace_bytes(const pluto_hip_delta_params* p) {
+  return pluto_hip_gdn_step_batch_workspace_bytes(p, 1);
+}
+
+int pluto_hip_gdn_step_batch(void* stream, const pluto_hip_delta_params* p, int batch,
+                             float* conv_states, float* recurrent_states, const float* qkv,
+                             const float* z, const float* a, const float* b,
+                             const float* conv_weight, const float* a_log, const float* dt_bias,
+                             const float* norm, float* output, void* workspace,
+                             size_t workspace_bytes) {
   int status = validate_delta(p);
   if (status != 0) return status;
+  if (batch <= 0) return PLUTO_HIP_EINVAL;
   // cached_attention_ops.cc:405-408
-  if (!conv_state || !recurrent_state || !qkv || !z || !a || !b || !conv_weight || !a_log ||
+  if (!conv_states || !recurrent_states || !qkv || !z || !a || !b || !conv_weight || !a_log ||
       !dt_bias || !norm || !output)
     return PLUTO_HIP_EINVAL;
-  if (!workspace || workspace_bytes < pluto_hip_gdn_step_workspace_bytes(p))
+  if (!workspace || workspace_bytes < pluto_hip_gdn_step_batch_workspace_bytes(p, batch))
     return PLUTO_HIP_EWORKSPACE;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bool round = p->round_to_bfloat16 != 0;
   const int kh = p->key_heads, vh = p->value_heads, kd = p->key_head_dim, vd = p->value_head_dim;
   const int channels = 2 * kh * kd + vh * vd;
+  const size_t n = static_cast<size_t>(batch);
   char* scratch = static_cast<char*>(workspace);
   float* convolved = reinterpret_cast<float*>(scratch);
-  size_t offset = align_up(static_cast<size_t>(channels) * 4, 256);
+  size_t offset = align_up(n * channels * 4, 256);
   float* log_decay = reinterpret_cast<float*>(scratch + offset);
-  offset += align_up(static_cast<size_t>(vh) * 4, 256);
+  offset += align_up(n * vh * 4, 256);
   float* beta = reinterpret_cast<float*>(scratch + offset);
-  offset += align_up(static_cast<size_t>(vh) * 4, 256);
+  offset += align_up(n * vh * 4, 256);
   float* core = reinterpret_cast<float*>(scratch + offset);
-  status = launch_gdn_conv_step(s, qkv, conv_weight, channels, p->conv_kernel_dim, round,
-                                conv_state, convolved);
+  status = launch_gdn_conv_step(s, qkv, conv_weight, batch, channels, p->conv_kernel_dim, round,
+                                conv_states, convolved);
   if (status != 0) return status;
-  status = launch_gdn_gates(s, a, b, PLUTO_HIP_F32, a_log, dt_bias, 1, vh, round, log_decay, beta);
+  if (!force_generic() && gdn_step_fused_supported(kd, vd))
+    return launch_gdn_step_fused(s, convolved, z, a, b, a_log, dt_bias, norm, batch, kh, vh, kd, vd,
+                                 p->rms_norm_epsilon, round, recurrent_states, output);
+  status =
+      launch_gdn_gates(s, a, b, PLUTO_HIP_F32, a_log, dt_bias, batch, vh, round, log_decay, beta);
   if (status != 0) return status;
   GdnArgs g;
   g.q = reinterpret_cast<const uint16_t*>(convolved);
@@ -275,9 +287,9 @@ int pluto_hip_gdn_step(void* stream, const pluto_hip_delta_params* p, float* con
   g.in_dtype = PLUTO_HIP_F32;
   g.log_decay = log_decay;
   g.beta = beta;
-  g.state = recurrent_state;
+  g.state = recurrent_states;
   g.out_any = core;
-  g.batch = 1;
+  g.batch = batch;
   g.length = 1;
   g.key_heads = kh;
   g.value_heads = vh;
@@ -288,8 +300,19 @@ int pluto_hip_gdn_step(void* stream, const pluto_hip_delta_params* p, float* con
   g.q_scale = 1.0f / std::sqrt(static_cast<float>(kd));
   status = launch_gdn_recurrence(s, g, PLUTO_HIP_F32);
   if (status != 0) return status;
-  return launch_gdn_output(s, core, PLUTO_HIP_F32, z, PLUTO_HIP_F32, norm, vh, vd,
-                           p->rms_norm_epsilon, round, output, PLUTO_HIP_F32);
+  return launch_gdn_output(s, core, PLUTO_HIP_F32, z, PLUTO_HIP_F32, norm,
+                           static_cast<long long>(batch) * vh, vd, p->rms_norm_epsilon, round,
+                           output, PLUTO_HIP_F32);
+}
+
+int pluto_hip_gdn_step(void* stream, const pluto_hip_delta_params* p, float* conv_state,
+                       float* recurrent_state, const float* qkv, const float* z,
+                       const float* a, const float* b, const float* conv_weight,
+                       const float* a_log, const float* dt_bias, const float* norm,
+                       float* output, void* workspace, size_t workspace_bytes) {
+  return pluto_hip_gdn_step_batch(stream, p, 1, conv_state, recurrent_state, qkv, z, a, b,
+                                  conv_weight, a_log, dt_bias, norm, output, workspace,
+                                  workspace_bytes);
 }
 
 }  // extern "C"

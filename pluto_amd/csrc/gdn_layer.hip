@@ -38,7 +38,11 @@ conv_step_kernel(const float* __restrict__ input, const float* __restrict__ weig
                  float* __restrict__ output) {
   const int c = blockIdx.x * 128 + threadIdx.x;
   if (c >= channels) return;
-  float* taps = state + static_cast<long long>(c) * kernel;
+  // blockIdx.y: the sequence, each with its own shift registers and row
+  const long long sequence = blockIdx.y;
+  input += sequence * channels;
+  output += sequence * channels;
+  float* taps = state + (sequence * channels + c) * kernel;
   const float* w = weight + static_cast<long long>(c) * kernel;
   float sum = 0.0f;
   // each channel is owned by one thread; shifting in ascending order never
@@ -101,7 +105,141 @@ output_kernel(const void* core, int core_dtype, const void* z, int z_dtype,
   }
 }
 
+// One token of the gated delta rule for one (sequence, value head) with the
+// gates before it and RMSNorm x SiLU(z) after it: DeltaRecurrenceKernel and
+// DeltaOutputKernel (cached_attention_ops.cc:205-272) with the gate
+// arithmetic of sequence_delta_net.cc:88-96 in one launch.  The state is read
+// and written exactly once, every load is issued before anything is waited
+// for: thread (half, column) = (tid / 128, tid % 128) owns rows 64 half ..
+// 64 half + 63 of its column.
+struct StepArgs {
+  const float* convolved = nullptr;  // [batch, channels] q | k | v after conv + SiLU
+  const float* z = nullptr;          // [batch, vh * vd]
+  const float* a = nullptr;          // [batch, vh]
+  const float* b = nullptr;
+  const float* a_log = nullptr;
+  const float* dt_bias = nullptr;
+  const float* norm = nullptr;
+  float* state = nullptr;            // [batch, vh, kd, vd]
+  float* out = nullptr;              // [batch, vh * vd]
+  int kh = 0, vh = 0, kd = 0, vd = 0;
+  float epsilon = 1e-6f;
+  bool round = true;
+};
+
+__global__ void __launch_bounds__(256)
+step_kernel(StepArgs a) {
+  __shared__ float ks[128], qs[128];
+  __shared__ float halves[2][128];
+  __shared__ float squares[2];
+  const int bh = blockIdx.x, seq = bh / a.vh, head = bh % a.vh;
+  const int key_head = head / (a.vh / a.kh);
+  const int kd = a.kd, vd = a.vd;
+  const int tid = threadIdx.x, column = tid % 128, half = tid / 128;
+  const int channels = 2 * a.kh * kd + a.vh * vd;
+  const float* token = a.convolved + static_cast<size_t>(seq) * channels;
+  float* state = a.state + static_cast<size_t>(bh) * kd * vd;
+  const bool active = column < vd;
+  const int column_read = active ? column : vd - 1;
+  // the state slice: rows beyond the key width read the last row and count as zero
+  float s[64];
+#pragma unroll
+  for (int r = 0; r < 64; ++r) {
+    const int row = 64 * half + r;
+    const float value = state[min(row, kd - 1) * vd + column_read];
+    s[r] = (row < kd && active) ? value : 0.0f;
+  }
+  if (tid < 128) {
+    const int d = min(tid, kd - 1);
+    const float kv = token[(a.kh + key_head) * kd + d], qv = token[key_head * kd + d];
+    ks[tid] = tid < kd ? kv : 0.0f;
+    qs[tid] = tid < kd ? qv : 0.0f;
+  }
+  const float value = token[2 * a.kh * kd + head * vd + column_read];
+  const float gate = a.z[(static_cast<size_t>(seq) * a.vh + head) * vd + column_read];
+  const float weight = a.norm[column_read];
+  const size_t scalar = static_cast<size_t>(seq) * a.vh + head;
+  const float alpha = a.a[scalar] + a.dt_bias[head];
+  // stable softplus: no overflow for strongly positive time steps
+  const float softplus = fmaxf(alpha, 0.0f) + log1pf(expf(-fabsf(alpha)));
+  const float decay = __expf(-expf(a.a_log[head]) * softplus);
+  const float beta = maybe_round(1.0f / (1.0f + expf(-a.b[scalar])), a.round);
+  __syncthreads();
+  // 1e-6 inside the root: cached_attention_ops.cc:224-228
+  float kk = 1e-6f, qq = 1e-6f;
+  for (int d = 0; d < 128; ++d) {
+    kk += ks[d] * ks[d];
+    qq += qs[d] * qs[d];
+  }
+  const float k_factor = rsqrtf(kk);
+  const float q_factor = rsqrtf(qq) / sqrtf(static_cast<float>(kd));
+  float prediction = 0.0f;
+#pragma unroll
+  for (int r = 0; r < 64; ++r) {
+    s[r] *= decay;
+    prediction += s[r] * (ks[64 * half + r] * k_factor);
+  }
+  halves[half][column] = prediction;
+  __syncthreads();
+  const float delta = (value - (halves[0][column] + halves[1][column])) * beta;
+  __syncthreads();
+  float output = 0.0f;
+#pragma unroll
+  for (int r = 0; r < 64; ++r) {
+    s[r] += (ks[64 * half + r] * k_factor) * delta;
+    output += s[r] * (qs[64 * half + r] * q_factor);
+  }
+#pragma unroll
+  for (int r = 0; r < 64; ++r) {
+    const int row = 64 * half + r;
+    if (row < kd && active) state[row * vd + column] = s[r];
+  }
+  halves[half][column] = output;
+  __syncthreads();
+  // RMSNorm over the head's columns, then the SiLU(z) gate
+  float core = 0.0f;
+  if (half == 0 && active) core = maybe_round(halves[0][column] + halves[1][column], a.round);
+  const float square = wave_sum(core * core);
+  if (half == 0 && tid % 64 == 0) squares[tid / 64] = square;
+  __syncthreads();
+  if (half != 0 || !active) return;
+  const float inverse = rsqrtf((squares[0] + squares[1]) / static_cast<float>(vd) + a.epsilon);
+  const float normalized = maybe_round(core * inverse, a.round);
+  const float affine = maybe_round(normalized * weight, a.round);
+  const float result = affine * (gate / (1.0f + expf(-gate)));
+  a.out[(static_cast<size_t>(seq) * a.vh + head) * vd + column] = maybe_round(result, a.round);
+}
+
 }  // namespace
+
+bool gdn_step_fused_supported(int key_dim, int value_dim) {
+  return key_dim <= 128 && value_dim <= 128;
+}
+
+int launch_gdn_step_fused(hipStream_t stream, const float* convolved, const float* z,
+                          const float* a, const float* b, const float* a_log,
+                          const float* dt_bias, const float* norm, int batch, int key_heads,
+                          int value_heads, int key_dim, int value_dim, float epsilon, bool round,
+                          float* state, float* out) {
+  StepArgs s;
+  s.convolved = convolved;
+  s.z = z;
+  s.a = a;
+  s.b = b;
+  s.a_log = a_log;
+  s.dt_bias = dt_bias;
+  s.norm = norm;
+  s.state = state;
+  s.out = out;
+  s.kh = key_heads;
+  s.vh = value_heads;
+  s.kd = key_dim;
+  s.vd = value_dim;
+  s.epsilon = epsilon;
+  s.round = round;
+  step_kernel<<<batch * value_heads, 256, 0, stream>>>(s);
+  return launch_status();
+}
 
 int launch_gdn_conv_sequence(hipStream_t stream, const void* input, int in_dtype,
                              const float* weight, int batch, int length, int channels,
@@ -112,10 +250,10 @@ int launch_gdn_conv_sequence(hipStream_t stream, const void* input, int in_dtype
   return launch_status();
 }
 
-int launch_gdn_conv_step(hipStream_t stream, const float* input, const float* weight,
+int launch_gdn_conv_step(hipStream_t stream, const float* input, const float* weight, int batch,
                          int channels, int kernel, bool round, float* state, float* output) {
-  conv_step_kernel<<<(channels + 127) / 128, 128, 0, stream>>>(input, weight, channels, kernel,
-                                                               round, state, output);
+  conv_step_kernel<<<dim3((channels + 127) / 128, batch), 128, 0, stream>>>(
+      input, weight, channels, kernel, round, state, output);
   return launch_status();
 }
 

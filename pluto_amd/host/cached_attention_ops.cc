@@ -2,6 +2,7 @@
 
 #include <cmath>
 #include <limits>
+#include <vector>
 
 namespace pluto::llm::cached_attention_ops {
 namespace {
@@ -81,9 +82,44 @@ Status CachedAttentionStep(hip::Executor& executor, const FullAttentionParameter
   return cache.Advance();
 }
 
+Status CachedAttentionStepBatch(hip::Executor& executor, const FullAttentionParameters& p,
+                                Span<KeyValueCache* const> caches, const float* q_gate,
+                                const float* k, const float* v, const float* q_norm,
+                                const float* k_norm, float* output) {
+  if (caches.empty()) return InvalidArgumentError("attention batch must not be empty");
+  if (!q_gate || !k || !v || !q_norm || !k_norm || !output)
+    return InvalidArgumentError("attention requires non-null device pointers");
+  std::vector<int> positions;
+  std::vector<pluto_hip_kv_cache_view> views;
+  for (KeyValueCache* cache : caches) {
+    if (cache == nullptr) return InvalidArgumentError("attention requires a cache per sequence");
+    RETURN_IF_ERROR(ValidateCachedAttention(executor, p, *cache));
+    if (cache->position() >= cache->capacity())
+      return ResourceExhaustedError("full-attention cache capacity reached");
+    for (size_t other = 0; other < views.size(); ++other)
+      if (caches[other] == cache)
+        return InvalidArgumentError("a cache serves one sequence of the batch");
+    positions.push_back(cache->position());
+    views.push_back(cache->view());
+  }
+  const pluto_hip_attention_params abi = ToAbi(p);
+  const int batch = static_cast<int>(caches.size());
+  const size_t workspace_bytes =
+      pluto_hip_gqa_decode_workspace_bytes(&abi, batch, positions.data(), 0);
+  ASSIGN_OR_RETURN(auto workspace, hip::Buffer::Allocate(executor, workspace_bytes));
+  RETURN_IF_ERROR(hip::HipStatus(
+      pluto_hip_gqa_decode(executor.stream(), &abi, batch, PLUTO_HIP_F32, q_gate, k, v, q_norm,
+                           k_norm, positions.data(), views.data(), output, nullptr, 0,
+                           workspace.data(), workspace_bytes),
+      "Qwen full attention"));
+  for (KeyValueCache* cache : caches) RETURN_IF_ERROR(cache->Advance());
+  return OkStatus();
+}
+
 // src/llm/layers/util/cached_attention_ops.cc:369-399
 StatusOr<std::unique_ptr<DeltaNetState>> DeltaNetState::Create(hip::Executor& executor,
-                                                               DeltaNetParameters p) {
+                                                               DeltaNetParameters p, int batch) {
+  if (batch <= 0) return InvalidArgumentError("DeltaNet batch must be positive");
   if (p.key_heads <= 0 || p.value_heads <= 0 || p.value_heads % p.key_heads != 0 ||
       p.key_head_dim <= 0 || p.key_head_dim > 128 || p.value_head_dim <= 0 ||
       p.value_head_dim > 256 || p.conv_kernel_dim <= 0 || p.conv_kernel_dim > 32 ||
@@ -93,15 +129,16 @@ StatusOr<std::unique_ptr<DeltaNetState>> DeltaNetState::Create(hip::Executor& ex
                           static_cast<size_t>(p.value_heads) * p.value_head_dim;
   if (channels > static_cast<size_t>(std::numeric_limits<int>::max()) / p.conv_kernel_dim)
     return ResourceExhaustedError("DeltaNet dimensions exceed indexing limit");
-  ASSIGN_OR_RETURN(auto convolution, AllocateFloats(executor, channels * p.conv_kernel_dim));
+  const size_t n = static_cast<size_t>(batch);
+  ASSIGN_OR_RETURN(auto convolution, AllocateFloats(executor, n * channels * p.conv_kernel_dim));
   ASSIGN_OR_RETURN(auto recurrence,
-                   AllocateFloats(executor, static_cast<size_t>(p.value_heads) * p.key_head_dim *
-                                                p.value_head_dim));
+                   AllocateFloats(executor, n * p.value_heads * p.key_head_dim * p.value_head_dim));
   const pluto_hip_delta_params abi = ToAbi(p);
   ASSIGN_OR_RETURN(auto workspace,
-                   hip::Buffer::Allocate(executor, pluto_hip_gdn_step_workspace_bytes(&abi)));
+                   hip::Buffer::Allocate(executor,
+                                         pluto_hip_gdn_step_batch_workspace_bytes(&abi, batch)));
   std::unique_ptr<DeltaNetState> result(new DeltaNetState(
-      executor, p, std::move(convolution), std::move(recurrence), std::move(workspace)));
+      executor, p, batch, std::move(convolution), std::move(recurrence), std::move(workspace)));
   RETURN_IF_ERROR(result->Reset());
   return result;
 }
@@ -114,10 +151,11 @@ Status DeltaNetState::Step(const float* qkv, const float* z, const float* a, con
     return InvalidArgumentError("DeltaNet requires non-null device pointers");
   const pluto_hip_delta_params abi = ToAbi(parameters_);
   return hip::HipStatus(
-      pluto_hip_gdn_step(executor_.stream(), &abi, static_cast<float*>(convolution_state_.data()),
-                         static_cast<float*>(recurrent_state_.data()), qkv, z, a, b, conv_weight,
-                         a_log, dt_bias, norm_weight, output, workspace_.data(),
-                         workspace_.size_bytes()),
+      pluto_hip_gdn_step_batch(executor_.stream(), &abi, batch_,
+                               static_cast<float*>(convolution_state_.data()),
+                               static_cast<float*>(recurrent_state_.data()), qkv, z, a, b,
+                               conv_weight, a_log, dt_bias, norm_weight, output, workspace_.data(),
+                               workspace_.size_bytes()),
       "Qwen gated delta step");
 }
 

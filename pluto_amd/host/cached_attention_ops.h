@@ -41,6 +41,20 @@ Status CachedAttentionStep(hip::Executor& executor, const FullAttentionParameter
                            const float* v, const float* q_norm, const float* k_norm,
                            float* output, float* probabilities = nullptr);
 
+// The same step for caches.size() independent sequences in one set of
+// launches: what a decoder step lifted from batch one (Model::Step,
+// src/llm/qwen/model.cc:405-428) to a batch feeds the cached attention with.
+// q_gate [batch, query_heads, 2, head_dim], k/v [batch, key_value_heads,
+// head_dim], output [batch, query_heads, head_dim]; sequence s attends to
+// caches[s] at that cache's own position.  Every cache is validated (and must
+// have room) before any GPU work; all advance together after the launches
+// succeeded.  No probabilities.
+Status CachedAttentionStepBatch(hip::Executor& executor,
+                                const FullAttentionParameters& parameters,
+                                Span<KeyValueCache* const> caches, const float* q_gate,
+                                const float* k, const float* v, const float* q_norm,
+                                const float* k_norm, float* output);
+
 struct DeltaNetParameters {
   int key_heads = 16;
   int value_heads = 48;
@@ -59,8 +73,13 @@ class DeltaNetState final {
  public:
   DeltaNetState(const DeltaNetState&) = delete;
   DeltaNetState& operator=(const DeltaNetState&) = delete;
+  // batch > 1: that many independent sequences, advanced together; every
+  // activation of Step then carries a leading [batch] axis (the reference's
+  // state is the batch-one case).
   static StatusOr<std::unique_ptr<DeltaNetState>> Create(hip::Executor& executor,
-                                                         DeltaNetParameters parameters);
+                                                         DeltaNetParameters parameters,
+                                                         int batch = 1);
+  int batch() const { return batch_; }
 
   // qkv packs [all Q, all K, all V]; z [value_heads, value_head_dim]; a, b,
   // a_log, dt_bias [value_heads]; conv_weight [qkv_channels, conv_kernel_dim]
@@ -72,13 +91,14 @@ class DeltaNetState final {
   Status Reset();
 
  private:
-  DeltaNetState(hip::Executor& executor, DeltaNetParameters parameters,
+  DeltaNetState(hip::Executor& executor, DeltaNetParameters parameters, int batch,
                 hip::Buffer convolution_state, hip::Buffer recurrent_state, hip::Buffer workspace)
-      : executor_(executor), parameters_(parameters),
+      : executor_(executor), parameters_(parameters), batch_(batch),
         convolution_state_(std::move(convolution_state)),
         recurrent_state_(std::move(recurrent_state)), workspace_(std::move(workspace)) {}
   hip::Executor& executor_;
   DeltaNetParameters parameters_;
+  int batch_;
   hip::Buffer convolution_state_;
   hip::Buffer recurrent_state_;
   hip::Buffer workspace_;  // convolved QKV and core output of one token

@@ -126,6 +126,130 @@ TEST(AttentionOpsTest, GqaPartialRopeGatingAndCacheMatchTheOracleAcrossTiles) {
   EXPECT_TRUE(got_values == values);
 }
 
+TEST(AttentionOpsTest, BatchedStepEqualsTheSingleStepOfEverySequence) {
+  // The decoder step of Model::Step (qwen/model.cc:405-428) lifted to several
+  // sequences: three caches at different positions advance together, every
+  // output row bit for bit that of CachedAttentionStep on its own.
+  using cached_attention_ops::CachedAttentionStepBatch;
+  for (auto storage : kStorages) {
+    auto executor = NewExecutor();
+    FullAttentionParameters p;
+    p.query_heads = 4;
+    p.key_value_heads = 2;
+    p.head_dim = 8;
+    p.rotary_dim = 4;
+    p.capacity = 40;
+    const int batch = 3, row = p.query_heads * p.head_dim, kv = p.key_value_heads * p.head_dim;
+    const auto q_norm = Values(8, 0.2, 0.3), k_norm = Values(8, 0.8, 0.4);
+    auto dq = Upload<float>(*executor, q_norm), dk = Upload<float>(*executor, k_norm);
+    std::vector<std::unique_ptr<KeyValueCache>> together, alone;
+    for (int s = 0; s < 2 * batch; ++s) {
+      auto cache = KeyValueCache::Create(*executor, 40, 2, 8, storage);
+      ASSERT_TRUE(cache.ok());
+      (s < batch ? together : alone).push_back(std::move(*cache));
+    }
+    auto token = [&](int s, int t, double phase, int count) {
+      return RoundedToBFloat16(Values(count, phase + 0.37 * s + 1.3 * t));
+    };
+    // different histories: sequence s starts with 5 s tokens of its own
+    for (int s = 0; s < batch; ++s)
+      for (int t = 0; t < 5 * s; ++t) {
+        auto qg = Upload<float>(*executor, token(s, t, 0.1, 2 * row));
+        auto k = Upload<float>(*executor, token(s, t, 0.7, kv));
+        auto v = Upload<float>(*executor, token(s, t, -0.4, kv));
+        auto out = hip::Buffer::Allocate(*executor, row * sizeof(float));
+        for (auto* cache : {together[s].get(), alone[s].get()})
+          ASSERT_TRUE(CachedAttentionStep(*executor, p, *cache, Data(*qg), Data(*k), Data(*v),
+                                          Data(*dq), Data(*dk), Data(*out)).ok());
+      }
+    std::vector<KeyValueCache*> caches;
+    for (auto& cache : together) caches.push_back(cache.get());
+    for (int t = 100; t < 103; ++t) {
+      std::vector<float> qg, k, v;
+      for (int s = 0; s < batch; ++s) {
+        const auto a = token(s, t, 0.1, 2 * row), b = token(s, t, 0.7, kv), c = token(s, t, -0.4, kv);
+        qg.insert(qg.end(), a.begin(), a.end());
+        k.insert(k.end(), b.begin(), b.end());
+        v.insert(v.end(), c.begin(), c.end());
+      }
+      auto dqg = Upload<float>(*executor, qg), dkk = Upload<float>(*executor, k),
+           dv = Upload<float>(*executor, v);
+      auto out = hip::Buffer::Allocate(*executor, batch * row * sizeof(float));
+      ASSERT_TRUE(CachedAttentionStepBatch(*executor, p, caches, Data(*dqg), Data(*dkk), Data(*dv),
+                                           Data(*dq), Data(*dk), Data(*out)).ok());
+      const auto got = Read<float>(*out);
+      for (int s = 0; s < batch; ++s) {
+        auto one = hip::Buffer::Allocate(*executor, row * sizeof(float));
+        ASSERT_TRUE(CachedAttentionStep(*executor, p, *alone[s], Data(*dqg) + s * 2 * row,
+                                        Data(*dkk) + s * kv, Data(*dv) + s * kv, Data(*dq),
+                                        Data(*dk), Data(*one)).ok());
+        const auto want = Read<float>(*one);
+        EXPECT_TRUE(std::equal(want.begin(), want.end(), got.begin() + s * row));
+        EXPECT_EQ(together[s]->position(), alone[s]->position());
+      }
+    }
+    // a full cache anywhere in the batch stops the call before any cache moves
+    auto full = KeyValueCache::Create(*executor, 40, 2, 8, storage);
+    ASSERT_TRUE(full.ok());
+    auto scratch = Upload<float>(*executor, std::vector<float>(batch * 2 * row, 0.f));
+    for (int t = 0; t < 40; ++t)
+      ASSERT_TRUE(CachedAttentionStep(*executor, p, **full, Data(*scratch), Data(*scratch),
+                                      Data(*scratch), Data(*dq), Data(*dk), Data(*scratch)).ok());
+    const int before = together[0]->position();
+    std::vector<KeyValueCache*> with_full = {together[0].get(), full->get()};
+    EXPECT_TRUE(IsResourceExhausted(CachedAttentionStepBatch(
+        *executor, p, with_full, Data(*scratch), Data(*scratch), Data(*scratch), Data(*dq),
+        Data(*dk), Data(*scratch))));
+    EXPECT_EQ(together[0]->position(), before);
+    std::vector<KeyValueCache*> twice = {together[0].get(), together[0].get()};
+    EXPECT_TRUE(IsInvalidArgument(CachedAttentionStepBatch(
+        *executor, p, twice, Data(*scratch), Data(*scratch), Data(*scratch), Data(*dq), Data(*dk),
+        Data(*scratch))));
+  }
+}
+
+TEST(AttentionOpsTest, BatchedDeltaNetStateEqualsIndependentStates) {
+  auto executor = NewExecutor();
+  cached_attention_ops::DeltaNetParameters delta;
+  delta.key_heads = 2;
+  delta.value_heads = 4;
+  delta.key_head_dim = 16;
+  delta.value_head_dim = 24;
+  const int batch = 3, channels = 2 * 2 * 16 + 4 * 24, width = 4 * 24, heads = 4;
+  EXPECT_TRUE(IsInvalidArgument(DeltaNetState::Create(*executor, delta, 0).status()));
+  auto together = DeltaNetState::Create(*executor, delta, batch);
+  ASSERT_TRUE(together.ok());
+  EXPECT_EQ((*together)->batch(), batch);
+  std::vector<std::unique_ptr<DeltaNetState>> alone;
+  for (int s = 0; s < batch; ++s) {
+    auto state = DeltaNetState::Create(*executor, delta);
+    ASSERT_TRUE(state.ok());
+    alone.push_back(std::move(*state));
+  }
+  auto conv = Upload<float>(*executor, Values(channels * 4, 0.73, 0.6));
+  auto a_log = Upload<float>(*executor, Values(heads, 0.18, 0.5));
+  auto dt = Upload<float>(*executor, Values(heads, -0.7, 0.3));
+  auto norm = Upload<float>(*executor, Values(24, 0.5, 0.6));
+  for (int t = 0; t < 4; ++t) {
+    auto qkv = Upload<float>(*executor, Values(batch * channels, 0.3 + t));
+    auto z = Upload<float>(*executor, Values(batch * width, -0.6 + t));
+    auto a = Upload<float>(*executor, Values(batch * heads, 0.1 + t));
+    auto b = Upload<float>(*executor, Values(batch * heads, -0.7 + t));
+    auto out = hip::Buffer::Allocate(*executor, batch * width * sizeof(float));
+    ASSERT_TRUE((*together)->Step(Data(*qkv), Data(*z), Data(*a), Data(*b), Data(*conv),
+                                  Data(*a_log), Data(*dt), Data(*norm), Data(*out)).ok());
+    const auto got = Read<float>(*out);
+    for (int s = 0; s < batch; ++s) {
+      auto one = hip::Buffer::Allocate(*executor, width * sizeof(float));
+      ASSERT_TRUE(alone[s]->Step(Data(*qkv) + s * channels, Data(*z) + s * width,
+                                 Data(*a) + s * heads, Data(*b) + s * heads, Data(*conv),
+                                 Data(*a_log), Data(*dt), Data(*norm), Data(*one)).ok());
+      const auto want = Read<float>(*one);
+      EXPECT_TRUE(std::equal(want.begin(), want.end(), got.begin() + s * width));
+    }
+  }
+}
+
 TEST(AttentionOpsTest, CachedAttentionRejectsInvalidParametersBeforeWork) {
   auto executor = NewExecutor();
   const auto p = Small();

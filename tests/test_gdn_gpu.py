@@ -229,6 +229,59 @@ def test_single_token_step_matches_scalar_specification(capi, oracle, dim, round
             np.testing.assert_array_equal(got, first)   # Reset replays bit-equal
 
 
+@pytest.mark.parametrize("round_flag", [False, True])
+@pytest.mark.parametrize("dim", [5, 128])
+def test_batched_step_is_the_single_step_of_every_sequence(capi, oracle, dim, round_flag):
+    """pluto_hip_gdn_step_batch: the decoder step of Model::Step
+    (qwen/model.cc:405-428) lifted to several sequences with their own
+    DeltaNetState.  Each row must be bit for bit what the single-sequence entry
+    point gives, over several tokens (so states carry over), and match the
+    scalar specification."""
+    kh, vh, kd, vd = 2, 6, dim, (7 if dim == 5 else 128)
+    batch, steps = 5, 4
+    p = capi.delta_params(kh, vh, kd, vd, round_to_bfloat16=round_flag)
+    po = oracle.delta_params(kh, vh, kd, vd, round_to_bfloat16=round_flag)
+    channels = 2 * kh * kd + vh * vd
+    w, a_log, dt, norm = layer_weights(kh, vh, kd, vd, 4)
+    dw, dal, ddt, dn = dev(w), dev(a_log), dev(dt), dev(norm)
+    together = capi.DeltaNetStep(p, batch=batch)
+    alone = [capi.DeltaNetStep(p) for _ in range(batch)]
+    reference = oracle.DeltaNetStep(po)   # sequence 3
+    rng = np.random.default_rng(dim + round_flag)
+    for step in range(steps):
+        qkv = rng.standard_normal((batch, channels)).astype(np.float32)
+        z = rng.standard_normal((batch, vh * vd)).astype(np.float32)
+        a = rng.standard_normal((batch, vh)).astype(np.float32)
+        b = rng.standard_normal((batch, vh)).astype(np.float32)
+        got = together.step(dev(qkv), dev(z), dev(a), dev(b), dw, dal, ddt, dn).cpu().numpy()
+        for s in range(batch):
+            one = alone[s].step(dev(qkv[s]), dev(z[s]), dev(a[s]), dev(b[s]), dw, dal, ddt, dn)
+            np.testing.assert_array_equal(got[s], one.cpu().numpy())
+        want = reference.step(qkv[3], z[3], a[3], b[3], w, a_log, dt, norm)
+        loose = 2e-4 + 1.6e-2 * np.abs(want) if round_flag else 3e-5 + 1e-4 * np.abs(want)
+        assert np.all(np.abs(got[3] - want) <= loose)
+    for s in range(batch):
+        np.testing.assert_array_equal(together.state[s].cpu().numpy(),
+                                      alone[s].state.cpu().numpy())
+        np.testing.assert_array_equal(together.conv[s].cpu().numpy(), alone[s].conv.cpu().numpy())
+
+
+def test_batched_step_rejects_bad_arguments(capi):
+    import ctypes
+    p = capi.delta_params(2, 4, 16, 16)
+    lib = capi.lib()
+    assert lib.pluto_hip_gdn_step_batch_workspace_bytes(ctypes.byref(p), 0) == 0
+    size = lib.pluto_hip_gdn_step_batch_workspace_bytes(ctypes.byref(p), 3)
+    assert size >= 3 * lib.pluto_hip_gdn_step_workspace_bytes(ctypes.byref(p)) // 2
+    x = torch.zeros(4096, device="cuda")
+    px = capi.ptr(x)
+    args = [px] * 11
+    assert lib.pluto_hip_gdn_step_batch(capi.current_stream(), ctypes.byref(p), 0, *args, px, size) != 0
+    assert lib.pluto_hip_gdn_step_batch(capi.current_stream(), ctypes.byref(p), 3, *args, px, 16) != 0
+    assert lib.pluto_hip_gdn_step_batch(capi.current_stream(), ctypes.byref(p), 3, None, *args[1:], px,
+                                        size) != 0
+
+
 @pytest.mark.parametrize("kh,vh,kd,vd,T,round_flag", [(2, 6, 5, 7, 9, False), (2, 6, 5, 7, 9, True),
                                                      (2, 4, 128, 128, 7, True), (2, 4, 128, 128, 200, True),
                                                      (1, 2, 128, 128, 70, False)])
