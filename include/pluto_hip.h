@@ -414,6 +414,34 @@ int pluto_hip_gdn_step_batch(void* stream, const pluto_hip_delta_params* p,
                              float* output, void* workspace,
                              size_t workspace_bytes);
 
+/* FullyConnectedLayer, trainable path: the projections either side of the
+ * attention layers (src/llm/layers/fully_connected.cc: DenseForwardKernel
+ * :97-131, DenseInputGradientKernel :134-164, DenseWeightGradientKernel
+ * :167-196, the bias gradient kernels :198-247; fwd_impl :415-454, bwd_impl
+ * :456-527).  dtype is the activation type (PLUTO_HIP_BF16 or PLUTO_HIP_F32;
+ * anything else PLUTO_HIP_EUNSUPPORTED).  Operands are multiplied as bf16
+ * (bf16 activations) or IEEE half (FP32 activations) values and summed in
+ * FP32, as the reference's MmaType does (:31-33).
+ *   input   [rows, input_dim] in dtype;  matrix fp32 [input_dim, output_dim];
+ *   bias fp32 [output_dim];  output [rows, output_dim] in dtype
+ *   d_output fp32 [rows, output_dim];  d_input fp32 [rows, input_dim]
+ *   d_matrix, d_bias: shapes of the parameters, OVERWRITTEN (:190-196,241-246)
+ * With output_dim = 3 * embedding_dim the forward output is the packed
+ * [rows, Q | K | V] operand of pluto_hip_mha_forward, in its storage type.
+ * Widths that are multiples of 64 run on the matrix cores; any other positive
+ * width is accepted and takes a slower kernel with the same arithmetic. */
+size_t pluto_hip_dense_workspace_bytes(int dtype, int rows, int input_dim,
+                                       int output_dim);
+int pluto_hip_dense_forward(void* stream, int dtype, const void* input,
+                            const float* matrix, const float* bias, int rows,
+                            int input_dim, int output_dim, void* output,
+                            void* workspace, size_t workspace_bytes);
+int pluto_hip_dense_backward(void* stream, int dtype, const void* input,
+                             const float* matrix, const float* d_output,
+                             int rows, int input_dim, int output_dim,
+                             float* d_input, float* d_matrix, float* d_bias,
+                             void* workspace, size_t workspace_bytes);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1064,3 +1064,78 @@ int pluto_oracle_gdn_step(const pluto_oracle_delta_params* p,
   free(q);
   return 0;
 }
+
+/* ---- FullyConnectedLayer (fully_connected.cc:97-247) -------------------- */
+
+/* float -> IEEE binary16 -> float, round to nearest even, with subnormals and
+ * overflow to infinity (what element_cast<__half> does). */
+float pluto_oracle_half_round(float value) {
+  if (isnan(value) || isinf(value)) return value;
+  const float magnitude = fabsf(value);
+  if (magnitude >= 65520.0f) return copysignf(INFINITY, value); /* above the largest half + 1/2 ulp */
+  float scaled;
+  if (magnitude < 6.103515625e-05f) {
+    /* subnormal halves: multiples of 2^-24 */
+    scaled = nearbyintf(magnitude * 16777216.0f) / 16777216.0f;
+  } else {
+    int exponent;
+    const float mantissa = frexpf(magnitude, &exponent); /* in [0.5, 1) */
+    scaled = ldexpf(nearbyintf(ldexpf(mantissa, 11)), exponent - 11);
+  }
+  return copysignf(scaled, value);
+}
+
+static float dense_operand(int dtype, float value) {
+  return dtype == PLUTO_ORACLE_BF16 ? pluto_oracle_bf16_round(value)
+                                    : pluto_oracle_half_round(value);
+}
+
+int pluto_oracle_dense_forward(int dtype, int rows, int input_dim, int output_dim,
+                               const float* x, const float* matrix, const float* bias,
+                               float* y) {
+  if ((dtype != PLUTO_ORACLE_BF16 && dtype != PLUTO_ORACLE_F32) || rows <= 0 || input_dim <= 0 ||
+      output_dim <= 0 || !x || !matrix || !bias || !y)
+    return 1;
+  for (int r = 0; r < rows; ++r)
+    for (int o = 0; o < output_dim; ++o) {
+      double sum = bias[o];
+      for (int i = 0; i < input_dim; ++i)
+        sum += (double)dense_operand(dtype, x[(size_t)r * input_dim + i]) *
+               (double)dense_operand(dtype, matrix[(size_t)i * output_dim + o]);
+      const float value = (float)sum;
+      y[(size_t)r * output_dim + o] =
+          dtype == PLUTO_ORACLE_BF16 ? pluto_oracle_bf16_round(value) : value;
+    }
+  return 0;
+}
+
+int pluto_oracle_dense_backward(int dtype, int rows, int input_dim, int output_dim,
+                                const float* x, const float* matrix, const float* dy,
+                                float* dx, float* d_matrix, float* d_bias) {
+  if ((dtype != PLUTO_ORACLE_BF16 && dtype != PLUTO_ORACLE_F32) || rows <= 0 || input_dim <= 0 ||
+      output_dim <= 0 || !x || !matrix || !dy || !dx || !d_matrix || !d_bias)
+    return 1;
+  for (int r = 0; r < rows; ++r)
+    for (int i = 0; i < input_dim; ++i) {
+      double sum = 0.0;
+      for (int o = 0; o < output_dim; ++o)
+        sum += (double)dense_operand(dtype, dy[(size_t)r * output_dim + o]) *
+               (double)dense_operand(dtype, matrix[(size_t)i * output_dim + o]);
+      dx[(size_t)r * input_dim + i] = (float)sum;
+    }
+  for (int i = 0; i < input_dim; ++i)
+    for (int o = 0; o < output_dim; ++o) {
+      double sum = 0.0;
+      for (int r = 0; r < rows; ++r)
+        sum += (double)dense_operand(dtype, x[(size_t)r * input_dim + i]) *
+               (double)dense_operand(dtype, dy[(size_t)r * output_dim + o]);
+      d_matrix[(size_t)i * output_dim + o] = (float)sum;
+    }
+  for (int o = 0; o < output_dim; ++o) {
+    double sum = 0.0;
+    for (int r = 0; r < rows; ++r) sum += dy[(size_t)r * output_dim + o];
+    d_bias[o] = (float)sum;
+  }
+  return 0;
+}
+

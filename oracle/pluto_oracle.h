@@ -213,6 +213,27 @@ int pluto_oracle_gdn_step(const pluto_oracle_delta_params* p,
                           const float* a_log, const float* dt_bias,
                           const float* norm, float* output);
 
+/* FullyConnectedLayer, trainable path (src/llm/layers/fully_connected.cc:
+ * DenseForwardKernel :97-131, DenseInputGradientKernel :134-164,
+ * DenseWeightGradientKernel :167-196, the bias gradient :198-247).  dtype is
+ * the activation storage: PLUTO_ORACLE_BF16 (0x1) multiplies operands rounded
+ * to bf16, PLUTO_ORACLE_F32 (0x0) operands rounded to IEEE half (MmaType,
+ * :31-33); sums are kept in double here (FP32 in the reference, order
+ * unspecified).  matrix is [input_dim, output_dim], bias [output_dim].
+ *   forward:  y[r, o] = bias[o] + sum_i R(x[r, i]) R(w[i, o]), stored in the
+ *             activation type (rounded to bf16 for bf16 storage)
+ *   backward: dx[r, i] = sum_o R(dy[r, o]) R(w[i, o])
+ *             dw[i, o] = sum_r R(x[r, i]) R(dy[r, o])
+ *             db[o]    = sum_r dy[r, o]            (dy unrounded)
+ * x is given as float values (bf16-representable for bf16 storage). */
+float pluto_oracle_half_round(float value);
+int pluto_oracle_dense_forward(int dtype, int rows, int input_dim, int output_dim,
+                               const float* x, const float* matrix, const float* bias,
+                               float* y);
+int pluto_oracle_dense_backward(int dtype, int rows, int input_dim, int output_dim,
+                                const float* x, const float* matrix, const float* dy,
+                                float* dx, float* d_matrix, float* d_bias);
+
 #ifdef __cplusplus
 }
 #endif

@@ -18,8 +18,9 @@ BF16 = 1
 
 def build(force=False):
     """Compile liboracle.so with the Makefile beside this file."""
-    if force or not os.path.exists(_LIB_PATH):
-        subprocess.check_call(["make", "-C", _HERE, "-B" if force else "-s"])
+    # make compares time stamps itself: a stale library is rebuilt, a current
+    # one costs a few milliseconds
+    subprocess.check_call(["make", "-C", _HERE, "-B" if force else "-s"])
     return _LIB_PATH
 
 
@@ -346,3 +347,46 @@ class DeltaNetStep:
         if rc != 0:
             raise ValueError("oracle rejected the delta-net step")
         return out
+
+
+def half_round(x):
+    """float32 -> IEEE half -> float32 (round to nearest even), elementwise."""
+    x = _f32(x)
+    out = np.empty_like(x)
+    fn = lib().pluto_oracle_half_round
+    fn.restype = ctypes.c_float
+    fn.argtypes = [ctypes.c_float]
+    flat_in, flat_out = x.ravel(), out.ravel()
+    for i in range(flat_in.size):
+        flat_out[i] = fn(float(flat_in[i]))
+    return out
+
+
+def dense_forward(dtype, x, matrix, bias):
+    """FullyConnectedLayer forward: x [rows, in] (float values), matrix [in, out],
+    bias [out] -> y [rows, out] in the activation type's value set."""
+    x, matrix, bias = _f32(x), _f32(matrix), _f32(bias)
+    rows, input_dim = x.shape
+    output_dim = matrix.shape[1]
+    y = np.zeros((rows, output_dim), np.float32)
+    fn = lib().pluto_oracle_dense_forward
+    fn.restype = ctypes.c_int
+    if fn(dtype, rows, input_dim, output_dim, _ptr(x), _ptr(matrix), _ptr(bias), _ptr(y)) != 0:
+        raise ValueError("oracle rejected the dense forward")
+    return y
+
+
+def dense_backward(dtype, x, matrix, dy):
+    """Gradients (dx [rows, in], d_matrix [in, out], d_bias [out]) of dense_forward."""
+    x, matrix, dy = _f32(x), _f32(matrix), _f32(dy)
+    rows, input_dim = x.shape
+    output_dim = matrix.shape[1]
+    dx = np.zeros((rows, input_dim), np.float32)
+    dw = np.zeros((input_dim, output_dim), np.float32)
+    db = np.zeros(output_dim, np.float32)
+    fn = lib().pluto_oracle_dense_backward
+    fn.restype = ctypes.c_int
+    if fn(dtype, rows, input_dim, output_dim, _ptr(x), _ptr(matrix), _ptr(dy), _ptr(dx), _ptr(dw),
+          _ptr(db)) != 0:
+        raise ValueError("oracle rejected the dense backward")
+    return dx, dw, db

@@ -121,6 +121,10 @@ SIGNATURES = {
     "pluto_hip_gdn_step_batch_workspace_bytes": (_SZ, [ctypes.POINTER(DeltaParams), _I]),
     "pluto_hip_gdn_step_batch": (_I, [_VP, ctypes.POINTER(DeltaParams), _I] + [_VP] * 11 +
                                  [_VP, _SZ]),
+    "pluto_hip_dense_workspace_bytes": (_SZ, [_I, _I, _I, _I]),
+    "pluto_hip_dense_forward": (_I, [_VP, _I, _VP, _VP, _VP, _I, _I, _I, _VP, _VP, _SZ]),
+    "pluto_hip_dense_backward": (_I, [_VP, _I, _VP, _VP, _VP, _I, _I, _I, _VP, _VP, _VP, _VP,
+                                      _SZ]),
     "pluto_hip_gdn_recurrence": (_I, [_VP, ctypes.POINTER(DeltaParams), _I, _I, _VP, _VP,
                                       _VP, _VP, _VP, _I, ctypes.c_float, _VP, _VP, _I]),
 }
@@ -464,3 +468,40 @@ class DeltaNetStep:
             ptr(self.state), ptr(qkv), ptr(z), ptr(a), ptr(b), ptr(conv_weight), ptr(a_log),
             ptr(dt_bias), ptr(norm), ptr(out), ptr(self.workspace), self.workspace.numel()))
         return out
+
+
+def dense_workspace(x, output_dim):
+    rows, input_dim = x.shape
+    size = lib().pluto_hip_dense_workspace_bytes(dtype_code(x), rows, input_dim, output_dim)
+    return torch.empty(max(size, 16), dtype=torch.uint8, device=x.device)
+
+
+def dense_forward(x, matrix, bias, workspace=None, out=None, stream=None):
+    """FullyConnectedLayer forward: x [rows, in] (float32 or bfloat16), matrix
+    fp32 [in, out], bias fp32 [out] -> [rows, out] in x's type."""
+    rows, input_dim = x.shape
+    output_dim = matrix.shape[1]
+    if workspace is None:
+        workspace = dense_workspace(x, output_dim)
+    if out is None:
+        out = torch.empty((rows, output_dim), dtype=x.dtype, device=x.device)
+    check(lib().pluto_hip_dense_forward(stream or current_stream(), dtype_code(x), ptr(x),
+                                        ptr(matrix), ptr(bias), rows, input_dim, output_dim,
+                                        ptr(out), ptr(workspace), workspace.numel()))
+    return out
+
+
+def dense_backward(x, matrix, d_out, workspace=None, stream=None):
+    """(d_input [rows, in], d_matrix [in, out], d_bias [out]), all fp32."""
+    rows, input_dim = x.shape
+    output_dim = matrix.shape[1]
+    if workspace is None:
+        workspace = dense_workspace(x, output_dim)
+    dx = torch.empty((rows, input_dim), dtype=torch.float32, device=x.device)
+    dw = torch.empty((input_dim, output_dim), dtype=torch.float32, device=x.device)
+    db = torch.empty(output_dim, dtype=torch.float32, device=x.device)
+    check(lib().pluto_hip_dense_backward(stream or current_stream(), dtype_code(x), ptr(x),
+                                         ptr(matrix), ptr(d_out), rows, input_dim, output_dim,
+                                         ptr(dx), ptr(dw), ptr(db), ptr(workspace),
+                                         workspace.numel()))
+    return dx, dw, db
