@@ -46,7 +46,7 @@ NAMES = ["mha_train_bf16", "mha_fwd_fp32", "gqa_prefill", "gqa_decode", "gdn_sca
 # "copy" is a plain device copy of known size: the calibration case for the
 # FETCH_SIZE / WRITE_SIZE counters that `roofline.traffic` is derived from.
 # "gqa_prefill_bwd" and "gdn_layer_bwd" time the two sequence backward passes.
-EXTRA = ["copy", "gqa_prefill_bwd", "gdn_layer_bwd", "gdn_decode"]
+EXTRA = ["copy", "gqa_prefill_bwd", "gdn_layer_bwd", "gdn_decode", "dense_qkv"]
 
 
 def parse_args():
@@ -322,6 +322,39 @@ def gdn_decode(torch, capi):
                 cpu=None)
 
 
+def dense_qkv(torch, capi):
+    """The QKV projection in front of the default workload (gpt2.cc:55-71):
+    FullyConnectedLayer 768 -> 2304 on 16 x 1024 bf16 rows, forward + backward.
+    A row after the headline ones, not part of --workload all."""
+    rows, n_in, n_out = 16 * 1024, 768, 2304
+    gen = torch.Generator(device="cuda").manual_seed(6)
+    x = torch.randn((rows, n_in), generator=gen, device="cuda").to(torch.bfloat16)
+    w = torch.randn((n_in, n_out), generator=gen, device="cuda") / math.sqrt(n_in)
+    b = torch.zeros(n_out, device="cuda")
+    dy = torch.randn((rows, n_out), generator=gen, device="cuda")
+    workspace = capi.dense_workspace(x, n_out)
+    out = torch.empty((rows, n_out), dtype=torch.bfloat16, device="cuda")
+
+    def forward():
+        capi.dense_forward(x, w, b, workspace=workspace, out=out)
+
+    def backward():
+        capi.dense_backward(x, w, dy, workspace=workspace)
+
+    def step():
+        forward()
+        backward()
+
+    product = 2.0 * rows * n_in * n_out
+    return dict(step=step, parts=[("forward", forward, product), ("backward", backward, 2 * product)],
+                work=3 * product, metric="dense_fwd_bwd_tflops", unit="TFLOP/s", dtype="bf16",
+                bound="mfma", peak=PEAK_BF16_TFLOPS,
+                config={"workload": "gpt2_small_qkv_projection_fwd_bwd", "rows": rows,
+                        "input_dim": n_in, "output_dim": n_out, "storage": "bf16",
+                        "accumulate": "fp32", "master_weights": "fp32"},
+                cpu=None)
+
+
 def copy(torch, capi):
     n = 256 * 2 ** 20   # 1 GiB read + 1 GiB written per step
     src = torch.ones(n, dtype=torch.float32, device="cuda")
@@ -337,7 +370,7 @@ def copy(torch, capi):
                         "bytes_written": n * 4}, cpu=None)
 
 
-WORKLOADS = {"copy": copy, "gdn_decode": gdn_decode, "mha_train_bf16": mha_train_bf16, "mha_fwd_fp32": mha_fwd_fp32,
+WORKLOADS = {"copy": copy, "gdn_decode": gdn_decode, "dense_qkv": dense_qkv, "mha_train_bf16": mha_train_bf16, "mha_fwd_fp32": mha_fwd_fp32,
              "gqa_prefill": gqa_prefill, "gqa_prefill_bwd": gqa_prefill_bwd, "gdn_layer_bwd": gdn_layer_bwd,
              "gqa_decode": gqa_decode,
              "gdn_scan": gdn_scan}

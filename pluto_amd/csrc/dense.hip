@@ -8,7 +8,7 @@
 // master matrix [input_dim, output_dim] and the FP32 gradient are converted
 // to 16 bits once per call; the products then run on v_mfma_f32_32x32x16_*
 // from LDS tiles filled by direct-to-LDS loads:
-//   y^T and dx^T:  rows of both operands are contiguous along the contraction
+//   y and dx:      rows of both operands are contiguous along the contraction
 //                  (x and w^T; dy and w) -> 16-byte row reads
 //   dw:            the contraction runs over tokens, both operands (x, dy) are
 //                  read through the LDS transpose read; the token range is
@@ -26,9 +26,7 @@ namespace {
 typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
 
 constexpr int kThreads = 256;
-constexpr int kTile = 128;        // output tile edge of the matrix-core kernels
 constexpr int kDepth = 64;        // contraction elements per LDS tile
-constexpr int kTileBytes = kTile * kDepth * 2;
 constexpr int kBiasRows = 256;    // fully_connected.cc:38
 
 template <bool HALF>
@@ -95,98 +93,135 @@ struct ProductArgs {
   bool out_bf16 = false;
 };
 
+// Workgroup barrier that leaves queued global loads in flight (the library
+// barrier waits for them too).
+__device__ inline void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+template <int COUNT>
+__device__ inline void wait_loads() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(COUNT) : "memory");
+}
+
 // out[m, n] = bias[n] + sum_k left[m, k] right[n, k]; depth % 64 == 0.  A
-// workgroup owns a 128 x 128 tile, wave w the 64 x 64 quarter (w / 2, w % 2).
-// The product is computed transposed (A operand = rows of `right`), so a lane
-// ends up with four consecutive n of one output row m: 8- or 16-byte stores.
-template <bool HALF>
-__global__ void __launch_bounds__(kThreads)
-__attribute__((amdgpu_waves_per_eu(2, 2)))
+// workgroup of NWAVES waves, arranged 2 x (NWAVES / 2), owns a
+// (64 JM) x (16 NWAVES JN) tile and each wave a (32 JM) x (32 JN) part of it.
+// STAGES LDS stages of 64 contraction elements are filled STAGES - 1 steps
+// ahead.
+template <bool HALF, int JM, int JN, int STAGES, int NWAVES>
+__global__ void __launch_bounds__(64 * NWAVES)
 product_rows_kernel(ProductArgs a) {
-  __shared__ __attribute__((aligned(1024))) unsigned char lds[4 * kTileBytes];
+  constexpr int THREADS = 64 * NWAVES;
+  constexpr int KS = kDepth / 16;  // matrix instructions along the contraction per stage
+  constexpr int TM = 64 * JM, TN = 32 * (NWAVES / 2) * JN;
+  constexpr int kLeftBytes = TM * kDepth * 2, kRightBytes = TN * kDepth * 2;
+  constexpr int kStageBytes = kLeftBytes + kRightBytes;
+  constexpr int LEFT_LOADS = TM * (kDepth / 8) / THREADS;
+  constexpr int RIGHT_LOADS = TN * (kDepth / 8) / THREADS;
+  __shared__ __attribute__((aligned(1024))) unsigned char lds[STAGES * kStageBytes];
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
   const int h = lane / 32, n = lane % 32;
-  const int n_tiles = (a.n_rows + kTile - 1) / kTile;
+  const int n_tiles = (a.n_rows + TN - 1) / TN;
   const int logical = xcd_logical_block();
-  const int m0 = (logical / n_tiles) * kTile, n0 = (logical % n_tiles) * kTile;
-  const int wm = 64 * (wave / 2), wn = 64 * (wave % 2);
-  constexpr int LOADS = kTile * (kDepth / 8) / kThreads;  // 4
-  uint32_t fill[LOADS];
+  const int m0 = (logical / n_tiles) * TM, n0 = (logical % n_tiles) * TN;
+  const int wm = 32 * JM * (wave / (NWAVES / 2)), wn = 32 * JN * (wave % (NWAVES / 2));
+  uint32_t left_fill[LEFT_LOADS], right_fill[RIGHT_LOADS];
 #pragma unroll
-  for (int i = 0; i < LOADS; ++i)
-    fill[i] = tile_fill_offset<kDepth>((wave * LOADS + i) * 64 + lane, a.depth);
-  int left_read[2][4], right_read[2][4];
+  for (int i = 0; i < LEFT_LOADS; ++i)
+    left_fill[i] = tile_fill_offset<kDepth>((wave * LEFT_LOADS + i) * 64 + lane, a.depth);
 #pragma unroll
-  for (int j = 0; j < 2; ++j)
+  for (int i = 0; i < RIGHT_LOADS; ++i)
+    right_fill[i] = tile_fill_offset<kDepth>((wave * RIGHT_LOADS + i) * 64 + lane, a.depth);
+  // Rows 32 apart share the swizzle: block j of a quarter is 32 j rows further.
+  constexpr int kBlockStep = 32 * (kDepth / 8) * 16;
+  int left_read[KS], right_read[KS];
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      left_read[j][ks] = tile_row_read<kDepth>(wm + 32 * j + n, 2 * ks + h);
-      right_read[j][ks] = tile_row_read<kDepth>(wn + 32 * j + n, 2 * ks + h);
-    }
-  // acc[jn][jm]: rows = output columns n (A operand), columns = output rows m
-  floatx16 acc[2][2];
+  for (int ks = 0; ks < KS; ++ks) {
+    left_read[ks] = tile_row_read<kDepth>(wm + n, 2 * ks + h);
+    right_read[ks] = tile_row_read<kDepth>(wn + n, 2 * ks + h);
+  }
+  // acc[jm][jn]: a lane holds output column n0 + wn + 32 jn + n of rows
+  // m0 + wm + 32 jm + 8 q + 4 h + i (element 4 q + i)
+  floatx16 acc[JM][JN];
 #pragma unroll
-  for (int jn = 0; jn < 2; ++jn)
+  for (int jn = 0; jn < JN; ++jn) {
+    const int column = n0 + wn + 32 * jn + n;
+    const float start = (a.bias && column < a.n_rows) ? a.bias[column] : 0.0f;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int column = n0 + wn + 32 * jn + 8 * (i / 4) + 4 * h + i % 4;
-      const float start = (a.bias && column < a.n_rows) ? a.bias[column] : 0.0f;
-      acc[jn][0][i] = start;
-      acc[jn][1][i] = start;
-    }
+    for (int jm = 0; jm < JM; ++jm)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[jm][jn][i] = start;
+  }
   const uint16_t* left = a.left + static_cast<long long>(m0) * a.depth;
   const uint16_t* right = a.right + static_cast<long long>(n0) * a.depth;
   const int steps = a.depth / kDepth;
   auto fill_stage = [&](int step) {
-    unsigned char* stage = lds + (step & 1) * 2 * kTileBytes;
-    tile_fill<kDepth, LOADS>(stage, wave, left + step * kDepth, a.depth, m0, a.m_rows, fill);
-    tile_fill<kDepth, LOADS>(stage + kTileBytes, wave, right + step * kDepth, a.depth, n0,
-                             a.n_rows, fill);
+    unsigned char* stage = lds + (step % STAGES) * kStageBytes;
+    tile_fill<kDepth, LEFT_LOADS>(stage, wave, left + step * kDepth, a.depth, m0, a.m_rows,
+                                  left_fill);
+    tile_fill<kDepth, RIGHT_LOADS>(stage + kLeftBytes, wave, right + step * kDepth, a.depth, n0,
+                                   a.n_rows, right_fill);
   };
-  fill_stage(0);
+  for (int step = 0; step < STAGES - 1 && step < steps; ++step) fill_stage(step);
   for (int step = 0; step < steps; ++step) {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    if (step + 1 < steps) fill_stage(step + 1);
-    const unsigned char* left_tile = lds + (step & 1) * 2 * kTileBytes;
-    const unsigned char* right_tile = left_tile + kTileBytes;
+    // stage `step` has landed once at most the STAGES - 2 later fills remain
+    if (step + STAGES - 2 < steps)
+      wait_loads<(STAGES - 2) * (LEFT_LOADS + RIGHT_LOADS)>();
+    else
+      wait_loads<0>();
+    lds_barrier();
+    if (step + STAGES - 1 < steps) fill_stage(step + STAGES - 1);
+    const unsigned char* left_tile = lds + (step % STAGES) * kStageBytes;
+    const unsigned char* right_tile = left_tile + kLeftBytes;
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      uint4 l[2], r[2];
+    for (int ks = 0; ks < KS; ++ks) {
+      uint4 l[JM], r[JN];
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        l[j] = *reinterpret_cast<const uint4*>(left_tile + left_read[j][ks]);
-        r[j] = *reinterpret_cast<const uint4*>(right_tile + right_read[j][ks]);
-      }
+      for (int j = 0; j < JM; ++j)
+        l[j] = *reinterpret_cast<const uint4*>(left_tile + left_read[ks] + j * kBlockStep);
 #pragma unroll
-      for (int jn = 0; jn < 2; ++jn)
+      for (int j = 0; j < JN; ++j)
+        r[j] = *reinterpret_cast<const uint4*>(right_tile + right_read[ks] + j * kBlockStep);
 #pragma unroll
-        for (int jm = 0; jm < 2; ++jm) acc[jn][jm] = mma<HALF>(r[jn], l[jm], acc[jn][jm]);
+      for (int jm = 0; jm < JM; ++jm)
+#pragma unroll
+        for (int jn = 0; jn < JN; ++jn) acc[jm][jn] = mma<HALF>(l[jm], r[jn], acc[jm][jn]);
     }
   }
+  // 32 lanes store 32 consecutive columns of a row: 64 or 128 contiguous bytes
 #pragma unroll
-  for (int jm = 0; jm < 2; ++jm) {
-    const int row = m0 + wm + 32 * jm + n;
-    if (row >= a.m_rows) continue;
+  for (int jm = 0; jm < JM; ++jm)
 #pragma unroll
-    for (int jn = 0; jn < 2; ++jn)
+    for (int jn = 0; jn < JN; ++jn) {
+      const int column = n0 + wn + 32 * jn + n;
+      if (column >= a.n_rows) continue;
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int column = n0 + wn + 32 * jn + 8 * q + 4 * h;
-        if (column >= a.n_rows) continue;  // n_rows is a multiple of 4 on this path
+      for (int i = 0; i < 16; ++i) {
+        const int row = m0 + wm + 32 * jm + 8 * (i / 4) + 4 * h + i % 4;
+        if (row >= a.m_rows) continue;
         const long long at = static_cast<long long>(row) * a.n_rows + column;
-        const floatx16& c = acc[jn][jm];
-        if (a.out_bf16) {
-          uint2 packed;
-          packed.x = pack_bf16(c[4 * q], c[4 * q + 1]);
-          packed.y = pack_bf16(c[4 * q + 2], c[4 * q + 3]);
-          *reinterpret_cast<uint2*>(static_cast<uint16_t*>(a.out) + at) = packed;
-        } else {
-          *reinterpret_cast<float4*>(static_cast<float*>(a.out) + at) =
-              make_float4(c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3]);
-        }
+        if (a.out_bf16)
+          static_cast<uint16_t*>(a.out)[at] = float_to_bf16_bits(acc[jm][jn][i]);
+        else
+          static_cast<float*>(a.out)[at] = acc[jm][jn][i];
       }
-  }
+    }
+}
+
+// Short contractions take 128 x 128 tiles (more workgroups to overlap the
+// start-up and the stores); from 1536 elements on, 256 x 256 tiles of eight
+// waves, which halve the operand traffic from L2, are faster.
+template <bool HALF>
+void launch_product_rows(hipStream_t s, const ProductArgs& p) {
+  auto blocks = [&](int tm, int tn) {
+    return static_cast<unsigned>((p.m_rows + tm - 1) / tm) *
+           static_cast<unsigned>((p.n_rows + tn - 1) / tn);
+  };
+  if (p.depth >= 1536)
+    product_rows_kernel<HALF, 4, 2, 2, 8><<<blocks(256, 256), 512, 0, s>>>(p);
+  else
+    product_rows_kernel<HALF, 2, 2, 2, 4><<<blocks(128, 128), 256, 0, s>>>(p);
 }
 
 struct GramArgs {
@@ -305,22 +340,57 @@ sum_slices_kernel(const float* partial, long long elements, int slices, float* o
 }
 
 // Column sums of [rows, width] in two levels with a fixed order
-// (fully_connected.cc:198-247: 256-row partitions, then the partitions).
+// (fully_connected.cc:198-247: 256-row partitions, then the partitions), and
+// optionally the 16-bit copy of the same values: the gradient is read once
+// for both.  A workgroup takes 64 columns of a 256-row partition; thread
+// (lane, quad) = (tid / 16, tid % 16) adds rows lane, lane + 16, ... of four
+// adjacent columns, and the sixteen lanes' sums are added in ascending order.
+template <bool HALF>
 __global__ void __launch_bounds__(256)
-column_partial_kernel(const float* in, int rows, int width, float* partial) {
-  const int c = blockIdx.x * 256 + threadIdx.x;
-  if (c >= width) return;
+column_partial_kernel(const float* in, int rows, int width, float* partial, uint16_t* copy) {
+  __shared__ float lanes[16][64];
+  const int quad = threadIdx.x % 16, lane = threadIdx.x / 16;
+  const int c = blockIdx.x * 64 + quad * 4;
   const int r0 = blockIdx.y * kBiasRows, r1 = min(r0 + kBiasRows, rows);
-  float sum = 0.0f;
-  for (int r = r0; r < r1; ++r) sum += in[static_cast<long long>(r) * width + c];
-  partial[static_cast<long long>(blockIdx.y) * width + c] = sum;
+  float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  if (width % 4 == 0 && c < width) {
+#pragma unroll 4
+    for (int r = r0 + lane; r < r1; r += 16) {
+      const long long at = static_cast<long long>(r) * width + c;
+      const float4 value = *reinterpret_cast<const float4*>(in + at);
+      sum[0] += value.x, sum[1] += value.y, sum[2] += value.z, sum[3] += value.w;
+      if (copy) {
+        ushort4 out;
+        out.x = to_operand<HALF>(value.x), out.y = to_operand<HALF>(value.y);
+        out.z = to_operand<HALF>(value.z), out.w = to_operand<HALF>(value.w);
+        *reinterpret_cast<ushort4*>(copy + at) = out;
+      }
+    }
+  } else {
+    for (int r = r0 + lane; r < r1; r += 16)
+      for (int e = 0; e < 4; ++e)
+        if (c + e < width) {
+          const float value = in[static_cast<long long>(r) * width + c + e];
+          sum[e] += value;
+          if (copy) copy[static_cast<long long>(r) * width + c + e] = to_operand<HALF>(value);
+        }
+  }
+  for (int e = 0; e < 4; ++e) lanes[lane][quad * 4 + e] = sum[e];
+  __syncthreads();
+  const int column = blockIdx.x * 64 + threadIdx.x;
+  if (threadIdx.x < 64 && column < width) {
+    float total = lanes[0][threadIdx.x];
+    for (int l = 1; l < 16; ++l) total += lanes[l][threadIdx.x];
+    partial[static_cast<long long>(blockIdx.y) * width + column] = total;
+  }
 }
 
 __global__ void __launch_bounds__(256)
 column_final_kernel(const float* partial, int parts, int width, float* out) {
-  const int c = blockIdx.x * 256 + threadIdx.x;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= width) return;
   float sum = 0.0f;
+#pragma unroll 16
   for (int p = 0; p < parts; ++p) sum += partial[static_cast<long long>(p) * width + c];
   out[c] = sum;
 }
@@ -375,7 +445,8 @@ bool matrix_cores(int input_dim, int output_dim) {
 
 int weight_slices(int rows, int input_dim, int output_dim) {
   const long long tiles = ((input_dim + 127) / 128) * static_cast<long long>((output_dim + 127) / 128);
-  long long slices = (512 + tiles - 1) / tiles;  // two workgroups a compute unit
+  // two workgroups a compute unit: as many slices as still run in one round
+  long long slices = 512 / tiles;
   const long long most = (rows + 255) / 256;     // at least 256 rows a slice
   if (slices > most) slices = most;
   return static_cast<int>(slices < 1 ? 1 : slices);
@@ -438,9 +509,7 @@ int forward(hipStream_t s, int dtype, const void* input, const float* matrix, co
   p.n_rows = output_dim;
   p.depth = input_dim;
   p.out_bf16 = dtype == PLUTO_HIP_BF16;
-  const unsigned grid = static_cast<unsigned>((rows + kTile - 1) / kTile) *
-                        static_cast<unsigned>((output_dim + kTile - 1) / kTile);
-  product_rows_kernel<HALF><<<grid, kThreads, 0, s>>>(p);
+  launch_product_rows<HALF>(s, p);
   return launch_status();
 }
 
@@ -452,11 +521,13 @@ int backward(hipStream_t s, int dtype, const void* input, const float* matrix,
   // bias gradient: 256-row partitions, then the partitions in order
   float* bias_partial = reinterpret_cast<float*>(scratch + l.bias_partial);
   const int parts = (rows + kBiasRows - 1) / kBiasRows;
-  column_partial_kernel<<<dim3((output_dim + 255) / 256, parts), 256, 0, s>>>(d_output, rows,
-                                                                              output_dim, bias_partial);
-  column_final_kernel<<<(output_dim + 255) / 256, 256, 0, s>>>(bias_partial, parts, output_dim,
-                                                               d_bias);
-  if (!matrix_cores(input_dim, output_dim)) {
+  const bool cores = matrix_cores(input_dim, output_dim);
+  uint16_t* gradient16 = reinterpret_cast<uint16_t*>(scratch + l.gradient16);  // dy [rows, out]
+  column_partial_kernel<HALF><<<dim3((output_dim + 63) / 64, parts), 256, 0, s>>>(
+      d_output, rows, output_dim, bias_partial, cores ? gradient16 : nullptr);
+  column_final_kernel<<<(output_dim + 63) / 64, 64, 0, s>>>(bias_partial, parts, output_dim,
+                                                            d_bias);
+  if (!cores) {
     generic_dense_kernel<HALF><<<blocks_for(1LL * rows * input_dim), 256, 0, s>>>(
         1, dtype, input, matrix, d_output, nullptr, rows, input_dim, output_dim, d_input);
     generic_dense_kernel<HALF><<<blocks_for(1LL * input_dim * output_dim), 256, 0, s>>>(
@@ -464,9 +535,7 @@ int backward(hipStream_t s, int dtype, const void* input, const float* matrix,
     return launch_status();
   }
   uint16_t* matrix16 = reinterpret_cast<uint16_t*>(scratch + l.matrix16);      // w [in, out]
-  uint16_t* gradient16 = reinterpret_cast<uint16_t*>(scratch + l.gradient16);  // dy [rows, out]
   convert<HALF, false>(s, matrix, input_dim, output_dim, matrix16);
-  convert<HALF, false>(s, d_output, rows, output_dim, gradient16);
   const uint16_t* input16 = static_cast<const uint16_t*>(input);
   if (dtype == PLUTO_HIP_F32) {
     uint16_t* copy = reinterpret_cast<uint16_t*>(scratch + l.input16);
@@ -481,9 +550,7 @@ int backward(hipStream_t s, int dtype, const void* input, const float* matrix,
   p.m_rows = rows;
   p.n_rows = input_dim;
   p.depth = output_dim;
-  const unsigned grid = static_cast<unsigned>((rows + kTile - 1) / kTile) *
-                        static_cast<unsigned>((input_dim + kTile - 1) / kTile);
-  product_rows_kernel<HALF><<<grid, kThreads, 0, s>>>(p);
+  launch_product_rows<HALF>(s, p);
   int status = launch_status();
   if (status != 0) return status;
   // dw[i, o] = sum_r x[r, i] dy[r, o], the rows in slices
