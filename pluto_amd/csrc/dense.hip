@@ -279,12 +279,11 @@ product_columns_kernel(GramArgs a) {
                        const uint32_t* offsets) {
     const long long begin = static_cast<long long>(r0) * stride + col0;
     const long long left_elements = static_cast<long long>(last) * stride - begin;
-    const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(
+    const int32x4 rsrc = make_rsrc(
         matrix + begin, left_elements <= 0 ? 0u : static_cast<uint32_t>(left_elements * 2));
 #pragma unroll
     for (int i = 0; i < LOADS; ++i)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(
-          rsrc, (lds_void*)(tile + (wave * LOADS + i) * 1024), 16, offsets[i], 0, 0, 0);
+      lds_fill<16>(rsrc, tile + (wave * LOADS + i) * 1024, offsets[i]);
   };
   auto fill_stage = [&](int step) {
     unsigned char* stage = lds + (step & 1) * 2 * kBytes;

@@ -262,10 +262,9 @@ __device__ inline void dkv_fill_stage(unsigned char* stage, int wave, int lane,
   if (wave < 2) {
     const float* source = wave == 0 ? lse2_base : delta_base;
     const int left = T - q0;
-    const __amdgpu_buffer_rsrc_t rsrc =
+    const int32x4 rsrc =
         make_rsrc(source + q0, left <= 0 ? 0u : static_cast<uint32_t>(left) * 4u);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(
-        rsrc, (lds_void*)(stage + 2 * kTileBytes + wave * 256), 4, lane * 4, 0, 0, 0);
+    lds_fill<4>(rsrc, stage + 2 * kTileBytes + wave * 256, lane * 4);
   }
 }
 

@@ -45,19 +45,17 @@ __device__ inline void fill_stage(unsigned char* stage, int wave, const uint16_t
                                   const uint32_t* k_fill, const uint32_t* v_fill) {
   constexpr int kTileBytes = BN * D * 2;
   const long long rows_left = kv_rows - 1 - k0;
-  const __amdgpu_buffer_rsrc_t k_rsrc =
+  const int32x4 k_rsrc =
       make_rsrc(k_base + static_cast<long long>(k0) * k_row_stride,
                 static_cast<uint32_t>((rows_left * k_row_stride + D) * 2));
-  const __amdgpu_buffer_rsrc_t v_rsrc =
+  const int32x4 v_rsrc =
       make_rsrc(v_base + static_cast<long long>(k0) * v_row_stride,
                 static_cast<uint32_t>((rows_left * v_row_stride + D) * 2));
 #pragma unroll
   for (int i = 0; i < LOADS; ++i) {
     const int at = (wave * LOADS + i) * 1024;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, (lds_void*)(stage + at), 16, k_fill[i], 0, 0,
-                                             0);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc, (lds_void*)(stage + kTileBytes + at), 16,
-                                             v_fill[i], 0, 0, 0);
+    lds_fill<16>(k_rsrc, stage + at, k_fill[i]);
+    lds_fill<16>(v_rsrc, stage + kTileBytes + at, v_fill[i]);
   }
 }
 

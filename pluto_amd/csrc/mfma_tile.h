@@ -87,9 +87,42 @@ __device__ inline floatx16 mfma32(bf16x8 a, bf16x8 b, floatx16 c) {
 typedef __attribute__((ext_vector_type(4))) short shortx4;
 typedef __attribute__((address_space(3))) void lds_void;
 
-// Buffer descriptor over [base, base + bytes): loads beyond `bytes` return 0.
-__device__ inline __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
+// Buffer descriptor over [base, base + bytes) for direct-to-LDS loads: loads
+// beyond `bytes` deliver 0.  base and bytes must be the same in every lane.
+typedef int int32x4 __attribute__((ext_vector_type(4)));
+__device__ inline int32x4 make_rsrc(const void* base, uint32_t bytes) {
+  const uint64_t address = reinterpret_cast<uint64_t>(base);
+  int32x4 d;
+  d.x = __builtin_amdgcn_readfirstlane(static_cast<int>(address));
+  d.y = __builtin_amdgcn_readfirstlane(static_cast<int>((address >> 32) & 0xffff));
+  d.z = __builtin_amdgcn_readfirstlane(static_cast<int>(bytes));
+  d.w = 0x00020000;
+  return d;
+}
+
+// One direct-to-LDS load: lane l's BYTES (16 or 4) from byte `offset` of the
+// descriptor land at `lds` + l * BYTES; `lds` is the same in every lane.
+// Written as assembly on purpose: for the builtin the compiler makes every
+// later LDS read wait for all outstanding fills (it cannot tell the stage that
+// is being filled from the one that is being read), which serializes a
+// double-buffered loop inside each wave.  Callers order fills and reads
+// themselves: s_waitcnt vmcnt + a workgroup barrier before a stage is read,
+// a barrier after its last read before it is refilled.
+template <int BYTES>
+__device__ inline void lds_fill(int32x4 descriptor, const void* lds, uint32_t offset) {
+  static_assert(BYTES == 16 || BYTES == 4);
+  const uint32_t address = __builtin_amdgcn_readfirstlane(
+      static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_void*)lds)));
+  if constexpr (BYTES == 16)
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                 :
+                 : "s"(address), "v"(offset), "s"(descriptor)
+                 : "memory");
+  else
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, 0 offen lds"
+                 :
+                 : "s"(address), "v"(offset), "s"(descriptor)
+                 : "memory");
 }
 
 // LDS transpose read (ds_read_b64_tr_b16).  Within every group of 16 lanes,
@@ -146,12 +179,11 @@ __device__ inline void tile_fill(unsigned char* tile, int wave, const uint16_t* 
                                  long long row_stride, int row0, int rows,
                                  const uint32_t* offsets) {
   const long long rows_left = rows - 1 - row0;
-  const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(
+  const int32x4 rsrc = make_rsrc(
       base, rows_left < 0 ? 0u : static_cast<uint32_t>((rows_left * row_stride + D) * 2));
 #pragma unroll
   for (int i = 0; i < LOADS; ++i)
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(
-        rsrc, (lds_void*)(tile + (wave * LOADS + i) * 1024), 16, offsets[i], 0, 0, 0);
+    lds_fill<16>(rsrc, tile + (wave * LOADS + i) * 1024, offsets[i]);
 }
 
 template <int D>
