@@ -36,7 +36,7 @@ def test_closed_form_two_tokens(oracle):
     w1, w2 = math.exp(2 * scale), math.exp(4 * scale)
     assert out[0, 0] == pytest.approx(1.0, abs=1e-6)
     assert out[1, 0] == pytest.approx((w1 + 2 * w2) / (w1 + w2), abs=1e-5)
-    # the survey's recorded value of the same closed form
+    # the same closed form evaluated for a head width of 16: sigmoid(0.5) + 1
     assert out[1, 0] == pytest.approx(1.622459, abs=1e-5)
     d_out = np.zeros((rows, E), np.float32)
     d_out[0, 0] = 1
