@@ -1,5 +1,5 @@
 // The attention block of a GPT-2 layer through the host API: QKV projection,
-// causal attention, output projection (src/llm/gpt2 builds the same chain from
+// causal attention, output projection (src/llm/gpt2.cc:55-68 builds the same chain from
 // FullyConnectedLayer and AttentionLayer).  Forward and backward are compared
 // with the same chain of CPU oracles.
 #include "pluto_amd/host/attention.h"
