@@ -107,7 +107,10 @@ __device__ inline int32x4 make_rsrc(const void* base, uint32_t bytes) {
 // is being filled from the one that is being read), which serializes a
 // double-buffered loop inside each wave.  Callers order fills and reads
 // themselves: s_waitcnt vmcnt + a workgroup barrier before a stage is read,
-// a barrier after its last read before it is refilled.
+// a barrier after its last read before it is refilled.  The statement
+// overwrites M0 without declaring it (the compiler rejects M0 in a clobber
+// list): kernels that use it must not index register arrays dynamically,
+// the only other thing the compiler would use M0 for on this target.
 template <int BYTES>
 __device__ inline void lds_fill(int32x4 descriptor, const void* lds, uint32_t offset) {
   static_assert(BYTES == 16 || BYTES == 4);
