@@ -36,7 +36,10 @@ def case(oracle, dtype, rows, n_in, n_out, seed):
 # tiles, a width of 64 mod 128 on either side, and widths the matrix-core
 # kernels do not take (fully_connected.h:18: any positive width)
 SHAPES = [(128, 64, 64), (200, 128, 192), (77, 192, 64), (300, 64, 320), (1, 128, 128),
-          (5, 7, 3), (70, 65, 129), (33, 128, 66)]
+          (5, 7, 3), (70, 65, 129), (33, 128, 66),
+          # contractions of 1536 and more take the 256 x 256 tiles (forward:
+          # input_dim, input gradient: output_dim), here with ragged tiles
+          (300, 1536, 64), (260, 64, 1536)]
 
 
 @pytest.mark.parametrize("dtype", ["bf16", "f32"])
@@ -68,6 +71,36 @@ def test_forward_and_backward_match_oracle(capi, oracle, dtype, shape):
     assert_close(dx.cpu().numpy(), want_dx, 1e-5, "dx %s" % (shape,))
     assert_close(dw.cpu().numpy(), want_dw, 2e-5, "dw %s" % (shape,))
     assert_close(db.cpu().numpy(), want_db, 1e-5, "db %s" % (shape,))
+
+
+def test_bench_shape_matches_float64_products(capi, oracle):
+    """The GPT-2-small QKV projection at its full size (16384 rows, 768 ->
+    2304, bf16): every output against float64 matrix products of the same
+    rounded operands, computed by the library on the GPU; the weight gradient
+    there runs in four row slices and the bias gradient in 64 partitions."""
+    rows, n_in, n_out = 16384, 768, 2304
+    g = torch.Generator(device="cuda").manual_seed(7)
+    x = torch.randn(rows, n_in, device="cuda", generator=g).to(torch.bfloat16)
+    w = torch.randn(n_in, n_out, device="cuda", generator=g) / n_in ** 0.5
+    b = torch.randn(n_out, device="cuda", generator=g)
+    dy = torch.randn(rows, n_out, device="cuda", generator=g)
+    y = capi.dense_forward(x, w, b)
+    dx, dw, db = capi.dense_backward(x, w, dy)
+    x64 = x.double()
+    w64 = w.to(torch.bfloat16).double()
+    dy64 = dy.to(torch.bfloat16).double()
+    want_y = x64 @ w64 + b.double()
+    diff = (y.double() - want_y).abs()
+    assert bool((diff <= 2.0 ** -7 * want_y.abs() + 1e-6).all()), float(diff.max())
+
+    def close(got, want, tolerance, what):
+        error = float((got.double() - want).abs().max())
+        scale = float(want.abs().max())
+        assert error <= tolerance * scale, (what, error, scale)
+
+    close(dx, dy64 @ w64.t(), 1e-5, "dx")
+    close(dw, x64.t() @ dy64, 2e-5, "dw")
+    close(db, dy.double().sum(0), 1e-5, "db")
 
 
 def test_gradients_are_overwritten_and_repeatable(capi, oracle):
