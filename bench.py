@@ -35,8 +35,8 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E (published)
 # the factors a 1 GiB device copy gives: `--workload copy`).  The summaries are
 # kept as profiles/*_hbm_traffic.md.  None = not measured.
 MEASURED_TRAFFIC_BYTES = {
-    ("mha_train_bf16", "forward"): 127.1e6,
-    ("mha_train_bf16", "backward"): 509.0e6,
+    ("mha_train_bf16", "forward"): 126.4e6,
+    ("mha_train_bf16", "backward"): 548.6e6,
     ("gqa_prefill", "prefill"): 538.6e6,
     ("gqa_decode", "decode"): 1055.9e6,
     ("gdn_scan", "scan"): 2105.3e6,
