@@ -1139,3 +1139,86 @@ int pluto_oracle_dense_backward(int dtype, int rows, int input_dim, int output_d
   return 0;
 }
 
+
+/* ---- imported projection (fully_connected.cc:40-94,295-341) --------------- */
+
+float pluto_oracle_fp8_e4m3_to_f32(uint8_t bits) {
+  const int sign = bits >> 7, exponent = (bits >> 3) & 15, mantissa = bits & 7;
+  float magnitude;
+  if (exponent == 15 && mantissa == 7) return NAN;
+  if (exponent == 0)
+    magnitude = ldexpf((float)mantissa, -9); /* subnormal: m/8 * 2^-6 */
+  else
+    magnitude = ldexpf(1.0f + mantissa / 8.0f, exponent - 7);
+  return sign ? -magnitude : magnitude;
+}
+
+uint8_t pluto_oracle_f32_to_fp8_e4m3(float value) {
+  if (isnan(value)) return 0x7f;
+  const uint8_t sign = signbit(value) ? 0x80 : 0;
+  const double a = fabs((double)value);
+  if (a >= 448.0) return sign | 0x7e; /* saturate (also infinities) */
+  /* spacing of the format at a: 2^(e-3) with e = max(floor(log2 a), -6) */
+  int e;
+  frexp(a, &e); /* a = f * 2^e, f in [0.5, 1) -> floor(log2 a) = e - 1 */
+  int exponent = a == 0.0 ? -6 : e - 1;
+  if (exponent < -6) exponent = -6;
+  const double step = ldexp(1.0, exponent - 3);
+  /* nearbyint rounds halfway cases to even in the default rounding mode */
+  double steps = nearbyint(a / step);
+  double rounded = steps * step;
+  if (rounded >= 448.0 + 1e-9) return sign | 0x7e;
+  if (rounded == 0.0) return sign;
+  frexp(rounded, &e);
+  int re = e - 1;
+  if (re < -6) { /* subnormal: rounded = m * 2^-9 */
+    return sign | (uint8_t)(int)(rounded / ldexp(1.0, -9));
+  }
+  const int mantissa = (int)((rounded / ldexp(1.0, re) - 1.0) * 8.0 + 0.5);
+  return sign | (uint8_t)(((re + 7) << 3) | mantissa);
+}
+
+void pluto_oracle_imported_quantize(const float* x, int n, float* out) {
+  for (int g0 = 0; g0 < n; g0 += 128) {
+    const int g1 = g0 + 128 < n ? g0 + 128 : n;
+    float largest = 0.0f;
+    for (int i = g0; i < g1; ++i) largest = fmaxf(largest, fabsf(x[i]));
+    const float scale = largest / 448.0f;
+    const float divisor = fmaxf(scale, 1e-12f);
+    for (int i = g0; i < g1; ++i)
+      out[i] = pluto_oracle_fp8_e4m3_to_f32(pluto_oracle_f32_to_fp8_e4m3(x[i] / divisor)) * scale;
+  }
+}
+
+int pluto_oracle_imported_matvec(int storage, const void* weights, const float* scales,
+                                 const float* x, int input_dim, int output_dim, float* y) {
+  if (storage < PLUTO_ORACLE_MATRIX_BF16 || storage > PLUTO_ORACLE_MATRIX_FP8_E4M3 ||
+      input_dim <= 0 || output_dim <= 0 || !weights || !x || !y)
+    return -1;
+  if ((storage == PLUTO_ORACLE_MATRIX_FP8_E4M3) != (scales != NULL)) return -1;
+  float* token = (float*)malloc(sizeof(float) * (size_t)input_dim);
+  if (!token) return -2;
+  if (storage == PLUTO_ORACLE_MATRIX_FP8_E4M3)
+    pluto_oracle_imported_quantize(x, input_dim, token);
+  else
+    memcpy(token, x, sizeof(float) * (size_t)input_dim);
+  const int scale_cols = (input_dim + 127) / 128;
+  for (int r = 0; r < output_dim; ++r) {
+    double sum = 0.0;
+    for (int c = 0; c < input_dim; ++c) {
+      const size_t i = (size_t)r * input_dim + c;
+      float w;
+      if (storage == PLUTO_ORACLE_MATRIX_BF16)
+        w = pluto_oracle_bf16_to_f32(((const uint16_t*)weights)[i]);
+      else if (storage == PLUTO_ORACLE_MATRIX_F32)
+        w = ((const float*)weights)[i];
+      else
+        w = pluto_oracle_fp8_e4m3_to_f32(((const uint8_t*)weights)[i]) *
+            scales[(size_t)(r / 128) * scale_cols + c / 128];
+      sum += (double)w * token[c];
+    }
+    y[r] = pluto_oracle_bf16_round((float)sum);
+  }
+  free(token);
+  return 0;
+}

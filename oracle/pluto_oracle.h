@@ -234,6 +234,27 @@ int pluto_oracle_dense_backward(int dtype, int rows, int input_dim, int output_d
                                 const float* x, const float* matrix, const float* dy,
                                 float* dx, float* d_matrix, float* d_bias);
 
+/* Imported (frozen, output-major) projection of FullyConnectedLayer
+ * (src/llm/layers/fully_connected.cc:40-94,295-341): one bf16 token
+ * [input_dim] against weights [output_dim, input_dim] stored as bf16, fp32 or
+ * FP8 E4M3 with FP32 scales [ceil(out/128), ceil(in/128)]; all arithmetic in
+ * FP32 (here: double sums, as the scalar projection of
+ * fully_connected_imported_test.cc:190-205), output rounded to bf16. */
+#define PLUTO_ORACLE_MATRIX_BF16 0
+#define PLUTO_ORACLE_MATRIX_F32 1
+#define PLUTO_ORACLE_MATRIX_FP8_E4M3 2
+/* OCP FP8 E4M3 (no infinities, 0x7f/0xff NaN, largest finite 448). */
+float pluto_oracle_fp8_e4m3_to_f32(uint8_t bits);
+/* Round to nearest even, saturating to +-448; NaN -> 0x7f. */
+uint8_t pluto_oracle_f32_to_fp8_e4m3(float value);
+/* QuantizeImportedInputKernel (fully_connected.cc:70-88): per group of 128
+ * elements scale = max|x| / 448, out = fp8(x / max(scale, 1e-12)) * scale. */
+void pluto_oracle_imported_quantize(const float* x, int n, float* out);
+/* x: the token as floats (bf16 values); FP8 storage quantizes it first.
+ * y: output_dim floats holding bf16 values. */
+int pluto_oracle_imported_matvec(int storage, const void* weights, const float* scales,
+                                 const float* x, int input_dim, int output_dim, float* y);
+
 #ifdef __cplusplus
 }
 #endif

@@ -390,3 +390,51 @@ def dense_backward(dtype, x, matrix, dy):
           _ptr(db)) != 0:
         raise ValueError("oracle rejected the dense backward")
     return dx, dw, db
+
+
+MATRIX_BF16, MATRIX_F32, MATRIX_FP8_E4M3 = 0, 1, 2
+
+
+def fp8_e4m3_to_f32(bits):
+    """Values of OCP FP8 E4M3 codes (uint8 array)."""
+    bits = np.ascontiguousarray(bits, np.uint8)
+    fn = lib().pluto_oracle_fp8_e4m3_to_f32
+    fn.restype = ctypes.c_float
+    fn.argtypes = [ctypes.c_uint8]
+    return np.array([fn(int(b)) for b in bits.ravel()], np.float32).reshape(bits.shape)
+
+
+def f32_to_fp8_e4m3(values):
+    """FP8 E4M3 codes of floats: nearest even, saturating to +-448."""
+    values = _f32(values)
+    fn = lib().pluto_oracle_f32_to_fp8_e4m3
+    fn.restype = ctypes.c_uint8
+    fn.argtypes = [ctypes.c_float]
+    return np.array([fn(float(v)) for v in values.ravel()], np.uint8).reshape(values.shape)
+
+
+def imported_quantize(x):
+    """Dynamic FP8 quantization of a token in groups of 128 (fully_connected.cc:70-88)."""
+    x = _f32(x)
+    out = np.zeros_like(x)
+    fn = lib().pluto_oracle_imported_quantize
+    fn.restype = None
+    fn(_ptr(x), ctypes.c_int(x.size), _ptr(out))
+    return out
+
+
+def imported_matvec(storage, weights, scales, x):
+    """Frozen output-major projection of one bf16 token: weights [out, in] as
+    uint16 bf16 bits, float32 or uint8 FP8 codes (+ float32 block scales)."""
+    weights = np.ascontiguousarray(weights)
+    output_dim, input_dim = weights.shape
+    x = _f32(x)
+    y = np.zeros(output_dim, np.float32)
+    fn = lib().pluto_oracle_imported_matvec
+    fn.restype = ctypes.c_int
+    s = None if scales is None else _f32(scales)
+    if fn(ctypes.c_int(storage), weights.ctypes.data_as(ctypes.c_void_p),
+          None if s is None else _ptr(s), _ptr(x), ctypes.c_int(input_dim),
+          ctypes.c_int(output_dim), _ptr(y)) != 0:
+        raise ValueError("oracle rejected the imported projection")
+    return y
