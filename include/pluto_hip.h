@@ -442,6 +442,28 @@ int pluto_hip_dense_backward(void* stream, int dtype, const void* input,
                              float* d_input, float* d_matrix, float* d_bias,
                              void* workspace, size_t workspace_bytes);
 
+/* FullyConnectedLayer, imported path (src/llm/layers/fully_connected.cc:
+ * ImportedMatVecKernel :40-68, QuantizeImportedInputKernel :70-88, Create
+ * :267-293, ImportedForward :295-341; storage enum matrix_common.h:10): a
+ * frozen checkpoint matrix, output-major [output_dim, input_dim], stored as
+ * bf16, fp32 or OCP FP8 E4M3 with FP32 block scales
+ * [ceil(output_dim/128), ceil(input_dim/128)], times ONE bf16 token
+ * [input_dim] -> bf16 [output_dim].  All arithmetic is FP32.  With FP8 weights
+ * the token is quantized first, in independent groups of 128 elements:
+ * scale = max|x| / 448, x -> fp8(x / max(scale, 1e-12)) * scale.  `scales`
+ * must be non-NULL exactly for FP8 storage; dimensions in [1, 1048576] (:271).
+ * workspace: pluto_hip_dense_imported_workspace_bytes(input_dim) bytes. */
+#define PLUTO_HIP_MATRIX_BF16 0
+#define PLUTO_HIP_MATRIX_F32 1
+#define PLUTO_HIP_MATRIX_FP8_E4M3 2
+#define PLUTO_HIP_IMPORTED_MAX_DIM 1048576
+size_t pluto_hip_dense_imported_workspace_bytes(int input_dim);
+int pluto_hip_dense_imported_forward(void* stream, int storage,
+                                     const void* weights, const float* scales,
+                                     const void* input, int input_dim,
+                                     int output_dim, void* output,
+                                     void* workspace, size_t workspace_bytes);
+
 #ifdef __cplusplus
 }
 #endif

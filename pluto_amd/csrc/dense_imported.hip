@@ -1,0 +1,198 @@
+// FullyConnectedLayer, imported path (src/llm/layers/fully_connected.cc):
+//   ImportedMatVecKernel          :40-68   y = bf16(W x), W output-major
+//   QuantizeImportedInputKernel   :70-88   FP8 storage: x -> fp8(x / s) * s in
+//                                          groups of 128, s = max|x| / 448
+//   ImportedForward               :295-341 bf16 token -> fp32 -> (quantize) ->
+//                                          mat-vec -> bf16
+// One frozen checkpoint matrix [output_dim, input_dim] in bf16, fp32 or OCP
+// FP8 E4M3 with FP32 scales [ceil(out/128), ceil(in/128)] times one bf16
+// token.  Byte-bound: every weight is read once.  A wave owns an output row
+// and reads it in 16-byte pieces (whenever rows start 16-byte aligned), the
+// token comes from the FP32 copy the first kernel leaves in the workspace;
+// all arithmetic is FP32, the 64 lane sums are added by a butterfly.
+#include "dense.h"
+
+namespace pluto_hip {
+namespace {
+
+constexpr int kGroup = 128;  // quantization group and scale block edge
+
+// Value of an OCP FP8 E4M3 code: 1-4-3 bits, bias 7, no infinities, S.1111.111
+// is NaN, subnormals m * 2^-9.
+__device__ inline float fp8_value(uint32_t bits) {
+  const uint32_t exponent = (bits >> 3) & 15u, mantissa = bits & 7u;
+  float magnitude;
+  if (exponent == 0)
+    magnitude = static_cast<float>(mantissa) * 0.001953125f;
+  else if (exponent == 15 && mantissa == 7)
+    magnitude = __builtin_nanf("");
+  else
+    magnitude = __uint_as_float(((exponent + 120u) << 23) | (mantissa << 20));
+  return (bits & 0x80u) ? -magnitude : magnitude;
+}
+
+// The FP8 E4M3 value nearest to v (ties to even, saturating at +-448), as a
+// float: what element_cast to FP8 and back gives (fully_connected.cc:86-87).
+__device__ inline float fp8_round(float v) {
+  const float a = fabsf(v);
+  if (a >= 448.0f) return copysignf(448.0f, v);
+  int exponent = static_cast<int>((__float_as_uint(a) >> 23) & 255u) - 127;  // floor(log2 a)
+  if (exponent < -6) exponent = -6;                                          // subnormal grid
+  const float step = __uint_as_float(static_cast<uint32_t>(exponent - 3 + 127) << 23);
+  const float rounded = __builtin_rintf(a / step) * step;  // a / step is exact
+  return copysignf(fminf(rounded, 448.0f), v);
+}
+
+// token[i] = float(x[i]), for FP8 storage quantized per group of 128.
+template <bool FP8>
+__global__ void __launch_bounds__(kGroup)
+imported_token_kernel(const uint16_t* x, int n, float* token) {
+  __shared__ float largest[2];
+  const int i = blockIdx.x * kGroup + threadIdx.x;
+  const float v = i < n ? bf16_bits_to_float(x[i]) : 0.0f;
+  if constexpr (!FP8) {
+    if (i < n) token[i] = v;
+  } else {
+    const float mine = wave_max(fabsf(v));
+    if (threadIdx.x % 64 == 0) largest[threadIdx.x / 64] = mine;
+    __syncthreads();
+    const float scale = fmaxf(largest[0], largest[1]) / 448.0f;
+    // only the divisor is floored: the result keeps the group's own scale
+    if (i < n) token[i] = fp8_round(v / fmaxf(scale, 1e-12f)) * scale;
+  }
+}
+
+struct MatVecArgs {
+  const void* weights = nullptr;
+  const float* scales = nullptr;  // FP8 only
+  const float* token = nullptr;
+  uint16_t* out = nullptr;
+  int cols = 0, rows = 0;
+};
+
+// STORAGE: 0 bf16, 1 fp32, 2 FP8 E4M3.  One wave per output row.
+template <int STORAGE>
+__global__ void __launch_bounds__(256) imported_matvec_kernel(MatVecArgs a) {
+  constexpr int kElementBytes = STORAGE == 0 ? 2 : (STORAGE == 1 ? 4 : 1);
+  constexpr int kPiece = 16 / kElementBytes;  // elements per 16-byte load
+  const int lane = threadIdx.x % 64;
+  const int row = blockIdx.x * 4 + threadIdx.x / 64;
+  if (row >= a.rows) return;
+  const size_t row_start = static_cast<size_t>(row) * a.cols;
+  const int scale_cols = (a.cols + kGroup - 1) / kGroup;
+  const float* scale_row =
+      STORAGE == 2 ? a.scales + static_cast<size_t>(row / kGroup) * scale_cols : nullptr;
+  float sum = 0.0f;
+  auto element = [&](int c) {
+    const size_t i = row_start + c;
+    if constexpr (STORAGE == 0)
+      return bf16_bits_to_float(static_cast<const uint16_t*>(a.weights)[i]);
+    else if constexpr (STORAGE == 1)
+      return static_cast<const float*>(a.weights)[i];
+    else
+      return fp8_value(static_cast<const uint8_t*>(a.weights)[i]) * scale_row[c / kGroup];
+  };
+  int done = 0;
+  if ((static_cast<size_t>(a.cols) * kElementBytes) % 16 == 0) {
+    // every row starts on a 16-byte boundary (the buffer itself is at least
+    // 256-byte aligned): whole pieces, a piece never straddles a scale block
+    const unsigned char* base =
+        static_cast<const unsigned char*>(a.weights) + row_start * kElementBytes;
+    const int pieces = a.cols / kPiece;
+    for (int p = lane; p < pieces; p += 64) {
+      const uint4 raw = *reinterpret_cast<const uint4*>(base + static_cast<size_t>(p) * 16);
+      const uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
+      const int c0 = p * kPiece;
+      if constexpr (STORAGE == 0) {
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          sum += __uint_as_float(words[w] << 16) * a.token[c0 + 2 * w];
+          sum += __uint_as_float(words[w] & 0xffff0000u) * a.token[c0 + 2 * w + 1];
+        }
+      } else if constexpr (STORAGE == 1) {
+#pragma unroll
+        for (int w = 0; w < 4; ++w) sum += __uint_as_float(words[w]) * a.token[c0 + w];
+      } else {
+        const float scale = scale_row[c0 / kGroup];
+        float part = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w)
+#pragma unroll
+          for (int b = 0; b < 4; ++b)
+            part += fp8_value((words[w] >> (8 * b)) & 0xffu) * a.token[c0 + 4 * w + b];
+        sum += part * scale;
+      }
+    }
+    done = pieces * kPiece;
+  }
+  for (int c = done + lane; c < a.cols; c += 64) sum += element(c) * a.token[c];
+  sum = wave_sum(sum);
+  if (lane == 0) a.out[row] = float_to_bf16_bits(sum);
+}
+
+}  // namespace
+
+size_t dense_imported_workspace_bytes(int input_dim) {
+  return align_up(static_cast<size_t>(input_dim) * sizeof(float), 256);
+}
+
+int launch_dense_imported_forward(hipStream_t s, int storage, const void* weights,
+                                  const float* scales, const void* input, int input_dim,
+                                  int output_dim, void* output, void* workspace) {
+  float* token = static_cast<float*>(workspace);
+  const unsigned groups = static_cast<unsigned>((input_dim + kGroup - 1) / kGroup);
+  if (storage == PLUTO_HIP_MATRIX_FP8_E4M3)
+    imported_token_kernel<true><<<groups, kGroup, 0, s>>>(static_cast<const uint16_t*>(input),
+                                                          input_dim, token);
+  else
+    imported_token_kernel<false><<<groups, kGroup, 0, s>>>(static_cast<const uint16_t*>(input),
+                                                           input_dim, token);
+  MatVecArgs a;
+  a.weights = weights;
+  a.scales = scales;
+  a.token = token;
+  a.out = static_cast<uint16_t*>(output);
+  a.cols = input_dim;
+  a.rows = output_dim;
+  const unsigned blocks = static_cast<unsigned>((output_dim + 3) / 4);
+  if (storage == PLUTO_HIP_MATRIX_BF16)
+    imported_matvec_kernel<0><<<blocks, 256, 0, s>>>(a);
+  else if (storage == PLUTO_HIP_MATRIX_F32)
+    imported_matvec_kernel<1><<<blocks, 256, 0, s>>>(a);
+  else
+    imported_matvec_kernel<2><<<blocks, 256, 0, s>>>(a);
+  return launch_status();
+}
+
+}  // namespace pluto_hip
+
+using namespace pluto_hip;
+
+extern "C" {
+
+size_t pluto_hip_dense_imported_workspace_bytes(int input_dim) {
+  if (input_dim <= 0 || input_dim > PLUTO_HIP_IMPORTED_MAX_DIM) return 0;
+  return dense_imported_workspace_bytes(input_dim);
+}
+
+int pluto_hip_dense_imported_forward(void* stream, int storage, const void* weights,
+                                     const float* scales, const void* input, int input_dim,
+                                     int output_dim, void* output, void* workspace,
+                                     size_t workspace_bytes) {
+  if (storage != PLUTO_HIP_MATRIX_BF16 && storage != PLUTO_HIP_MATRIX_F32 &&
+      storage != PLUTO_HIP_MATRIX_FP8_E4M3)
+    return PLUTO_HIP_EINVAL;
+  // fully_connected.cc:271-275: dimensions in [1, 1048576]
+  if (input_dim <= 0 || input_dim > PLUTO_HIP_IMPORTED_MAX_DIM || output_dim <= 0 ||
+      output_dim > PLUTO_HIP_IMPORTED_MAX_DIM)
+    return PLUTO_HIP_EINVAL;
+  // :279-281: only FP8 weights have block scales
+  if ((storage == PLUTO_HIP_MATRIX_FP8_E4M3) != (scales != nullptr)) return PLUTO_HIP_EINVAL;
+  if (!weights || !input || !output) return PLUTO_HIP_EINVAL;
+  if (!workspace || workspace_bytes < dense_imported_workspace_bytes(input_dim))
+    return PLUTO_HIP_EWORKSPACE;
+  return launch_dense_imported_forward(static_cast<hipStream_t>(stream), storage, weights, scales,
+                                       input, input_dim, output_dim, output, workspace);
+}
+
+}  // extern "C"

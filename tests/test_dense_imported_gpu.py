@@ -1,0 +1,119 @@
+"""GPU parity of the imported FullyConnectedLayer projection
+(fully_connected.cc:40-94,295-341) with the CPU oracle, through the C ABI; the
+cases are those of fully_connected_imported_test.cc."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+
+@pytest.fixture(scope="module")
+def capi():
+    from pluto_amd import capi
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    capi.lib()
+    return capi
+
+
+def bf16_tensor(oracle, values):
+    return torch.from_numpy(oracle.bf16_round(np.float32(values))).cuda().to(torch.bfloat16)
+
+
+def run(capi, oracle, storage, source, scales, x):
+    """(library result, oracle result) for weights given as float values."""
+    if storage == oracle.MATRIX_F32:
+        host = np.float32(source)
+        device = torch.from_numpy(host).cuda()
+    elif storage == oracle.MATRIX_BF16:
+        rounded = oracle.bf16_round(np.float32(source))
+        host = (rounded.view(np.uint32) >> 16).astype(np.uint16)
+        device = torch.from_numpy(rounded).cuda().to(torch.bfloat16)
+    else:
+        host = oracle.f32_to_fp8_e4m3(np.float32(source))
+        device = torch.from_numpy(host).cuda()
+    s_host = None if scales is None else np.float32(scales)
+    s_device = None if scales is None else torch.from_numpy(s_host).cuda()
+    token = oracle.bf16_round(np.float32(x))
+    got = capi.dense_imported_forward(storage, device, s_device, bf16_tensor(oracle, token))
+    torch.cuda.synchronize()
+    want = oracle.imported_matvec(storage, host, s_host, token)
+    return got.float().cpu().numpy(), want
+
+
+def test_smallest_case_for_every_storage(capi, oracle):
+    # fully_connected_imported_test.cc:93-136
+    w = [[1, 2, 3], [4, 5, 6]]
+    for storage, scales in ((oracle.MATRIX_F32, None), (oracle.MATRIX_BF16, None),
+                            (oracle.MATRIX_FP8_E4M3, [1.0])):
+        got, want = run(capi, oracle, storage, w, scales, [1, 0, -1])
+        assert list(got) == [-2, -2] and list(want) == [-2, -2]
+
+
+@pytest.mark.parametrize("cols,rows", [(263, 259), (5120, 131), (1024, 1000), (130, 9)])
+def test_block_scales_tails_and_real_width(capi, oracle, cols, rows):
+    # fully_connected_imported_test.cc:143-211: straddles the row tiles and the
+    # 128 x 128 scale blocks, includes the checkpoint's 5120-wide input; rows
+    # that start 16-byte aligned (vector loads) and rows that do not
+    i = np.arange(cols * rows)
+    source = (1.9 * np.sin((i % 1009).astype(np.float32) * np.float32(0.037))).reshape(rows, cols)
+    x = (np.cos(np.arange(cols) * 0.123) * 0.25).astype(np.float32)
+    scale_cols, scale_rows = (cols + 127) // 128, (rows + 127) // 128
+    scales = [[(r + 1) * (c + 1) * 0.03125 for c in range(scale_cols)] for r in range(scale_rows)]
+    for storage, s in ((oracle.MATRIX_F32, None), (oracle.MATRIX_BF16, None),
+                       (oracle.MATRIX_FP8_E4M3, scales)):
+        got, want = run(capi, oracle, storage, source, s, x)
+        # the reference's own bound for this test (:206), FP32 against double sums
+        assert np.all(np.abs(got - want) <= 5e-5 + 0.008 * np.abs(want)), storage
+        # and nearly every output is the same bf16 value
+        assert np.mean(got != want) <= 0.05, storage
+
+
+def test_dynamic_quantization_zero_tiny_ties_and_tail(capi, oracle):
+    # fully_connected_imported_test.cc:213-253: an identity matrix exposes every
+    # quantized input
+    width = 389
+    x = np.zeros(width, np.float32)
+    for i in range(128, 256):
+        x[i] = ((i % 31) - 15) * 0.0625
+    x[128], x[129], x[130], x[131] = 448, -448, 1.0625, 1.1875
+    for i in range(256, 384):
+        x[i] = (i % 5 - 2) * 1e-14
+    for i in range(384, width):
+        x[i] = (i - 386) * 25.3
+    x = oracle.bf16_round(x)
+    got, want = run(capi, oracle, oracle.MATRIX_FP8_E4M3, np.eye(width, dtype=np.float32),
+                    np.ones((4, 4), np.float32), x)
+    expected = oracle.bf16_round(oracle.imported_quantize(x))
+    assert np.array_equal(want, expected)
+    assert np.array_equal(got, expected)   # one product per row: no summation-order slack
+    assert got[130] == 1.0 and got[131] == 1.25
+    assert np.all(got[:128] == 0) and got[128] == 448 and got[129] == -448
+    assert np.abs(got[256:384]).max() > 0
+
+
+def test_rejects_bad_arguments(capi):
+    lib = capi.lib()
+    w = torch.zeros(6, dtype=torch.float32, device="cuda")
+    x = torch.zeros(3, dtype=torch.bfloat16, device="cuda")
+    y = torch.zeros(2, dtype=torch.bfloat16, device="cuda")
+    ws = torch.zeros(4096, dtype=torch.uint8, device="cuda")
+    s = torch.ones(1, dtype=torch.float32, device="cuda")
+    stream = capi.current_stream()
+
+    def call(storage=capi.MATRIX_F32, scales=None, cols=3, rows=2, workspace_bytes=4096):
+        return lib.pluto_hip_dense_imported_forward(
+            stream, storage, capi.ptr(w), None if scales is None else capi.ptr(scales),
+            capi.ptr(x), cols, rows, capi.ptr(y), capi.ptr(ws), workspace_bytes)
+
+    assert call() == 0
+    assert call(storage=7) == capi.EINVAL
+    assert call(scales=s) == capi.EINVAL                       # scales without FP8 weights
+    assert call(storage=capi.MATRIX_FP8_E4M3) == capi.EINVAL   # FP8 weights without scales
+    assert call(cols=0) == capi.EINVAL and call(rows=-1) == capi.EINVAL
+    assert call(cols=1048577) == capi.EINVAL
+    assert call(workspace_bytes=4) == capi.EWORKSPACE
+    assert lib.pluto_hip_dense_imported_workspace_bytes(0) == 0
+    assert lib.pluto_hip_dense_imported_workspace_bytes(3) >= 12
+    torch.cuda.synchronize()
