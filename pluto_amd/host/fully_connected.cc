@@ -16,7 +16,80 @@ Status ValidatePositiveExtent(int extent, const char* name) {
   return OkStatus();
 }
 
+int StorageCode(MatrixStorage storage) {
+  switch (storage) {
+    case MatrixStorage::kBFloat16: return PLUTO_HIP_MATRIX_BF16;
+    case MatrixStorage::kFloat32: return PLUTO_HIP_MATRIX_F32;
+    case MatrixStorage::kFp8E4M3: return PLUTO_HIP_MATRIX_FP8_E4M3;
+  }
+  return -1;
+}
+
 }  // namespace
+
+// src/llm/layers/matrix_common.cc
+StatusOr<size_t> MatrixElementBytes(MatrixStorage storage) {
+  switch (storage) {
+    case MatrixStorage::kBFloat16: return size_t{2};
+    case MatrixStorage::kFloat32: return size_t{4};
+    case MatrixStorage::kFp8E4M3: return size_t{1};
+  }
+  return InvalidArgumentError("unknown matrix storage");
+}
+
+FullyConnectedLayer::FullyConnectedLayer(hip::Executor& executor, int input_dim, int output_dim,
+                                         BufferVec weights, MatrixStorage storage)
+    : executor_(executor), input_dim_(input_dim), output_dim_(output_dim),
+      output_type_(DataType::BF16), weights_(std::move(weights)), imported_storage_(storage) {
+  input_types_.emplace_back(DataType::BF16, std::vector<int64_t>{1, 1, 1LL * input_dim});
+  output_types_.emplace_back(DataType::BF16, std::vector<int64_t>{1, 1, 1LL * output_dim});
+}
+
+// src/llm/layers/fully_connected.cc:267-293
+StatusOr<std::unique_ptr<FullyConnectedLayer>> FullyConnectedLayer::Create(
+    hip::Executor& executor, Buffer weights, MatrixStorage storage, int input_dim, int output_dim,
+    std::optional<Buffer> scales) {
+  if (input_dim <= 0 || input_dim > kMaximumDimension || output_dim <= 0 ||
+      output_dim > kMaximumDimension)
+    return InvalidArgumentError("imported linear dimensions must be in [1, 1048576]");
+  ASSIGN_OR_RETURN(size_t element_bytes, MatrixElementBytes(storage));
+  RETURN_IF_ERROR(internal::ValidateBuffer(
+      executor, weights, static_cast<size_t>(input_dim) * output_dim * element_bytes,
+      "imported linear weights"));
+  if ((storage == MatrixStorage::kFp8E4M3) != scales.has_value())
+    return InvalidArgumentError("only FP8 linear weights require block scales");
+  BufferVec buffers{std::move(weights)};
+  if (scales) {
+    RETURN_IF_ERROR(internal::ValidateBuffer(
+        executor, *scales,
+        static_cast<size_t>((input_dim + 127) / 128) * ((output_dim + 127) / 128) * sizeof(float),
+        "imported linear block scales"));
+    buffers.push_back(std::move(*scales));
+  }
+  return std::unique_ptr<FullyConnectedLayer>(
+      new FullyConnectedLayer(executor, input_dim, output_dim, std::move(buffers), storage));
+}
+
+// src/llm/layers/fully_connected.cc:295-341; the cast of the token to FP32 and
+// its FP8 quantization happen inside the library call.
+StatusOr<FwdResult> FullyConnectedLayer::ImportedForward(hip::Executor& executor,
+                                                         Span<const Buffer> inputs) const {
+  const int counts[] = {input_dim_};
+  RETURN_IF_ERROR(internal::ValidateBFloat16Inputs(executor, inputs, counts));
+  ASSIGN_OR_RETURN(Buffer output,
+                   Buffer::Allocate(executor, static_cast<size_t>(output_dim_) * 2));
+  const size_t workspace_bytes = pluto_hip_dense_imported_workspace_bytes(input_dim_);
+  ASSIGN_OR_RETURN(Buffer workspace, Buffer::Allocate(executor, workspace_bytes));
+  const float* scales =
+      weights_.size() == 2 ? static_cast<const float*>(weights_[1].data()) : nullptr;
+  RETURN_IF_ERROR(hip::HipStatus(
+      pluto_hip_dense_imported_forward(executor.stream(), StorageCode(*imported_storage_),
+                                       weights_[0].data(), scales, inputs[0].data(), input_dim_,
+                                       output_dim_, output.data(), workspace.data(),
+                                       workspace_bytes),
+      "imported projection launch"));
+  return FwdResult{{std::move(output)}, {}};
+}
 
 FullyConnectedLayer::FullyConnectedLayer(hip::Executor& executor, int input_dim, int output_dim,
                                          DataType data_type, BufferVec weights, BufferVec gradients,
@@ -55,6 +128,8 @@ StatusOr<std::unique_ptr<FullyConnectedLayer>> FullyConnectedLayer::Create(
 
 // src/llm/layers/fully_connected.cc:372-389
 Status FullyConnectedLayer::InitializeIdentity(float scale) {
+  if (imported_storage_)
+    return FailedPreconditionError("cannot initialize frozen imported linear weights");
   ASSIGN_OR_RETURN(auto matrix, hip::PageLockedHostArray<float>::Allocate(
                                     executor_, static_cast<size_t>(input_dim_) * output_dim_));
   std::fill(matrix.begin(), matrix.end(), 0.0f);
@@ -68,6 +143,8 @@ Status FullyConnectedLayer::InitializeIdentity(float scale) {
 
 // src/llm/layers/fully_connected.cc:391-413
 Status FullyConnectedLayer::InitializeNormal(float standard_deviation, uint64_t seed) {
+  if (imported_storage_)
+    return FailedPreconditionError("cannot initialize frozen imported linear weights");
   if (!(standard_deviation > 0.0f))
     return InvalidArgumentError("dense initialization standard deviation must be positive");
   std::mt19937_64 random(seed);
@@ -84,6 +161,7 @@ Status FullyConnectedLayer::InitializeNormal(float standard_deviation, uint64_t 
 StatusOr<FwdResult> FullyConnectedLayer::fwd_impl(hip::Executor& executor,
                                                   Span<const Buffer> inputs, LayerHooks*) const {
   RETURN_IF_ERROR(internal::ValidateExecutor(executor_, executor, "FullyConnectedLayer"));
+  if (imported_storage_) return ImportedForward(executor, inputs);
   if (inputs.size() != 1) return InvalidArgumentError("FullyConnectedLayer fwd expects one input");
   ASSIGN_OR_RETURN(int rows, internal::ActivationRows(executor, inputs[0], input_dim_,
                                                       output_type_, "dense input"));
@@ -110,6 +188,8 @@ StatusOr<BufferVec> FullyConnectedLayer::bwd_impl(hip::Executor& executor,
                                                   Span<const Buffer> output_gradients,
                                                   BackwardState state, LayerHooks*) {
   RETURN_IF_ERROR(internal::ValidateExecutor(executor_, executor, "FullyConnectedLayer"));
+  if (imported_storage_)
+    return UnimplementedError("imported linear weights do not support backward");
   if (output_gradients.size() != 1 || state.intermediates.size() != 1)
     return InvalidArgumentError(
         "FullyConnectedLayer bwd received an incompatible gradient or state");

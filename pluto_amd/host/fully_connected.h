@@ -1,19 +1,30 @@
-// A rectangular projection with a bias, FP32 master parameters and FP32
-// gradients: the trainable FullyConnectedLayer of
-// src/llm/layers/fully_connected.h:20-112 on MI355X.  Operands are multiplied
-// as bfloat16 (BF16 policy) or IEEE half (FP16 policy, FP32 activations) and
-// summed in FP32; widths need not be multiples of the compute tiles.  Each
-// backward call overwrites the matrix and bias gradients, and reductions run
-// in a fixed order, so repeated calls are bitwise stable.  The frozen imported
-// single-token path (fully_connected.h:38-46) is not part of this library.
+// A rectangular projection: FullyConnectedLayer of
+// src/llm/layers/fully_connected.h:20-112 on MI355X.
+// Trainable projections have a bias, FP32 master parameters and FP32
+// gradients.  Operands are multiplied as bfloat16 (BF16 policy) or IEEE half
+// (FP16 policy, FP32 activations) and summed in FP32; widths need not be
+// multiples of the compute tiles.  Each backward call overwrites the matrix
+// and bias gradients, and reductions run in a fixed order, so repeated calls
+// are bitwise stable.
+// Imported projections share frozen, biasless, output-major checkpoint
+// weights without copying them, take and give one BF16 token [1, 1, width],
+// compute in FP32, and have no gradients: initialization is a failed
+// precondition and backward is unimplemented.
 #pragma once
 
 #include <cstdint>
 #include <memory>
+#include <optional>
 
 #include "pluto_amd/host/layer.h"
 
 namespace pluto::llm {
+
+// Physical storage of an imported checkpoint matrix
+// (src/llm/layers/matrix_common.h:10).  FP8 matrices come with FP32 block
+// scales [ceil(output_dim/128), ceil(input_dim/128)].
+enum class MatrixStorage { kBFloat16, kFloat32, kFp8E4M3 };
+StatusOr<size_t> MatrixElementBytes(MatrixStorage storage);
 
 class FullyConnectedLayer final : public Layer {
  public:
@@ -30,6 +41,15 @@ class FullyConnectedLayer final : public Layer {
                                                                int sequence_length = 1) {
     return Create(executor, model_width, model_width, data_type, sequence_length);
   }
+
+  // Imports a biasless [output_dim, input_dim] matrix without copying it.  The
+  // FP8 path quantizes its input in independent groups of 128 elements.
+  static StatusOr<std::unique_ptr<FullyConnectedLayer>> Create(
+      hip::Executor& executor, Buffer weights, MatrixStorage storage, int input_dim,
+      int output_dim, std::optional<Buffer> scales = std::nullopt);
+
+  // Bound of the imported single-token kernels; not a trainable-layer limit.
+  static constexpr int kMaximumDimension = 1048576;
 
   // A scaled identity on the available diagonal; the bias is left as it is.
   Status InitializeIdentity(float scale = 1.0f);
@@ -49,6 +69,9 @@ class FullyConnectedLayer final : public Layer {
  private:
   FullyConnectedLayer(hip::Executor& executor, int input_dim, int output_dim, DataType data_type,
                       BufferVec weights, BufferVec gradients, int sequence_length);
+  FullyConnectedLayer(hip::Executor& executor, int input_dim, int output_dim, BufferVec weights,
+                      MatrixStorage storage);
+  StatusOr<FwdResult> ImportedForward(hip::Executor& executor, Span<const Buffer> inputs) const;
   StatusOr<FwdResult> fwd_impl(hip::Executor& executor, Span<const Buffer> inputs,
                                LayerHooks* hooks) const override;
   StatusOr<BufferVec> bwd_impl(hip::Executor& executor, Span<const Buffer> output_gradients,
@@ -58,6 +81,8 @@ class FullyConnectedLayer final : public Layer {
   int input_dim_, output_dim_;
   DataType output_type_;
   BufferVec weights_, gradients_;
+  // Engaged only for the frozen output-major checkpoint representation.
+  std::optional<MatrixStorage> imported_storage_;
   std::vector<ActivationType> input_types_, output_types_;
 };
 

@@ -53,6 +53,7 @@ inline Status FailedPreconditionError(std::string m) { return {StatusCode::kFail
 inline bool IsInvalidArgument(const Status& s) { return s.code() == StatusCode::kInvalidArgument; }
 inline bool IsResourceExhausted(const Status& s) { return s.code() == StatusCode::kResourceExhausted; }
 inline bool IsUnimplemented(const Status& s) { return s.code() == StatusCode::kUnimplemented; }
+inline bool IsFailedPrecondition(const Status& s) { return s.code() == StatusCode::kFailedPrecondition; }
 
 inline const char* StatusCodeName(StatusCode code) {
   switch (code) {
