@@ -46,7 +46,7 @@ NAMES = ["mha_train_bf16", "mha_fwd_fp32", "gqa_prefill", "gqa_decode", "gdn_sca
 # "copy" is a plain device copy of known size: the calibration case for the
 # FETCH_SIZE / WRITE_SIZE counters that `roofline.traffic` is derived from.
 # "gqa_prefill_bwd" and "gdn_layer_bwd" time the two sequence backward passes.
-EXTRA = ["copy", "gqa_prefill_bwd", "gdn_layer_bwd", "gdn_decode", "dense_qkv"]
+EXTRA = ["copy", "gqa_prefill_bwd", "gdn_layer_bwd", "gdn_decode", "dense_qkv", "dense_imported"]
 
 
 def parse_args():
@@ -355,6 +355,34 @@ def dense_qkv(torch, capi):
                 cpu=None)
 
 
+def dense_imported(torch, capi):
+    """A frozen FP8 checkpoint projection at decode time (qwen/model.cc:192-227
+    builds its projections from imported FullyConnectedLayers): one bf16 token
+    of the checkpoint's 5120-wide residual stream times a [12288, 5120] FP8
+    E4M3 matrix with 128 x 128 block scales.  Byte-bound: every weight is read
+    once.  A row after the headline ones, not part of --workload all."""
+    n_in, n_out = 5120, 12288
+    gen = torch.Generator(device="cuda").manual_seed(8)
+    weights = torch.randint(0, 0x7e, (n_out, n_in), generator=gen, device="cuda", dtype=torch.uint8)
+    scales = torch.rand(((n_out + 127) // 128, (n_in + 127) // 128), generator=gen,
+                        device="cuda") * 0.01
+    x = torch.randn(n_in, generator=gen, device="cuda").to(torch.bfloat16)
+
+    workspace = capi.dense_imported_workspace(n_in, x.device)
+    out = torch.empty(n_out, dtype=torch.bfloat16, device="cuda")
+
+    def step():
+        capi.dense_imported_forward(capi.MATRIX_FP8_E4M3, weights, scales, x, workspace, out)
+
+    work = float(n_in * n_out + scales.numel() * 4 + n_in * 2 + n_out * 2)
+    return dict(step=step, parts=[("projection", step, work)], work=work,
+                metric="imported_projection_gbs", unit="GB/s", dtype="f32", bound="hbm",
+                peak=PEAK_HBM_GBS,
+                config={"workload": "qwen_imported_fp8_projection_one_token", "input_dim": n_in,
+                        "output_dim": n_out, "storage": "fp8_e4m3", "block_scales": "128x128 fp32"},
+                cpu=None)
+
+
 def copy(torch, capi):
     n = 256 * 2 ** 20   # 1 GiB read + 1 GiB written per step
     src = torch.ones(n, dtype=torch.float32, device="cuda")
@@ -370,7 +398,7 @@ def copy(torch, capi):
                         "bytes_written": n * 4}, cpu=None)
 
 
-WORKLOADS = {"copy": copy, "gdn_decode": gdn_decode, "dense_qkv": dense_qkv, "mha_train_bf16": mha_train_bf16, "mha_fwd_fp32": mha_fwd_fp32,
+WORKLOADS = {"copy": copy, "gdn_decode": gdn_decode, "dense_qkv": dense_qkv, "dense_imported": dense_imported, "mha_train_bf16": mha_train_bf16, "mha_fwd_fp32": mha_fwd_fp32,
              "gqa_prefill": gqa_prefill, "gqa_prefill_bwd": gqa_prefill_bwd, "gdn_layer_bwd": gdn_layer_bwd,
              "gqa_decode": gqa_decode,
              "gdn_scan": gdn_scan}

@@ -512,14 +512,20 @@ def dense_backward(x, matrix, d_out, workspace=None, stream=None):
 MATRIX_BF16, MATRIX_F32, MATRIX_FP8_E4M3 = 0, 1, 2
 
 
-def dense_imported_forward(storage, weights, scales, x, stream=None):
+def dense_imported_workspace(input_dim, device):
+    bytes_needed = lib().pluto_hip_dense_imported_workspace_bytes(input_dim)
+    return torch.empty(max(bytes_needed, 1), dtype=torch.uint8, device=device)
+
+
+def dense_imported_forward(storage, weights, scales, x, workspace=None, out=None, stream=None):
     """Imported FullyConnectedLayer projection of one bf16 token: weights
     [out, in] (bfloat16, float32, or uint8 FP8 E4M3 codes with float32 block
     scales) times x bf16 [in] -> bf16 [out]."""
     output_dim, input_dim = weights.shape
-    bytes_needed = lib().pluto_hip_dense_imported_workspace_bytes(input_dim)
-    workspace = torch.empty(max(bytes_needed, 1), dtype=torch.uint8, device=x.device)
-    out = torch.empty(output_dim, dtype=torch.bfloat16, device=x.device)
+    if workspace is None:
+        workspace = dense_imported_workspace(input_dim, x.device)
+    if out is None:
+        out = torch.empty(output_dim, dtype=torch.bfloat16, device=x.device)
     check(lib().pluto_hip_dense_imported_forward(
         stream or current_stream(), storage, ptr(weights), None if scales is None else ptr(scales),
         ptr(x), input_dim, output_dim, ptr(out), ptr(workspace), workspace.numel()))

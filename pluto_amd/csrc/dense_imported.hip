@@ -6,9 +6,9 @@
 //                                          mat-vec -> bf16
 // One frozen checkpoint matrix [output_dim, input_dim] in bf16, fp32 or OCP
 // FP8 E4M3 with FP32 scales [ceil(out/128), ceil(in/128)] times one bf16
-// token.  Byte-bound: every weight is read once.  A wave owns an output row
-// and reads it in 16-byte pieces (whenever rows start 16-byte aligned), the
-// token comes from the FP32 copy the first kernel leaves in the workspace;
+// token.  Byte-bound: every weight is read once.  A wave owns four output
+// rows and reads them in 16-byte pieces (whenever rows start 16-byte aligned),
+// the token comes from the FP32 copy the first kernel leaves in the workspace;
 // all arithmetic is FP32, the 64 lane sums are added by a butterfly.
 #include "dense.h"
 
@@ -70,64 +70,107 @@ struct MatVecArgs {
   int cols = 0, rows = 0;
 };
 
-// STORAGE: 0 bf16, 1 fp32, 2 FP8 E4M3.  One wave per output row.
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+
+// Four FP8 E4M3 codes of a word as floats, by the hardware conversion.
+__device__ inline void fp8_word(uint32_t word, float* out) {
+  const floatx2 lo = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(word), false);
+  const floatx2 hi = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(word), true);
+  out[0] = lo.x, out[1] = lo.y, out[2] = hi.x, out[3] = hi.y;
+}
+
+constexpr int kRowsPerWave = 4;
+
+// STORAGE: 0 bf16, 1 fp32, 2 FP8 E4M3.  A wave owns four consecutive output
+// rows: a lane takes 16-byte pieces of them at the same columns, so the token
+// values of a piece are loaded once for four rows and four weight loads are
+// in flight per lane.
 template <int STORAGE>
 __global__ void __launch_bounds__(256) imported_matvec_kernel(MatVecArgs a) {
   constexpr int kElementBytes = STORAGE == 0 ? 2 : (STORAGE == 1 ? 4 : 1);
   constexpr int kPiece = 16 / kElementBytes;  // elements per 16-byte load
+  constexpr int R = kRowsPerWave;
   const int lane = threadIdx.x % 64;
-  const int row = blockIdx.x * 4 + threadIdx.x / 64;
-  if (row >= a.rows) return;
-  const size_t row_start = static_cast<size_t>(row) * a.cols;
+  const int row0 = (blockIdx.x * 4 + threadIdx.x / 64) * R;
+  if (row0 >= a.rows) return;
   const int scale_cols = (a.cols + kGroup - 1) / kGroup;
-  const float* scale_row =
-      STORAGE == 2 ? a.scales + static_cast<size_t>(row / kGroup) * scale_cols : nullptr;
-  float sum = 0.0f;
-  auto element = [&](int c) {
-    const size_t i = row_start + c;
+  size_t row_start[R];
+  const float* scale_row[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int row = min(row0 + r, a.rows - 1);  // rows past the end repeat the last one
+    row_start[r] = static_cast<size_t>(row) * a.cols;
+    scale_row[r] =
+        STORAGE == 2 ? a.scales + static_cast<size_t>(row / kGroup) * scale_cols : nullptr;
+  }
+  float sum[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) sum[r] = 0.0f;
+  auto element = [&](int r, int c) {
+    const size_t i = row_start[r] + c;
     if constexpr (STORAGE == 0)
       return bf16_bits_to_float(static_cast<const uint16_t*>(a.weights)[i]);
     else if constexpr (STORAGE == 1)
       return static_cast<const float*>(a.weights)[i];
     else
-      return fp8_value(static_cast<const uint8_t*>(a.weights)[i]) * scale_row[c / kGroup];
+      return fp8_value(static_cast<const uint8_t*>(a.weights)[i]) * scale_row[r][c / kGroup];
   };
   int done = 0;
   if ((static_cast<size_t>(a.cols) * kElementBytes) % 16 == 0) {
     // every row starts on a 16-byte boundary (the buffer itself is at least
     // 256-byte aligned): whole pieces, a piece never straddles a scale block
-    const unsigned char* base =
-        static_cast<const unsigned char*>(a.weights) + row_start * kElementBytes;
+    const unsigned char* base = static_cast<const unsigned char*>(a.weights);
     const int pieces = a.cols / kPiece;
     for (int p = lane; p < pieces; p += 64) {
-      const uint4 raw = *reinterpret_cast<const uint4*>(base + static_cast<size_t>(p) * 16);
-      const uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
       const int c0 = p * kPiece;
-      if constexpr (STORAGE == 0) {
+      uint4 raw[R];
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
-          sum += __uint_as_float(words[w] << 16) * a.token[c0 + 2 * w];
-          sum += __uint_as_float(words[w] & 0xffff0000u) * a.token[c0 + 2 * w + 1];
+      for (int r = 0; r < R; ++r)
+        raw[r] = *reinterpret_cast<const uint4*>(base + row_start[r] * kElementBytes +
+                                                 static_cast<size_t>(p) * 16);
+      float x[kPiece];
+#pragma unroll
+      for (int q = 0; q < kPiece / 4; ++q) {
+        const float4 v = *reinterpret_cast<const float4*>(a.token + c0 + 4 * q);
+        x[4 * q] = v.x, x[4 * q + 1] = v.y, x[4 * q + 2] = v.z, x[4 * q + 3] = v.w;
+      }
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const uint32_t words[4] = {raw[r].x, raw[r].y, raw[r].z, raw[r].w};
+        if constexpr (STORAGE == 0) {
+#pragma unroll
+          for (int w = 0; w < 4; ++w) {
+            sum[r] += __uint_as_float(words[w] << 16) * x[2 * w];
+            sum[r] += __uint_as_float(words[w] & 0xffff0000u) * x[2 * w + 1];
+          }
+        } else if constexpr (STORAGE == 1) {
+#pragma unroll
+          for (int w = 0; w < 4; ++w) sum[r] += __uint_as_float(words[w]) * x[w];
+        } else {
+          float part = 0.0f;
+#pragma unroll
+          for (int w = 0; w < 4; ++w) {
+            float values[4];
+            fp8_word(words[w], values);
+#pragma unroll
+            for (int b = 0; b < 4; ++b) part += values[b] * x[4 * w + b];
+          }
+          sum[r] += part * scale_row[r][c0 / kGroup];
         }
-      } else if constexpr (STORAGE == 1) {
-#pragma unroll
-        for (int w = 0; w < 4; ++w) sum += __uint_as_float(words[w]) * a.token[c0 + w];
-      } else {
-        const float scale = scale_row[c0 / kGroup];
-        float part = 0.0f;
-#pragma unroll
-        for (int w = 0; w < 4; ++w)
-#pragma unroll
-          for (int b = 0; b < 4; ++b)
-            part += fp8_value((words[w] >> (8 * b)) & 0xffu) * a.token[c0 + 4 * w + b];
-        sum += part * scale;
       }
     }
     done = pieces * kPiece;
   }
-  for (int c = done + lane; c < a.cols; c += 64) sum += element(c) * a.token[c];
-  sum = wave_sum(sum);
-  if (lane == 0) a.out[row] = float_to_bf16_bits(sum);
+  for (int c = done + lane; c < a.cols; c += 64) {
+    const float x = a.token[c];
+#pragma unroll
+    for (int r = 0; r < R; ++r) sum[r] += element(r, c) * x;
+  }
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const float total = wave_sum(sum[r]);
+    if (lane == 0 && row0 + r < a.rows) a.out[row0 + r] = float_to_bf16_bits(total);
+  }
 }
 
 }  // namespace
@@ -154,7 +197,8 @@ int launch_dense_imported_forward(hipStream_t s, int storage, const void* weight
   a.out = static_cast<uint16_t*>(output);
   a.cols = input_dim;
   a.rows = output_dim;
-  const unsigned blocks = static_cast<unsigned>((output_dim + 3) / 4);
+  const unsigned blocks =
+      static_cast<unsigned>((output_dim + 4 * kRowsPerWave - 1) / (4 * kRowsPerWave));
   if (storage == PLUTO_HIP_MATRIX_BF16)
     imported_matvec_kernel<0><<<blocks, 256, 0, s>>>(a);
   else if (storage == PLUTO_HIP_MATRIX_F32)

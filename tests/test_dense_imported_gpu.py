@@ -93,6 +93,26 @@ def test_dynamic_quantization_zero_tiny_ties_and_tail(capi, oracle):
     assert np.abs(got[256:384]).max() > 0
 
 
+def test_every_fp8_code_as_a_weight(capi, oracle):
+    """Row r holds code r once, in a column that the 16-byte path reads (rows
+    of 128 codes) or in one that the element path reads (rows of 130)."""
+    codes = np.arange(256)
+    keep = (codes & 0x7f) != 0x7f   # the two NaN codes
+    for cols, column in ((128, 37), (130, 129)):
+        weights = np.zeros((256, cols), np.uint8)
+        weights[codes, column] = codes
+        x = np.zeros(cols, np.float32)
+        x[column] = 1.0     # a group maximum of 1: quantized exactly
+        scales = np.ones((2, (cols + 127) // 128), np.float32)
+        got = capi.dense_imported_forward(capi.MATRIX_FP8_E4M3, torch.from_numpy(weights).cuda(),
+                                          torch.from_numpy(scales).cuda(), bf16_tensor(oracle, x))
+        torch.cuda.synchronize()
+        got = got.float().cpu().numpy()
+        want = oracle.bf16_round(oracle.fp8_e4m3_to_f32(codes.astype(np.uint8)))
+        assert np.array_equal(got[keep], want[keep]), cols
+        assert np.all(np.isnan(got[~keep]))
+
+
 def test_rejects_bad_arguments(capi):
     lib = capi.lib()
     w = torch.zeros(6, dtype=torch.float32, device="cuda")
