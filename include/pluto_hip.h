@@ -457,12 +457,26 @@ int pluto_hip_dense_backward(void* stream, int dtype, const void* input,
 #define PLUTO_HIP_MATRIX_F32 1
 #define PLUTO_HIP_MATRIX_FP8_E4M3 2
 #define PLUTO_HIP_IMPORTED_MAX_DIM 1048576
+#define PLUTO_HIP_IMPORTED_MAX_TOKENS 4096
 size_t pluto_hip_dense_imported_workspace_bytes(int input_dim);
 int pluto_hip_dense_imported_forward(void* stream, int storage,
                                      const void* weights, const float* scales,
                                      const void* input, int input_dim,
                                      int output_dim, void* output,
                                      void* workspace, size_t workspace_bytes);
+/* The same projection for `tokens` independent tokens (the decoder step of
+ * several sequences, qwen/model.cc:405-428 lifted from batch one): input bf16
+ * [tokens, input_dim] -> output bf16 [tokens, output_dim].  Up to eight tokens
+ * share one pass over the weights; row t of the result is bit for bit what
+ * the one-token call gives for token t. */
+size_t pluto_hip_dense_imported_batch_workspace_bytes(int tokens, int input_dim);
+int pluto_hip_dense_imported_forward_batch(void* stream, int storage,
+                                           const void* weights,
+                                           const float* scales,
+                                           const void* input, int tokens,
+                                           int input_dim, int output_dim,
+                                           void* output, void* workspace,
+                                           size_t workspace_bytes);
 
 #ifdef __cplusplus
 }

@@ -127,6 +127,9 @@ SIGNATURES = {
                                       _SZ]),
     "pluto_hip_dense_imported_workspace_bytes": (_SZ, [_I]),
     "pluto_hip_dense_imported_forward": (_I, [_VP, _I, _VP, _VP, _VP, _I, _I, _VP, _VP, _SZ]),
+    "pluto_hip_dense_imported_batch_workspace_bytes": (_SZ, [_I, _I]),
+    "pluto_hip_dense_imported_forward_batch": (_I, [_VP, _I, _VP, _VP, _VP, _I, _I, _I, _VP, _VP,
+                                                    _SZ]),
     "pluto_hip_gdn_recurrence": (_I, [_VP, ctypes.POINTER(DeltaParams), _I, _I, _VP, _VP,
                                       _VP, _VP, _VP, _I, ctypes.c_float, _VP, _VP, _I]),
 }
@@ -529,4 +532,20 @@ def dense_imported_forward(storage, weights, scales, x, workspace=None, out=None
     check(lib().pluto_hip_dense_imported_forward(
         stream or current_stream(), storage, ptr(weights), None if scales is None else ptr(scales),
         ptr(x), input_dim, output_dim, ptr(out), ptr(workspace), workspace.numel()))
+    return out
+
+
+def dense_imported_forward_batch(storage, weights, scales, x, workspace=None, out=None,
+                                 stream=None):
+    """The imported projection for x bf16 [tokens, in] -> bf16 [tokens, out]."""
+    output_dim, input_dim = weights.shape
+    tokens = x.shape[0]
+    if workspace is None:
+        bytes_needed = lib().pluto_hip_dense_imported_batch_workspace_bytes(tokens, input_dim)
+        workspace = torch.empty(max(bytes_needed, 1), dtype=torch.uint8, device=x.device)
+    if out is None:
+        out = torch.empty((tokens, output_dim), dtype=torch.bfloat16, device=x.device)
+    check(lib().pluto_hip_dense_imported_forward_batch(
+        stream or current_stream(), storage, ptr(weights), None if scales is None else ptr(scales),
+        ptr(x), tokens, input_dim, output_dim, ptr(out), ptr(workspace), workspace.numel()))
     return out

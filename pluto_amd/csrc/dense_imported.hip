@@ -48,6 +48,8 @@ template <bool FP8>
 __global__ void __launch_bounds__(kGroup)
 imported_token_kernel(const uint16_t* x, int n, float* token) {
   __shared__ float largest[2];
+  x += static_cast<size_t>(blockIdx.y) * n;      // one token per grid row
+  token += static_cast<size_t>(blockIdx.y) * n;
   const int i = blockIdx.x * kGroup + threadIdx.x;
   const float v = i < n ? bf16_bits_to_float(x[i]) : 0.0f;
   if constexpr (!FP8) {
@@ -65,8 +67,8 @@ imported_token_kernel(const uint16_t* x, int n, float* token) {
 struct MatVecArgs {
   const void* weights = nullptr;
   const float* scales = nullptr;  // FP8 only
-  const float* token = nullptr;
-  uint16_t* out = nullptr;
+  const float* token = nullptr;  // [tokens, cols]
+  uint16_t* out = nullptr;       // [tokens, rows]
   int cols = 0, rows = 0;
 };
 
@@ -84,8 +86,9 @@ constexpr int kRowsPerWave = 4;
 // STORAGE: 0 bf16, 1 fp32, 2 FP8 E4M3.  A wave owns four consecutive output
 // rows: a lane takes 16-byte pieces of them at the same columns, so the token
 // values of a piece are loaded once for four rows and four weight loads are
-// in flight per lane.
-template <int STORAGE>
+// in flight per lane.  TOKENS tokens share one pass over the weights; each
+// token's sum is formed exactly as in the one-token kernel.
+template <int STORAGE, int TOKENS>
 __global__ void __launch_bounds__(256) imported_matvec_kernel(MatVecArgs a) {
   constexpr int kElementBytes = STORAGE == 0 ? 2 : (STORAGE == 1 ? 4 : 1);
   constexpr int kPiece = 16 / kElementBytes;  // elements per 16-byte load
@@ -103,9 +106,11 @@ __global__ void __launch_bounds__(256) imported_matvec_kernel(MatVecArgs a) {
     scale_row[r] =
         STORAGE == 2 ? a.scales + static_cast<size_t>(row / kGroup) * scale_cols : nullptr;
   }
-  float sum[R];
+  float sum[TOKENS][R];
 #pragma unroll
-  for (int r = 0; r < R; ++r) sum[r] = 0.0f;
+  for (int t = 0; t < TOKENS; ++t)
+#pragma unroll
+    for (int r = 0; r < R; ++r) sum[t][r] = 0.0f;
   auto element = [&](int r, int c) {
     const size_t i = row_start[r] + c;
     if constexpr (STORAGE == 0)
@@ -128,62 +133,102 @@ __global__ void __launch_bounds__(256) imported_matvec_kernel(MatVecArgs a) {
       for (int r = 0; r < R; ++r)
         raw[r] = *reinterpret_cast<const uint4*>(base + row_start[r] * kElementBytes +
                                                  static_cast<size_t>(p) * 16);
-      float x[kPiece];
-#pragma unroll
-      for (int q = 0; q < kPiece / 4; ++q) {
-        const float4 v = *reinterpret_cast<const float4*>(a.token + c0 + 4 * q);
-        x[4 * q] = v.x, x[4 * q + 1] = v.y, x[4 * q + 2] = v.z, x[4 * q + 3] = v.w;
-      }
+      // the rows' values of this piece, decoded once for all tokens
+      float w[R][kPiece];
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         const uint32_t words[4] = {raw[r].x, raw[r].y, raw[r].z, raw[r].w};
-        if constexpr (STORAGE == 0) {
 #pragma unroll
-          for (int w = 0; w < 4; ++w) {
-            sum[r] += __uint_as_float(words[w] << 16) * x[2 * w];
-            sum[r] += __uint_as_float(words[w] & 0xffff0000u) * x[2 * w + 1];
+        for (int k = 0; k < 4; ++k) {
+          if constexpr (STORAGE == 0) {
+            w[r][2 * k] = __uint_as_float(words[k] << 16);
+            w[r][2 * k + 1] = __uint_as_float(words[k] & 0xffff0000u);
+          } else if constexpr (STORAGE == 1) {
+            w[r][k] = __uint_as_float(words[k]);
+          } else {
+            fp8_word(words[k], &w[r][4 * k]);
           }
-        } else if constexpr (STORAGE == 1) {
+        }
+      }
 #pragma unroll
-          for (int w = 0; w < 4; ++w) sum[r] += __uint_as_float(words[w]) * x[w];
-        } else {
-          float part = 0.0f;
+      for (int t = 0; t < TOKENS; ++t) {
+        float x[kPiece];
 #pragma unroll
-          for (int w = 0; w < 4; ++w) {
-            float values[4];
-            fp8_word(words[w], values);
+        for (int q = 0; q < kPiece / 4; ++q) {
+          const float4 v = *reinterpret_cast<const float4*>(
+              a.token + static_cast<size_t>(t) * a.cols + c0 + 4 * q);
+          x[4 * q] = v.x, x[4 * q + 1] = v.y, x[4 * q + 2] = v.z, x[4 * q + 3] = v.w;
+        }
 #pragma unroll
-            for (int b = 0; b < 4; ++b) part += values[b] * x[4 * w + b];
+        for (int r = 0; r < R; ++r) {
+          if constexpr (STORAGE == 2) {
+            float part = 0.0f;
+#pragma unroll
+            for (int e = 0; e < kPiece; ++e) part += w[r][e] * x[e];
+            sum[t][r] += part * scale_row[r][c0 / kGroup];
+          } else {
+#pragma unroll
+            for (int e = 0; e < kPiece; ++e) sum[t][r] += w[r][e] * x[e];
           }
-          sum[r] += part * scale_row[r][c0 / kGroup];
         }
       }
     }
     done = pieces * kPiece;
   }
   for (int c = done + lane; c < a.cols; c += 64) {
-    const float x = a.token[c];
+    float value[R];
 #pragma unroll
-    for (int r = 0; r < R; ++r) sum[r] += element(r, c) * x;
+    for (int r = 0; r < R; ++r) value[r] = element(r, c);
+#pragma unroll
+    for (int t = 0; t < TOKENS; ++t) {
+      const float x = a.token[static_cast<size_t>(t) * a.cols + c];
+#pragma unroll
+      for (int r = 0; r < R; ++r) sum[t][r] += value[r] * x;
+    }
   }
 #pragma unroll
-  for (int r = 0; r < R; ++r) {
-    const float total = wave_sum(sum[r]);
-    if (lane == 0 && row0 + r < a.rows) a.out[row0 + r] = float_to_bf16_bits(total);
+  for (int t = 0; t < TOKENS; ++t)
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const float total = wave_sum(sum[t][r]);
+      if (lane == 0 && row0 + r < a.rows)
+        a.out[static_cast<size_t>(t) * a.rows + row0 + r] = float_to_bf16_bits(total);
+    }
+}
+
+template <int STORAGE>
+void launch_matvec(hipStream_t s, MatVecArgs a, int tokens) {
+  const unsigned blocks =
+      static_cast<unsigned>((a.rows + 4 * kRowsPerWave - 1) / (4 * kRowsPerWave));
+  // up to eight tokens share a pass over the weights
+  while (tokens > 0) {
+    const int now = tokens >= 8 ? 8 : (tokens >= 4 ? 4 : (tokens >= 2 ? 2 : 1));
+    if (now == 8)
+      imported_matvec_kernel<STORAGE, 8><<<blocks, 256, 0, s>>>(a);
+    else if (now == 4)
+      imported_matvec_kernel<STORAGE, 4><<<blocks, 256, 0, s>>>(a);
+    else if (now == 2)
+      imported_matvec_kernel<STORAGE, 2><<<blocks, 256, 0, s>>>(a);
+    else
+      imported_matvec_kernel<STORAGE, 1><<<blocks, 256, 0, s>>>(a);
+    a.token += static_cast<size_t>(now) * a.cols;
+    a.out += static_cast<size_t>(now) * a.rows;
+    tokens -= now;
   }
 }
 
 }  // namespace
 
-size_t dense_imported_workspace_bytes(int input_dim) {
-  return align_up(static_cast<size_t>(input_dim) * sizeof(float), 256);
+size_t dense_imported_workspace_bytes(int tokens, int input_dim) {
+  return align_up(static_cast<size_t>(tokens) * input_dim * sizeof(float), 256);
 }
 
 int launch_dense_imported_forward(hipStream_t s, int storage, const void* weights,
-                                  const float* scales, const void* input, int input_dim,
-                                  int output_dim, void* output, void* workspace) {
+                                  const float* scales, const void* input, int tokens,
+                                  int input_dim, int output_dim, void* output, void* workspace) {
   float* token = static_cast<float*>(workspace);
-  const unsigned groups = static_cast<unsigned>((input_dim + kGroup - 1) / kGroup);
+  const dim3 groups(static_cast<unsigned>((input_dim + kGroup - 1) / kGroup),
+                    static_cast<unsigned>(tokens));
   if (storage == PLUTO_HIP_MATRIX_FP8_E4M3)
     imported_token_kernel<true><<<groups, kGroup, 0, s>>>(static_cast<const uint16_t*>(input),
                                                           input_dim, token);
@@ -197,14 +242,12 @@ int launch_dense_imported_forward(hipStream_t s, int storage, const void* weight
   a.out = static_cast<uint16_t*>(output);
   a.cols = input_dim;
   a.rows = output_dim;
-  const unsigned blocks =
-      static_cast<unsigned>((output_dim + 4 * kRowsPerWave - 1) / (4 * kRowsPerWave));
   if (storage == PLUTO_HIP_MATRIX_BF16)
-    imported_matvec_kernel<0><<<blocks, 256, 0, s>>>(a);
+    launch_matvec<0>(s, a, tokens);
   else if (storage == PLUTO_HIP_MATRIX_F32)
-    imported_matvec_kernel<1><<<blocks, 256, 0, s>>>(a);
+    launch_matvec<1>(s, a, tokens);
   else
-    imported_matvec_kernel<2><<<blocks, 256, 0, s>>>(a);
+    launch_matvec<2>(s, a, tokens);
   return launch_status();
 }
 
@@ -214,15 +257,8 @@ using namespace pluto_hip;
 
 extern "C" {
 
-size_t pluto_hip_dense_imported_workspace_bytes(int input_dim) {
-  if (input_dim <= 0 || input_dim > PLUTO_HIP_IMPORTED_MAX_DIM) return 0;
-  return dense_imported_workspace_bytes(input_dim);
-}
-
-int pluto_hip_dense_imported_forward(void* stream, int storage, const void* weights,
-                                     const float* scales, const void* input, int input_dim,
-                                     int output_dim, void* output, void* workspace,
-                                     size_t workspace_bytes) {
+static int validate_imported(int storage, const float* scales, int tokens, int input_dim,
+                             int output_dim) {
   if (storage != PLUTO_HIP_MATRIX_BF16 && storage != PLUTO_HIP_MATRIX_F32 &&
       storage != PLUTO_HIP_MATRIX_FP8_E4M3)
     return PLUTO_HIP_EINVAL;
@@ -230,13 +266,43 @@ int pluto_hip_dense_imported_forward(void* stream, int storage, const void* weig
   if (input_dim <= 0 || input_dim > PLUTO_HIP_IMPORTED_MAX_DIM || output_dim <= 0 ||
       output_dim > PLUTO_HIP_IMPORTED_MAX_DIM)
     return PLUTO_HIP_EINVAL;
+  if (tokens <= 0 || tokens > PLUTO_HIP_IMPORTED_MAX_TOKENS) return PLUTO_HIP_EINVAL;
   // :279-281: only FP8 weights have block scales
   if ((storage == PLUTO_HIP_MATRIX_FP8_E4M3) != (scales != nullptr)) return PLUTO_HIP_EINVAL;
+  return 0;
+}
+
+size_t pluto_hip_dense_imported_workspace_bytes(int input_dim) {
+  return pluto_hip_dense_imported_batch_workspace_bytes(1, input_dim);
+}
+
+size_t pluto_hip_dense_imported_batch_workspace_bytes(int tokens, int input_dim) {
+  if (input_dim <= 0 || input_dim > PLUTO_HIP_IMPORTED_MAX_DIM || tokens <= 0 ||
+      tokens > PLUTO_HIP_IMPORTED_MAX_TOKENS)
+    return 0;
+  return dense_imported_workspace_bytes(tokens, input_dim);
+}
+
+int pluto_hip_dense_imported_forward(void* stream, int storage, const void* weights,
+                                     const float* scales, const void* input, int input_dim,
+                                     int output_dim, void* output, void* workspace,
+                                     size_t workspace_bytes) {
+  return pluto_hip_dense_imported_forward_batch(stream, storage, weights, scales, input, 1,
+                                                input_dim, output_dim, output, workspace,
+                                                workspace_bytes);
+}
+
+int pluto_hip_dense_imported_forward_batch(void* stream, int storage, const void* weights,
+                                           const float* scales, const void* input, int tokens,
+                                           int input_dim, int output_dim, void* output,
+                                           void* workspace, size_t workspace_bytes) {
+  const int status = validate_imported(storage, scales, tokens, input_dim, output_dim);
+  if (status != 0) return status;
   if (!weights || !input || !output) return PLUTO_HIP_EINVAL;
-  if (!workspace || workspace_bytes < dense_imported_workspace_bytes(input_dim))
+  if (!workspace || workspace_bytes < dense_imported_workspace_bytes(tokens, input_dim))
     return PLUTO_HIP_EWORKSPACE;
   return launch_dense_imported_forward(static_cast<hipStream_t>(stream), storage, weights, scales,
-                                       input, input_dim, output_dim, output, workspace);
+                                       input, tokens, input_dim, output_dim, output, workspace);
 }
 
 }  // extern "C"

@@ -113,6 +113,31 @@ def test_every_fp8_code_as_a_weight(capi, oracle):
         assert np.all(np.isnan(got[~keep]))
 
 
+@pytest.mark.parametrize("cols", [263, 512])
+def test_batch_rows_equal_the_one_token_calls(capi, oracle, cols):
+    """Eleven tokens run as passes of 8, 2 and 1 tokens; every row must be bit
+    for bit the one-token result (vector path: 512 columns, element path: 263)."""
+    rows, tokens = 70, 11
+    rng = np.random.default_rng(cols)
+    source = rng.standard_normal((rows, cols)).astype(np.float32)
+    x = bf16_tensor(oracle, rng.standard_normal((tokens, cols)))
+    scales = torch.from_numpy(rng.uniform(0.5, 2.0, ((rows + 127) // 128, (cols + 127) // 128))
+                              .astype(np.float32)).cuda()
+    cases = [(capi.MATRIX_F32, torch.from_numpy(source).cuda(), None),
+             (capi.MATRIX_BF16, torch.from_numpy(source).cuda().to(torch.bfloat16), None),
+             (capi.MATRIX_FP8_E4M3, torch.from_numpy(oracle.f32_to_fp8_e4m3(source)).cuda(), scales)]
+    for storage, weights, s in cases:
+        batch = capi.dense_imported_forward_batch(storage, weights, s, x)
+        singles = torch.stack([capi.dense_imported_forward(storage, weights, s, x[t].contiguous())
+                               for t in range(tokens)])
+        torch.cuda.synchronize()
+        assert torch.equal(batch.view(torch.int16), singles.view(torch.int16)), storage
+    lib = capi.lib()
+    assert lib.pluto_hip_dense_imported_batch_workspace_bytes(0, cols) == 0
+    assert lib.pluto_hip_dense_imported_batch_workspace_bytes(4097, cols) == 0
+    assert lib.pluto_hip_dense_imported_batch_workspace_bytes(tokens, cols) >= tokens * cols * 4
+
+
 def test_rejects_bad_arguments(capi):
     lib = capi.lib()
     w = torch.zeros(6, dtype=torch.float32, device="cuda")
