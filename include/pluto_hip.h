@@ -467,8 +467,10 @@ int pluto_hip_dense_imported_forward(void* stream, int storage,
 /* The same projection for `tokens` independent tokens (the decoder step of
  * several sequences, qwen/model.cc:405-428 lifted from batch one): input bf16
  * [tokens, input_dim] -> output bf16 [tokens, output_dim].  Up to eight tokens
- * share one pass over the weights; row t of the result is bit for bit what
- * the one-token call gives for token t. */
+ * share one vector pass over the weights, and row t of the result is bit for
+ * bit what the one-token call gives for token t; larger batches of bf16 or
+ * FP8 weights with input_dim a multiple of 128 run on the matrix cores and
+ * agree with the one-token calls to FP32 summation order. */
 size_t pluto_hip_dense_imported_batch_workspace_bytes(int tokens, int input_dim);
 int pluto_hip_dense_imported_forward_batch(void* stream, int storage,
                                            const void* weights,

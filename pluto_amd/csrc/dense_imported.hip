@@ -196,6 +196,133 @@ __global__ void __launch_bounds__(256) imported_matvec_kernel(MatVecArgs a) {
     }
 }
 
+// ---- more than eight tokens: the matrix cores --------------------------------
+// out[t, r] = sum_k w[r, k] x[t, k] as a 32-row x 32-token tile per wave on
+// v_mfma_f32_32x32x16_bf16.  bf16 weights and tokens are exact operands.  FP8
+// codes are exact in bf16 too, so FP8 weights are multiplied unscaled with the
+// FP8 values of the quantized tokens, and each block of 128 contraction
+// elements is scaled once by (weight block scale) x (token group scale):
+// the same products as (w s_w)(x s_x), summed in FP32 in a different order.
+// Lane (n, h) covers elements [64 h, 64 h + 64) of a 128-element block, for
+// weight row n (A operand) and for token n (B operand).  The four waves of a
+// workgroup share a tile and take every fourth block; their partial tiles are
+// added in wave order through LDS.
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(16))) float floatx16;
+
+// tokens as FP8 values in bf16 [tokens, n] and their group scales [tokens, n / 128]
+__global__ void __launch_bounds__(kGroup)
+imported_token_fp8_kernel(const uint16_t* x, int n, uint16_t* values, float* scales) {
+  __shared__ float largest[2];
+  x += static_cast<size_t>(blockIdx.y) * n;
+  values += static_cast<size_t>(blockIdx.y) * n;
+  const int i = blockIdx.x * kGroup + threadIdx.x;
+  const float v = i < n ? bf16_bits_to_float(x[i]) : 0.0f;
+  const float mine = wave_max(fabsf(v));
+  if (threadIdx.x % 64 == 0) largest[threadIdx.x / 64] = mine;
+  __syncthreads();
+  const float scale = fmaxf(largest[0], largest[1]) / 448.0f;
+  if (i < n) values[i] = float_to_bf16_bits(fp8_round(v / fmaxf(scale, 1e-12f)));
+  if (threadIdx.x == 0) scales[static_cast<size_t>(blockIdx.y) * gridDim.x + blockIdx.x] = scale;
+}
+
+struct TileArgs {
+  const void* weights = nullptr;
+  const float* weight_scales = nullptr;  // FP8 only
+  const uint16_t* tokens = nullptr;      // bf16 [count, cols]
+  const float* token_scales = nullptr;   // FP8 only: [count, cols / 128]
+  uint16_t* out = nullptr;               // [count, rows]
+  int cols = 0, rows = 0, count = 0;     // count <= 32
+};
+
+template <bool HIGH>
+__device__ inline uint32_t fp8_pair_to_bf16(uint32_t word) {
+  const floatx2 v = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(word), HIGH);
+  return (__float_as_uint(v.y) & 0xffff0000u) | (__float_as_uint(v.x) >> 16);
+}
+
+template <bool FP8>
+__global__ void __launch_bounds__(256) imported_tile_kernel(TileArgs a) {
+  __shared__ float partial[3][16][64];
+  const int lane = threadIdx.x % 64, n = lane % 32, h = lane / 32;
+  const int wave = threadIdx.x / 64;
+  const int row_base = blockIdx.x * 32;
+  const int row = min(row_base + n, a.rows - 1);   // rows and tokens past the end repeat
+  const int token = min(n, a.count - 1);           // the last one and are not stored
+  const int groups = a.cols / kGroup;
+  const unsigned char* w = static_cast<const unsigned char*>(a.weights) +
+                           (static_cast<size_t>(row) * a.cols + 64 * h) * (FP8 ? 1 : 2);
+  const uint16_t* x = a.tokens + static_cast<size_t>(token) * a.cols + 64 * h;
+  const float* block_scale =
+      FP8 ? a.weight_scales + static_cast<size_t>(row_base / kGroup) * groups : nullptr;
+  const float* group_scale = FP8 ? a.token_scales + static_cast<size_t>(token) * groups : nullptr;
+  floatx16 total;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) total[i] = 0.0f;
+  for (int g = wave; g < groups; g += 4) {
+    uint4 xs[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) xs[j] = *reinterpret_cast<const uint4*>(x + g * kGroup + 8 * j);
+    if constexpr (FP8) {
+      uint4 raw[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        raw[j] = *reinterpret_cast<const uint4*>(w + static_cast<size_t>(g) * kGroup + 16 * j);
+      floatx16 acc;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const uint32_t lo = j % 2 == 0 ? raw[j / 2].x : raw[j / 2].z;
+        const uint32_t hi = j % 2 == 0 ? raw[j / 2].y : raw[j / 2].w;
+        const uint4 bits = make_uint4(fp8_pair_to_bf16<false>(lo), fp8_pair_to_bf16<true>(lo),
+                                      fp8_pair_to_bf16<false>(hi), fp8_pair_to_bf16<true>(hi));
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, bits),
+                                                      __builtin_bit_cast(bf16x8, xs[j]), acc, 0, 0,
+                                                      0);
+      }
+      const float scale = block_scale[g] * group_scale[g];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) total[i] += acc[i] * scale;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const uint4 bits =
+            *reinterpret_cast<const uint4*>(w + (static_cast<size_t>(g) * kGroup + 8 * j) * 2);
+        total = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, bits),
+                                                        __builtin_bit_cast(bf16x8, xs[j]), total,
+                                                        0, 0, 0);
+      }
+    }
+  }
+  if (wave > 0) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) partial[wave - 1][i][lane] = total[i];
+  }
+  __syncthreads();
+  if (wave > 0) return;
+#pragma unroll
+  for (int i = 0; i < 16; ++i)
+    total[i] = ((total[i] + partial[0][i][lane]) + partial[1][i][lane]) + partial[2][i][lane];
+  // accumulator element 4 q + i = (row 8 q + 4 h + i, token n)
+  if (n >= a.count) return;
+#pragma unroll
+  for (int q = 0; q < 4; ++q)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = row_base + 8 * q + 4 * h + i;
+      if (r < a.rows)
+        a.out[static_cast<size_t>(n) * a.rows + r] = float_to_bf16_bits(total[4 * q + i]);
+    }
+}
+
+// The matrix-core path takes bf16 and FP8 weights whose rows are whole
+// 128-element blocks; fewer than nine tokens are cheaper on the vector path.
+bool tile_path(int storage, int tokens, int input_dim) {
+  return storage != PLUTO_HIP_MATRIX_F32 && tokens > 8 && input_dim % kGroup == 0;
+}
+
 template <int STORAGE>
 void launch_matvec(hipStream_t s, MatVecArgs a, int tokens) {
   const unsigned blocks =
@@ -220,15 +347,48 @@ void launch_matvec(hipStream_t s, MatVecArgs a, int tokens) {
 }  // namespace
 
 size_t dense_imported_workspace_bytes(int tokens, int input_dim) {
-  return align_up(static_cast<size_t>(tokens) * input_dim * sizeof(float), 256);
+  // FP32 tokens (vector path), or their FP8 values in bf16 and the group
+  // scales (matrix-core path): the first is the larger
+  return align_up(static_cast<size_t>(tokens) * input_dim * sizeof(float), 256) + 256;
 }
 
 int launch_dense_imported_forward(hipStream_t s, int storage, const void* weights,
                                   const float* scales, const void* input, int tokens,
                                   int input_dim, int output_dim, void* output, void* workspace) {
-  float* token = static_cast<float*>(workspace);
   const dim3 groups(static_cast<unsigned>((input_dim + kGroup - 1) / kGroup),
                     static_cast<unsigned>(tokens));
+  if (tile_path(storage, tokens, input_dim)) {
+    const bool fp8 = storage == PLUTO_HIP_MATRIX_FP8_E4M3;
+    TileArgs t;
+    t.weights = weights;
+    t.weight_scales = scales;
+    t.tokens = static_cast<const uint16_t*>(input);
+    t.cols = input_dim;
+    t.rows = output_dim;
+    if (fp8) {
+      uint16_t* values = static_cast<uint16_t*>(workspace);
+      float* token_scales = reinterpret_cast<float*>(
+          static_cast<char*>(workspace) + align_up(static_cast<size_t>(tokens) * input_dim * 2, 256));
+      imported_token_fp8_kernel<<<groups, kGroup, 0, s>>>(static_cast<const uint16_t*>(input),
+                                                          input_dim, values, token_scales);
+      t.tokens = values;
+      t.token_scales = token_scales;
+    }
+    t.out = static_cast<uint16_t*>(output);
+    const unsigned blocks = static_cast<unsigned>((output_dim + 31) / 32);
+    for (int done = 0; done < tokens; done += 32) {
+      t.count = tokens - done < 32 ? tokens - done : 32;
+      if (fp8)
+        imported_tile_kernel<true><<<blocks, 256, 0, s>>>(t);
+      else
+        imported_tile_kernel<false><<<blocks, 256, 0, s>>>(t);
+      t.tokens += static_cast<size_t>(32) * input_dim;
+      if (fp8) t.token_scales += static_cast<size_t>(32) * (input_dim / kGroup);
+      t.out += static_cast<size_t>(32) * output_dim;
+    }
+    return launch_status();
+  }
+  float* token = static_cast<float*>(workspace);
   if (storage == PLUTO_HIP_MATRIX_FP8_E4M3)
     imported_token_kernel<true><<<groups, kGroup, 0, s>>>(static_cast<const uint16_t*>(input),
                                                           input_dim, token);
