@@ -204,8 +204,8 @@ __global__ void __launch_bounds__(256) imported_matvec_kernel(MatVecArgs a) {
 // elements is scaled once by (weight block scale) x (token group scale):
 // the same products as (w s_w)(x s_x), summed in FP32 in a different order.
 // Lane (n, h) covers elements [64 h, 64 h + 64) of a 128-element block, for
-// weight row n (A operand) and for token n (B operand).  The four waves of a
-// workgroup share a tile and take every fourth block; their partial tiles are
+// weight row n (A operand) and for token n (B operand).  The eight waves of a
+// workgroup share a tile and take every eighth block; their partial tiles are
 // added in wave order through LDS.
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -242,9 +242,11 @@ __device__ inline uint32_t fp8_pair_to_bf16(uint32_t word) {
   return (__float_as_uint(v.y) & 0xffff0000u) | (__float_as_uint(v.x) >> 16);
 }
 
+constexpr int kTileWaves = 8;  // waves that split a tile's contraction
+
 template <bool FP8>
-__global__ void __launch_bounds__(256) imported_tile_kernel(TileArgs a) {
-  __shared__ float partial[3][16][64];
+__global__ void __launch_bounds__(64 * kTileWaves) imported_tile_kernel(TileArgs a) {
+  __shared__ float partial[kTileWaves - 1][16][64];
   const int lane = threadIdx.x % 64, n = lane % 32, h = lane / 32;
   const int wave = threadIdx.x / 64;
   const int row_base = blockIdx.x * 32;
@@ -260,7 +262,7 @@ __global__ void __launch_bounds__(256) imported_tile_kernel(TileArgs a) {
   floatx16 total;
 #pragma unroll
   for (int i = 0; i < 16; ++i) total[i] = 0.0f;
-  for (int g = wave; g < groups; g += 4) {
+  for (int g = wave; g < groups; g += kTileWaves) {
     uint4 xs[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) xs[j] = *reinterpret_cast<const uint4*>(x + g * kGroup + 8 * j);
@@ -304,7 +306,8 @@ __global__ void __launch_bounds__(256) imported_tile_kernel(TileArgs a) {
   if (wave > 0) return;
 #pragma unroll
   for (int i = 0; i < 16; ++i)
-    total[i] = ((total[i] + partial[0][i][lane]) + partial[1][i][lane]) + partial[2][i][lane];
+#pragma unroll
+    for (int w = 0; w < kTileWaves - 1; ++w) total[i] += partial[w][i][lane];
   // accumulator element 4 q + i = (row 8 q + 4 h + i, token n)
   if (n >= a.count) return;
 #pragma unroll
@@ -379,9 +382,9 @@ int launch_dense_imported_forward(hipStream_t s, int storage, const void* weight
     for (int done = 0; done < tokens; done += 32) {
       t.count = tokens - done < 32 ? tokens - done : 32;
       if (fp8)
-        imported_tile_kernel<true><<<blocks, 256, 0, s>>>(t);
+        imported_tile_kernel<true><<<blocks, 64 * kTileWaves, 0, s>>>(t);
       else
-        imported_tile_kernel<false><<<blocks, 256, 0, s>>>(t);
+        imported_tile_kernel<false><<<blocks, 64 * kTileWaves, 0, s>>>(t);
       t.tokens += static_cast<size_t>(32) * input_dim;
       if (fp8) t.token_scales += static_cast<size_t>(32) * (input_dim / kGroup);
       t.out += static_cast<size_t>(32) * output_dim;
