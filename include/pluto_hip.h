@@ -480,6 +480,17 @@ int pluto_hip_dense_imported_forward_batch(void* stream, int storage,
                                            void* output, void* workspace,
                                            size_t workspace_bytes);
 
+/* ------------------------------------------------------------------------
+ * Test support.  No counterpart in the reference.
+ * --------------------------------------------------------------------- */
+
+/* Routes every later call of this library, on any thread, through the
+ * any-shape FP32-arithmetic kernels (enabled != 0) or back to normal kernel
+ * selection (0), so that tests can compare the two implementations on the
+ * device.  Returns the previous setting.  This switch is the only
+ * process-wide state of the library; nothing else writes it. */
+int pluto_hip_test_force_generic(int enabled);
+
 #ifdef __cplusplus
 }
 #endif

@@ -107,6 +107,10 @@ def build_host(force=False, verbose=True):
     tests = sorted(glob.glob(os.path.join(HOST_TEST_SOURCES, "*.cc")))
     test_headers = glob.glob(os.path.join(HOST_TEST_SOURCES, "*.h"))
     if tests and (force or not _newer(HOST_TEST, tests + test_headers + headers + [HOST_LIB])):
+        # The runner (test infrastructure, unlike the two libraries above) checks
+        # results against the CPU oracle and links it: build that first, so a
+        # clean checkout needs no particular order of build steps.
+        _run(["make", "-C", os.path.join(ROOT, "oracle"), "-s"])
         with concurrent.futures.ThreadPoolExecutor(max_workers=8) as pool:
             objects = list(pool.map(_compile_host, tests))
         _run([CXX, "-o", HOST_TEST] + objects +

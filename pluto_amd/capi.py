@@ -68,6 +68,7 @@ _SZ = ctypes.c_size_t
 SIGNATURES = {
     "pluto_hip_error_name": (ctypes.c_char_p, [_I]),
     "pluto_hip_error_string": (ctypes.c_char_p, [_I]),
+    "pluto_hip_test_force_generic": (_I, [_I]),
     "pluto_hip_abi_version": (_I, []),
     "pluto_hip_target_arch": (ctypes.c_char_p, []),
     "pluto_hip_executor_create": (_I, [ctypes.POINTER(_VP)]),
@@ -151,6 +152,18 @@ def lib():
             fn.argtypes = argtypes
         _lib = handle
     return _lib
+
+
+class force_generic:
+    """Context manager around the library's test switch: inside it every call
+    runs the any-shape FP32-arithmetic kernels."""
+
+    def __enter__(self):
+        self.previous = lib().pluto_hip_test_force_generic(1)
+
+    def __exit__(self, *exc):
+        lib().pluto_hip_test_force_generic(self.previous)
+        return False
 
 
 def check(code):

@@ -462,6 +462,11 @@ bool flash_backward_supported(const GenericBackwardArgs& a) {
   auto aligned = [](const void* p) {
     return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
   };
+  // tiles of one sequence are addressed through 32-bit buffer offsets and a
+  // 32-bit descriptor size: a sequence's rows of the packed operand (the
+  // widest, 3E bf16 per row) must stay below 2 GiB
+  if (static_cast<long long>(a.context_length) * 3 * a.embedding_dim * 2 >= (1LL << 31))
+    return false;
   return aligned(a.qkv) && aligned(a.out) && aligned(a.d_out) && aligned(a.d_qkv);
 }
 

@@ -107,25 +107,31 @@ __device__ inline int32x4 make_rsrc(const void* base, uint32_t bytes) {
 // is being filled from the one that is being read), which serializes a
 // double-buffered loop inside each wave.  Callers order fills and reads
 // themselves: s_waitcnt vmcnt + a workgroup barrier before a stage is read,
-// a barrier after its last read before it is refilled.  The statement
-// overwrites M0 without declaring it (the compiler rejects M0 in a clobber
-// list): kernels that use it must not index register arrays dynamically,
-// the only other thing the compiler would use M0 for on this target.
+// a barrier after its last read before it is refilled.  The instruction takes
+// the LDS base from M0, which cannot be named as a clobber, so the statement
+// saves M0 in a scalar temporary and restores it after the load has been
+// issued (the base is read at issue): whatever the compiler keeps in M0
+// survives.
 template <int BYTES>
 __device__ inline void lds_fill(int32x4 descriptor, const void* lds, uint32_t offset) {
   static_assert(BYTES == 16 || BYTES == 4);
   const uint32_t address = __builtin_amdgcn_readfirstlane(
       static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_void*)lds)));
+  uint32_t saved_m0;
   if constexpr (BYTES == 16)
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
-                 :
-                 : "s"(address), "v"(offset), "s"(descriptor)
-                 : "memory");
+    asm volatile(
+        "s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\t"
+        "buffer_load_dwordx4 %2, %3, 0 offen lds\n\ts_mov_b32 m0, %0"
+        : "=&s"(saved_m0)
+        : "s"(address), "v"(offset), "s"(descriptor)
+        : "memory");
   else
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, 0 offen lds"
-                 :
-                 : "s"(address), "v"(offset), "s"(descriptor)
-                 : "memory");
+    asm volatile(
+        "s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\t"
+        "buffer_load_dword %2, %3, 0 offen lds\n\ts_mov_b32 m0, %0"
+        : "=&s"(saved_m0)
+        : "s"(address), "v"(offset), "s"(descriptor)
+        : "memory");
 }
 
 // LDS transpose read (ds_read_b64_tr_b16).  Within every group of 16 lanes,

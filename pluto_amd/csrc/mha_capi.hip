@@ -1,8 +1,8 @@
 // C ABI of GPT-2 style causal multi-head attention: validation and kernel
 // selection.  The layer-level contract is that of AttentionLayer
 // (src/llm/layers/attention.cc:400-596).
+#include <atomic>
 #include <cmath>
-#include <cstdlib>
 
 #include "attn_generic.h"
 #include "flash_bwd_mfma.h"
@@ -10,13 +10,14 @@
 
 namespace pluto_hip {
 
-// Test hook: PLUTO_HIP_FORCE_GENERIC=1 routes everything through the
+// Test hook (pluto_hip_test_force_generic): routes everything through the
 // any-shape FP32-arithmetic kernels so the two implementations can be checked
-// against each other on the device.
-bool force_generic() {
-  const char* value = std::getenv("PLUTO_HIP_FORCE_GENERIC");
-  return value != nullptr && value[0] == '1';
+// against each other on the device.  The one process-wide switch of the
+// library; nothing on the product path writes it.
+namespace {
+std::atomic<int> force_generic_flag{0};
 }
+bool force_generic() { return force_generic_flag.load(std::memory_order_relaxed) != 0; }
 
 namespace {
 
@@ -66,6 +67,10 @@ GenericForwardArgs packed_forward_args(int dtype, const void* qkv, int rows,
 using namespace pluto_hip;
 
 extern "C" {
+
+int pluto_hip_test_force_generic(int enabled) {
+  return force_generic_flag.exchange(enabled != 0 ? 1 : 0);
+}
 
 int pluto_hip_mha_forward(void* stream, int dtype, const void* qkv, int rows,
                           int context_length, int num_heads, int embedding_dim,

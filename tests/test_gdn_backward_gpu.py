@@ -155,11 +155,8 @@ def test_chunked_and_token_by_token_kernels_agree(capi):
         return {k: v.cpu().numpy() for k, v in named.items()}
 
     chunked = once()
-    os.environ["PLUTO_HIP_FORCE_GENERIC"] = "1"
-    try:
+    with capi.force_generic():
         sequential = once()
-    finally:
-        del os.environ["PLUTO_HIP_FORCE_GENERIC"]
     for name in sequential:
         assert_close(chunked[name], sequential[name], 2e-4, name)
 

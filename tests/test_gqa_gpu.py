@@ -266,13 +266,10 @@ def test_config3_prefill_8192(capi, oracle):
         assert np.mean(keys != want["keys"]) <= 2e-3
         np.testing.assert_array_equal(cache.token_major(cache.values)[:r1], want["values"])
     # every other row: against the any-shape FP32-arithmetic kernels
-    os.environ["PLUTO_HIP_FORCE_GENERIC"] = "1"
-    try:
+    with capi.force_generic():
         other = capi.KvCache(T, kh, d)
         out2 = capi.gqa_prefill(p, dq, dk, dv, dev(qw), dev(kw_), other)
         torch.cuda.synchronize()
-    finally:
-        del os.environ["PLUTO_HIP_FORCE_GENERIC"]
     assert torch.equal(cache.keys, other.keys) and torch.equal(cache.values, other.values)
     assert_close_bf16(got, out2.float().cpu().numpy(), "config 3 vs fp32-arithmetic kernel")
 
@@ -319,13 +316,10 @@ def test_config4_batched_decode(capi, oracle):
         want = oracle.gqa_attend(po, q, q_gate[b, :, 1], keys, vals)
         near(got[b], want, True)
     # all sequences: against the any-shape FP32-arithmetic kernels
-    os.environ["PLUTO_HIP_FORCE_GENERIC"] = "1"
-    try:
+    with capi.force_generic():
         out2 = capi.gqa_decode(p, dev(q_gate, bf), dev(k, bf), dev(v, bf), dev(qw), dev(kw_), caches,
                                split_tokens=512, advance=False)
         torch.cuda.synchronize()
-    finally:
-        del os.environ["PLUTO_HIP_FORCE_GENERIC"]
     near(got, out2.float().cpu().numpy(), True)
     # bitwise repeatable (fixed-order split-K combine)
     again = capi.gqa_decode(p, dev(q_gate, bf), dev(k, bf), dev(v, bf), dev(qw), dev(kw_), caches,

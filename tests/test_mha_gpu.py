@@ -222,13 +222,10 @@ def test_config2_gpt2_small_forward_backward_bf16(capi, oracle):
         for part, name in ((0, "dQ"), (1, "dK"), (2, "dV")):
             c = slice(part * E + head * D, part * E + (head + 1) * D)
             assert_close_bf16(g[:, c], want_g[rows, c], tag + name)
-    os.environ["PLUTO_HIP_FORCE_GENERIC"] = "1"
-    try:
+    with capi.force_generic():
         out2, m2, n2 = capi.mha_forward(xt, T, H)
         d2 = capi.mha_backward(xt, out2, gt, m2, n2, T, H)
         torch.cuda.synchronize()
-    finally:
-        del os.environ["PLUTO_HIP_FORCE_GENERIC"]
     assert_close_bf16(out.float().cpu().numpy(), out2.float().cpu().numpy(), "config 2 out vs fp32-arithmetic kernel")
     g1, g2 = d_qkv.cpu().numpy(), d2.cpu().numpy()
     for part, name in ((0, "dQ"), (1, "dK"), (2, "dV")):
