@@ -33,6 +33,7 @@ extern "C" {
 #define PLUTO_HIP_ERANGE (-2)       /* capacity exhausted (absl::ResourceExhausted) */
 #define PLUTO_HIP_EUNSUPPORTED (-3) /* not implemented (absl::Unimplemented) */
 #define PLUTO_HIP_EWORKSPACE (-4)   /* workspace missing or too small */
+#define PLUTO_HIP_ELIMIT (-5)       /* request larger than an entry point's fixed scratch */
 
 /* Storage type of an activation buffer.  The reference's DataType::FP16
  * compute policy keeps FP32 storage (src/llm/layer.h:86-88). */
@@ -282,6 +283,30 @@ int pluto_hip_gqa_decode(void* stream, const pluto_hip_attention_params* p,
                          const pluto_hip_kv_cache_view* caches, void* out,
                          float* const* probabilities, int split_tokens,
                          void* workspace, size_t workspace_bytes);
+
+/* pluto_hip_gqa_decode for callers that cannot allocate device memory or
+ * pass a workspace: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  No counterpart in the reference.  Same
+ * arguments, results and errors as pluto_hip_gqa_decode (bit for bit), but the
+ * scratch (prepared queries and split-K partial results) is a fixed array of
+ * PLUTO_HIP_GQA_DECODE_STATIC_BYTES that the library keeps on every GPU it
+ * runs on, and the call allocates nothing.  A call that would need more than
+ * that (pluto_hip_gqa_decode_workspace_bytes says how much) returns
+ * PLUTO_HIP_ELIMIT and queues nothing; the decode configuration (batch 32,
+ * contexts up to 32768, 24 query heads of 128, 512-token blocks) needs about
+ * 13 MiB.  All calls on one GPU share the array: calls that overlap there, on
+ * whatever streams, race on it.  pluto_hip_gqa_decode_static_prepare looks
+ * the array's device address up for the calling thread's current device (the
+ * entry point does it itself on its first call there). */
+#define PLUTO_HIP_GQA_DECODE_STATIC_BYTES (16u << 20)
+size_t pluto_hip_gqa_decode_static_bytes(void);
+int pluto_hip_gqa_decode_static_prepare(void);
+int pluto_hip_gqa_decode_static(void* stream, const pluto_hip_attention_params* p,
+                                int batch, int io_dtype, const void* q_gate,
+                                const void* k, const void* v, const float* q_norm,
+                                const float* k_norm, const int* positions,
+                                const pluto_hip_kv_cache_view* caches, void* out,
+                                float* const* probabilities, int split_tokens);
 
 /* ------------------------------------------------------------------------
  * Gated delta-net.

@@ -16,7 +16,7 @@ LIB_PATH = os.path.join(HERE, "libpluto_hip.so")
 F32 = 0
 BF16 = 1
 
-EINVAL, ERANGE, EUNSUPPORTED, EWORKSPACE = -1, -2, -3, -4
+EINVAL, ERANGE, EUNSUPPORTED, EWORKSPACE, ELIMIT = -1, -2, -3, -4, -5
 
 
 class PlutoHipError(RuntimeError):
@@ -108,6 +108,12 @@ SIGNATURES = {
                                   _VP, _VP, _VP, _VP, ctypes.POINTER(_I),
                                   ctypes.POINTER(KvCacheView), _VP,
                                   ctypes.POINTER(_VP), _I, _VP, _SZ]),
+    "pluto_hip_gqa_decode_static_bytes": (_SZ, []),
+    "pluto_hip_gqa_decode_static_prepare": (_I, []),
+    "pluto_hip_gqa_decode_static": (_I, [_VP, ctypes.POINTER(AttentionParams), _I, _I, _VP,
+                                         _VP, _VP, _VP, _VP, ctypes.POINTER(_I),
+                                         ctypes.POINTER(KvCacheView), _VP,
+                                         ctypes.POINTER(_VP), _I]),
     "pluto_hip_gdn_scan_workspace_bytes": (_SZ, [ctypes.POINTER(DeltaParams), _I, _I, _I]),
     "pluto_hip_gdn_scan": (_I, [_VP, ctypes.POINTER(DeltaParams), _I, _I, _I, _VP, _VP,
                                 _VP, _VP, _VP, _I, ctypes.c_float, _VP, _VP, _VP, _SZ]),
@@ -371,6 +377,20 @@ def gqa_decode(p, q_gate, k, v, q_norm, k_norm, caches, positions=None, split_to
     if advance:
         for c in caches:
             c.position += 1
+    return out
+
+
+def gqa_decode_static(p, q_gate, k, v, q_norm, k_norm, caches, positions, out, split_tokens=0,
+                      stream=None):
+    """pluto_hip_gqa_decode_static: the decode step on the library's fixed
+    scratch.  Nothing is allocated here either: the caller passes `out`."""
+    batch = q_gate.shape[0]
+    pos = (ctypes.c_int * batch)(*positions)
+    views = (KvCacheView * batch)(*[c.view() for c in caches])
+    check(lib().pluto_hip_gqa_decode_static(stream or current_stream(), ctypes.byref(p), batch,
+                                            dtype_code(q_gate), ptr(q_gate), ptr(k), ptr(v),
+                                            ptr(q_norm), ptr(k_norm), pos, views, ptr(out), None,
+                                            split_tokens))
     return out
 
 

@@ -1,15 +1,51 @@
 // C ABI of Qwen grouped-query attention: validation, workspace carving and
 // kernel selection for whole-sequence prefill and batched single-token decode.
+#include <atomic>
 #include <cmath>
 #include <limits>
+#include <mutex>
 
 #include "attn_generic.h"
 #include "flash_fwd_mfma.h"
 #include "gqa.h"
 
+// Fixed scratch of pluto_hip_gqa_decode_static: split-K partial results and
+// the prepared queries of one decode call.  Every GPU the library runs on
+// holds its own copy of the array until the process ends.  In host code the
+// array's name is only a handle for hipGetSymbolAddress: kernels and copies
+// take the per-device address kept in static_scratch_address.
+constexpr size_t kStaticScratchBytes = PLUTO_HIP_GQA_DECODE_STATIC_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 namespace pluto_hip {
 bool force_generic();  // mha_capi.hip
 namespace {
+
+constexpr int kMaxDevices = 64;
+std::atomic<void*> static_scratch_address[kMaxDevices];
+std::mutex static_scratch_mutex;
+
+// Device address of `scratch` on the calling thread's current device, looked
+// up once per device.
+int static_scratch(void** address) {
+  int device = 0;
+  hipError_t error = hipGetDevice(&device);
+  if (error != hipSuccess) return static_cast<int>(error);
+  if (device < 0 || device >= kMaxDevices) return PLUTO_HIP_EUNSUPPORTED;
+  void* known = static_scratch_address[device].load(std::memory_order_acquire);
+  if (!known) {
+    std::lock_guard<std::mutex> lock(static_scratch_mutex);
+    known = static_scratch_address[device].load(std::memory_order_relaxed);
+    if (!known) {
+      error = hipGetSymbolAddress(&known, HIP_SYMBOL(scratch));
+      if (error != hipSuccess) return static_cast<int>(error);
+      if (!known) return static_cast<int>(hipErrorInvalidSymbol);
+      static_scratch_address[device].store(known, std::memory_order_release);
+    }
+  }
+  *address = known;
+  return 0;
+}
 
 // ValidateCachedAttention, parameter part (cached_attention_ops.cc:286-297).
 int validate_params(const pluto_hip_attention_params* p) {
@@ -406,12 +442,12 @@ size_t pluto_hip_gqa_decode_workspace_bytes(const pluto_hip_attention_params* p,
   return bytes;
 }
 
-int pluto_hip_gqa_decode(void* stream, const pluto_hip_attention_params* p, int batch,
-                         int io_dtype, const void* q_gate, const void* k, const void* v,
-                         const float* q_norm, const float* k_norm, const int* positions,
-                         const pluto_hip_kv_cache_view* caches, void* out,
-                         float* const* probabilities, int split_tokens, void* workspace,
-                         size_t workspace_bytes) {
+// Argument checks of the decode entry points; everything is rejected before
+// any work is queued.
+static int decode_check(const pluto_hip_attention_params* p, int batch, int io_dtype,
+                        const void* q_gate, const void* k, const void* v, const float* q_norm,
+                        const float* k_norm, const int* positions,
+                        const pluto_hip_kv_cache_view* caches, const void* out, int split) {
   int status = validate_params(p);
   if (status != 0) return status;
   if (batch <= 0 || (io_dtype != PLUTO_HIP_F32 && io_dtype != PLUTO_HIP_BF16))
@@ -419,7 +455,6 @@ int pluto_hip_gqa_decode(void* stream, const pluto_hip_attention_params* p, int 
   // cached_attention_ops.cc:314-317: null pointers are rejected before any work.
   if (!q_gate || !k || !v || !q_norm || !k_norm || !out || !positions || !caches)
     return PLUTO_HIP_EINVAL;
-  const int split = split_or_default(split_tokens);
   if (split < 64 || split > 512 || split % 64 != 0) return PLUTO_HIP_EINVAL;
   for (int b = 0; b < batch; ++b) {
     status = validate_cache(&caches[b], p);
@@ -431,22 +466,76 @@ int pluto_hip_gqa_decode(void* stream, const pluto_hip_attention_params* p, int 
   }
   for (int b = 0; b < batch; ++b)  // cached_attention_ops.cc:318-320
     if (positions[b] >= p->capacity) return PLUTO_HIP_ERANGE;
+  return 0;
+}
+
+static int decode_run(void* stream, const pluto_hip_attention_params* p, int batch, int io_dtype,
+                      const void* q_gate, const void* k, const void* v, const float* q_norm,
+                      const float* k_norm, const int* positions,
+                      const pluto_hip_kv_cache_view* caches, void* out,
+                      float* const* probabilities, int split, void* workspace);
+
+int pluto_hip_gqa_decode(void* stream, const pluto_hip_attention_params* p, int batch,
+                         int io_dtype, const void* q_gate, const void* k, const void* v,
+                         const float* q_norm, const float* k_norm, const int* positions,
+                         const pluto_hip_kv_cache_view* caches, void* out,
+                         float* const* probabilities, int split_tokens, void* workspace,
+                         size_t workspace_bytes) {
+  const int split = split_or_default(split_tokens);
+  const int status =
+      decode_check(p, batch, io_dtype, q_gate, k, v, q_norm, k_norm, positions, caches, out, split);
+  if (status != 0) return status;
   const size_t needed = pluto_hip_gqa_decode_workspace_bytes(p, batch, positions, split);
   if (!workspace || workspace_bytes < needed) return PLUTO_HIP_EWORKSPACE;
+  return decode_run(stream, p, batch, io_dtype, q_gate, k, v, q_norm, k_norm, positions, caches,
+                    out, probabilities, split, workspace);
+}
 
+size_t pluto_hip_gqa_decode_static_bytes(void) { return kStaticScratchBytes; }
+
+int pluto_hip_gqa_decode_static_prepare(void) {
+  void* address = nullptr;
+  return static_scratch(&address);
+}
+
+int pluto_hip_gqa_decode_static(void* stream, const pluto_hip_attention_params* p, int batch,
+                                int io_dtype, const void* q_gate, const void* k, const void* v,
+                                const float* q_norm, const float* k_norm, const int* positions,
+                                const pluto_hip_kv_cache_view* caches, void* out,
+                                float* const* probabilities, int split_tokens) {
+  const int split = split_or_default(split_tokens);
+  int status =
+      decode_check(p, batch, io_dtype, q_gate, k, v, q_norm, k_norm, positions, caches, out, split);
+  if (status != 0) return status;
+  const size_t needed = pluto_hip_gqa_decode_workspace_bytes(p, batch, positions, split);
+  if (needed == 0) return PLUTO_HIP_EINVAL;
+  if (needed > kStaticScratchBytes) return PLUTO_HIP_ELIMIT;
+  void* address = nullptr;
+  status = static_scratch(&address);
+  if (status != 0) return status;
+  return decode_run(stream, p, batch, io_dtype, q_gate, k, v, q_norm, k_norm, positions, caches,
+                    out, probabilities, split, address);
+}
+
+static int decode_run(void* stream, const pluto_hip_attention_params* p, int batch, int io_dtype,
+                      const void* q_gate, const void* k, const void* v, const float* q_norm,
+                      const float* k_norm, const int* positions,
+                      const pluto_hip_kv_cache_view* caches, void* out,
+                      float* const* probabilities, int split, void* workspace) {
+  int status = 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int qh = p->query_heads, kh = p->key_value_heads, d = p->head_dim;
   const int group = qh / kh;
   const bool round = p->round_to_bfloat16 != 0;
   const long long blocks = decode_blocks(batch, positions, split);
-  char* scratch = static_cast<char*>(workspace);
-  void* queries = scratch;
+  char* area = static_cast<char*>(workspace);
+  void* queries = area;
   size_t offset = align_up(static_cast<size_t>(batch) * qh * d * 4, 256);
-  float* part_o = reinterpret_cast<float*>(scratch + offset);
+  float* part_o = reinterpret_cast<float*>(area + offset);
   offset += align_up(static_cast<size_t>(blocks) * qh * d * 4, 256);
-  float* part_m = reinterpret_cast<float*>(scratch + offset);
+  float* part_m = reinterpret_cast<float*>(area + offset);
   offset += align_up(static_cast<size_t>(blocks) * qh * 4, 256);
-  float* part_l = reinterpret_cast<float*>(scratch + offset);
+  float* part_l = reinterpret_cast<float*>(area + offset);
 
   const pluto_hip_kv_cache_view& c0 = caches[0];
   bool fast = round && c0.dtype == PLUTO_HIP_BF16 && decode_fast_supported(d, group) &&

@@ -41,23 +41,24 @@ constexpr size_t kPinnedCacheLimit = 64ull << 20;  // executor.cc:90-95
 const char* const kNegativeNames[] = {"PLUTO_HIP_OK", "PLUTO_HIP_EINVAL",
                                       "PLUTO_HIP_ERANGE",
                                       "PLUTO_HIP_EUNSUPPORTED",
-                                      "PLUTO_HIP_EWORKSPACE"};
+                                      "PLUTO_HIP_EWORKSPACE", "PLUTO_HIP_ELIMIT"};
 const char* const kNegativeStrings[] = {
     "success", "invalid argument", "capacity exhausted",
-    "unsupported configuration", "workspace missing or too small"};
+    "unsupported configuration", "workspace missing or too small",
+    "request larger than the fixed scratch of this entry point"};
 
 }  // namespace
 
 extern "C" {
 
 const char* pluto_hip_error_name(int code) {
-  if (code <= 0 && code >= -4) return kNegativeNames[-code];
+  if (code <= 0 && code >= -5) return kNegativeNames[-code];
   if (code > 0) return hipGetErrorName(static_cast<hipError_t>(code));
   return "PLUTO_HIP_EUNKNOWN";
 }
 
 const char* pluto_hip_error_string(int code) {
-  if (code <= 0 && code >= -4) return kNegativeStrings[-code];
+  if (code <= 0 && code >= -5) return kNegativeStrings[-code];
   if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
   return "unknown error code";
 }
