@@ -4,16 +4,22 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
 
 A step is one pass of the hot path over one batch of synthetic input that is
-already resident in HBM when the timed region starts.  The default workload is
-the configuration the headline metric is quoted on: GPT-2-small causal
-attention forward+backward, bf16 storage with fp32 accumulation, B=16, T=1024,
-H=12, D=64.  The other configurations of the path can be selected with
---workload; --workload all appends their figures under "workloads".
+already resident in HBM when the timed region starts.  The headline workload
+is the configuration the metric is quoted on: GPT-2-small causal attention
+forward+backward, bf16 storage with fp32 accumulation, B=16, T=1024, H=12,
+D=64.  The default run (--workload all) appends the other four configurations
+of the path under "workloads", each with its own `roofline` and
+`cpu_baseline`; --workload NAME runs one workload alone.
 
-Exactly one JSON line is printed.  `roofline` describes the dominant kernel
-group of the step (its own average duration is measured with HIP events on
-the launch stream); `cpu_baseline` is the scalar CPU oracle timed on this
-host on a bounded sample of the same workload (a reported baseline only).
+Exactly one JSON line is printed.  `roofline` describes the kernel of the
+step that takes longest: its average duration is measured live with HIP
+events on the launch stream around calls that queue only that kernel (the
+library's measurement hook switches the other kernels of the call off after
+a complete step has filled every buffer), `achieved` is the kernel's
+algorithmic work divided by that duration.  `cpu_baseline` is the scalar CPU
+oracle timed on this host on a bounded sample of the same workload, on one
+thread as the reference runs it (`value`, `cores` 1) and on `threads.cores`
+threads over independent units (a reported baseline only).
 """
 import argparse
 import json
@@ -35,11 +41,10 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E (published)
 # the factors a 1 GiB device copy gives: `--workload copy`).  The summaries are
 # kept as profiles/*_hbm_traffic.md.  None = not measured.
 MEASURED_TRAFFIC_BYTES = {
-    ("mha_train_bf16", "forward"): 126.4e6,
-    ("mha_train_bf16", "backward"): 548.6e6,
-    ("gqa_prefill", "prefill"): 538.6e6,
-    ("gqa_decode", "decode"): 1055.9e6,
-    ("gdn_scan", "scan"): 2105.3e6,
+    ("mha_train_bf16", "flash_forward_kernel<64>"): 126.4e6,
+    ("gqa_prefill", "flash_forward_kernel<128>"): 347.7e6 + 50.3e6,
+    ("gqa_decode", "decode_split_kernel<128,6>"): 1028.3e6 + 12.6e6,
+    ("gdn_scan", "gdn_chunk_prepare + gdn_chunk_scan"): 2105.3e6,
 }
 
 NAMES = ["mha_train_bf16", "mha_fwd_fp32", "gqa_prefill", "gqa_decode", "gdn_scan"]
@@ -54,7 +59,9 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="mha_train_bf16", choices=NAMES + EXTRA + ["all"])
+    ap.add_argument("--workload", default="all", choices=NAMES + EXTRA + ["all"])
+    ap.add_argument("--cpu-seconds", type=float, default=5.0,
+                    help="CPU time budget of each cpu_baseline leg")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     return ap.parse_args()
 
@@ -86,7 +93,7 @@ def mha_train_bf16(torch, capi):
     state = {}
 
     def forward():
-        state["fwd"] = capi.mha_forward(qkv, T, H)
+        state["fwd"] = capi.mha_forward(qkv, T, H, into=state.get("fwd"))
 
     def backward():
         out, maxima, normalizers = state["fwd"]
@@ -98,7 +105,13 @@ def mha_train_bf16(torch, capi):
 
     fwd = 4.0 * B * H * D * causal_pairs(T)
     bwd = 10.0 * B * H * D * causal_pairs(T)
-    return dict(step=step, parts=[("forward", forward, fwd), ("backward", backward, bwd)],
+    # The backward is two kernels that both recompute the scores and dP: the
+    # query-owned one executes 3 products (S, dP, dQ), the key-owned one 4 (S,
+    # dP, dK, dV).  The 5 counted products are shared out in that proportion.
+    return dict(step=step,
+                kernels=[("flash_forward_kernel<64>", forward, None, fwd),
+                         ("flash_dq_kernel<64>", backward, capi.QUERY_KERNEL, bwd * 3 / 7),
+                         ("flash_dkv_kernel<64>", backward, capi.MAIN_KERNEL, bwd * 4 / 7)],
                 work=fwd + bwd, metric="attention_fwd_bwd_tflops", unit="TFLOP/s", dtype="bf16",
                 bound="mfma", peak=PEAK_BF16_TFLOPS,
                 config={"workload": "gpt2_small_causal_mha_fwd_bwd", "batch": B, "seq_len": T,
@@ -112,11 +125,13 @@ def mha_fwd_fp32(torch, capi):
     gen = torch.Generator(device="cuda").manual_seed(0)
     qkv = torch.randn((B * T, 3 * E), generator=gen, device="cuda")
 
+    state = {}
+
     def forward():
-        capi.mha_forward(qkv, T, H)
+        state["fwd"] = capi.mha_forward(qkv, T, H, into=state.get("fwd"))
 
     work = 4.0 * B * H * D * causal_pairs(T)
-    return dict(step=forward, parts=[("forward", forward, work)], work=work,
+    return dict(step=forward, kernels=[("f32_forward_kernel<64>", forward, None, work)], work=work,
                 metric="attention_fwd_tflops", unit="TFLOP/s", dtype="f32", bound="mfma",
                 peak=PEAK_FP32_TFLOPS,
                 config={"workload": "gpt2_small_causal_mha_fwd_fp32", "batch": B, "seq_len": T,
@@ -136,17 +151,23 @@ def gqa_prefill(torch, capi):
     qw = torch.from_numpy(values(np, d, 0.2, 0.3)).cuda()
     kw = torch.from_numpy(values(np, d, 0.8, 0.4)).cuda()
     cache = capi.KvCache(T, kh, d)
+    out = torch.empty((T, qh, d), dtype=bf, device="cuda")
+    size = capi.lib().pluto_hip_gqa_prefill_workspace_bytes(p, T)
+    workspace = torch.empty(size, dtype=torch.uint8, device="cuda")
 
     def step():
-        capi.gqa_prefill(p, qg, k, v, qw, kw, cache)
+        capi.gqa_prefill(p, qg, k, v, qw, kw, cache, out=out, workspace=workspace)
 
     work = 4.0 * qh * d * causal_pairs(T)
-    return dict(step=step, parts=[("prefill", step, work)], work=work,
+    return dict(step=step,
+                kernels=[("flash_forward_kernel<128>", step, capi.MAIN_KERNEL, work),
+                         ("rope table + prepare", step, capi.AUXILIARY_KERNELS, None)],
+                work=work,
                 metric="gqa_prefill_tflops", unit="TFLOP/s", dtype="bf16", bound="mfma",
                 peak=PEAK_BF16_TFLOPS,
                 config={"workload": "qwen_gqa_prefill", "batch": 1, "seq_len": T, "query_heads": qh,
                         "kv_heads": kh, "head_dim": d, "kv_cache": "bf16 [1,4,8192,128], written by the call"},
-                cpu=None)
+                cpu=("gqa_prefill", dict(T=T, qh=qh, kh=kh, d=d)))
 
 
 def gqa_prefill_bwd(torch, capi):
@@ -174,7 +195,7 @@ def gqa_prefill_bwd(torch, capi):
         capi.gqa_prefill_backward(p, qg, k, v, qw, kw, dy, saved=saved)
 
     work = 10.0 * qh * d * causal_pairs(T)
-    return dict(step=step, parts=[("backward", step, work)], work=work,
+    return dict(step=step, kernels=[("whole call", step, None, work)], work=work,
                 metric="gqa_sequence_backward_tflops", unit="TFLOP/s", dtype="bf16", bound="mfma",
                 peak=PEAK_BF16_TFLOPS,
                 config={"workload": "qwen_gqa_sequence_backward", "batch": 1, "seq_len": T,
@@ -215,7 +236,7 @@ def gdn_layer_bwd(torch, capi):
     # recurrence form, per token, head and state element: 7 FLOPs to repeat the
     # forward (decay, prediction, update, output) and 15 for the reverse sweep
     work = 22.0 * B * T * H * dk * dv
-    return dict(step=step, parts=[("backward", step, work)], work=work,
+    return dict(step=step, kernels=[("whole call", step, None, work)], work=work,
                 metric="gdn_layer_backward_tflops", unit="TFLOP/s", dtype="f32", bound="mfma",
                 peak=PEAK_FP32_TFLOPS,
                 config={"workload": "gated_delta_net_layer_backward", "batch": B, "seq_len": T,
@@ -253,13 +274,16 @@ def gqa_decode(torch, capi):
                         workspace=workspace, out=out, advance=False)
 
     work = 2.0 * kh * d * 2 * float(lengths.sum())   # K and V bytes of the valid prefix
-    return dict(step=step, parts=[("decode", step, work)], work=work,
+    return dict(step=step,
+                kernels=[("decode_split_kernel<128,6>", step, capi.MAIN_KERNEL, work),
+                         ("prepare + combine", step, capi.AUXILIARY_KERNELS, None)],
+                work=work,
                 metric="gqa_decode_hbm_gbs", unit="GB/s", dtype="bf16", bound="hbm",
                 peak=PEAK_HBM_GBS,
                 config={"workload": "qwen_gqa_decode", "batch": batch, "sum_context": int(lengths.sum()),
                         "query_heads": qh, "kv_heads": kh, "head_dim": d, "split_tokens": 512,
                         "kv_cache": "bf16 head-major"},
-                cpu=None)
+                cpu=("gqa_decode", dict(lengths=[int(L) for L in lengths], qh=qh, kh=kh, d=d)))
 
 
 def gdn_scan(torch, capi):
@@ -277,18 +301,23 @@ def gdn_scan(torch, capi):
     out = torch.empty((B, T, H, dv), dtype=bf, device="cuda")
     scale = 1.0 / math.sqrt(dk)
 
-    def step():
-        state.zero_()
+    def scan():
         capi.gdn_scan(p, q, k, v, g, beta, state, q_scale=scale, chunk=64, workspace=workspace,
                       out=out)
 
+    def step():
+        state.zero_()
+        scan()
+
     work = B * T * H * (2 * dk + 2 * dv) * 2.0 + 2.0 * B * T * H * 4 + B * H * dk * dv * 4.0
-    return dict(step=step, parts=[("scan", step, work)], work=work,
+    return dict(step=step,
+                kernels=[("gdn_chunk_prepare + gdn_chunk_scan", scan, None, work)],
+                work=work,
                 metric="gated_delta_scan_hbm_gbs", unit="GB/s", dtype="bf16", bound="hbm",
                 peak=PEAK_HBM_GBS,
                 config={"workload": "gated_delta_net_chunked_scan", "batch": B, "seq_len": T,
                         "heads": H, "d_k": dk, "d_v": dv, "chunk": 64, "state": "fp32"},
-                cpu=None)
+                cpu=("gdn_scan", dict(T=T, H=H, dk=dk, dv=dv)))
 
 
 def gdn_decode(torch, capi):
@@ -314,7 +343,7 @@ def gdn_decode(torch, capi):
 
     # every recurrent state is read and written once; so is every convolution state
     work = 2.0 * batch * (H * dk * dv + channels * K) * 4
-    return dict(step=step, parts=[("step", step, work)], work=work,
+    return dict(step=step, kernels=[("whole call", step, None, work)], work=work,
                 metric="gdn_decode_step_hbm_gbs", unit="GB/s", dtype="f32", bound="hbm",
                 peak=PEAK_HBM_GBS,
                 config={"workload": "gated_delta_net_decode_step", "batch": batch, "heads": H,
@@ -346,7 +375,8 @@ def dense_qkv(torch, capi):
         backward()
 
     product = 2.0 * rows * n_in * n_out
-    return dict(step=step, parts=[("forward", forward, product), ("backward", backward, 2 * product)],
+    return dict(step=step, kernels=[("forward", forward, None, product),
+                                    ("backward", backward, None, 2 * product)],
                 work=3 * product, metric="dense_fwd_bwd_tflops", unit="TFLOP/s", dtype="bf16",
                 bound="mfma", peak=PEAK_BF16_TFLOPS,
                 config={"workload": "gpt2_small_qkv_projection_fwd_bwd", "rows": rows,
@@ -375,7 +405,7 @@ def dense_imported(torch, capi):
         capi.dense_imported_forward(capi.MATRIX_FP8_E4M3, weights, scales, x, workspace, out)
 
     work = float(n_in * n_out + scales.numel() * 4 + n_in * 2 + n_out * 2)
-    return dict(step=step, parts=[("projection", step, work)], work=work,
+    return dict(step=step, kernels=[("whole call", step, None, work)], work=work,
                 metric="imported_projection_gbs", unit="GB/s", dtype="f32", bound="hbm",
                 peak=PEAK_HBM_GBS,
                 config={"workload": "qwen_imported_fp8_projection_one_token", "input_dim": n_in,
@@ -392,7 +422,7 @@ def copy(torch, capi):
         dst.copy_(src)
 
     work = 2.0 * n * 4
-    return dict(step=step, parts=[("copy", step, work)], work=work, metric="device_copy_gbs",
+    return dict(step=step, kernels=[("copy", step, None, work)], work=work, metric="device_copy_gbs",
                 unit="GB/s", dtype="f32", bound="hbm", peak=PEAK_HBM_GBS,
                 config={"workload": "device_copy_calibration", "bytes_read": n * 4,
                         "bytes_written": n * 4}, cpu=None)
@@ -404,9 +434,13 @@ WORKLOADS = {"copy": copy, "gdn_decode": gdn_decode, "dense_qkv": dense_qkv, "de
              "gdn_scan": gdn_scan}
 
 
-def cpu_baseline_mha(spec):
-    """Scalar CPU oracle (one thread) on whole (sequence, head) units of the same
-    workload; the rate is per unit of algorithmic work, so it needs no scaling."""
+# --------------------------------------------------------------------------
+# CPU baseline: the scalar oracle on independent units of the same workload.
+# Each maker returns (run_unit(i) -> algorithmic work of that unit, number of
+# units, description of a unit).
+# --------------------------------------------------------------------------
+
+def cpu_units_mha(spec):
     import numpy as np
     from oracle import pyoracle as oracle
     B, T, H, D = spec["B"], spec["T"], spec["H"], spec["D"]
@@ -416,21 +450,130 @@ def cpu_baseline_mha(spec):
     d_out = rng.standard_normal((T, E)).astype(np.float32)
     dtype = oracle.BF16 if spec["bf16"] else oracle.F32
     data = oracle.f32_to_bf16_bits(x).reshape(x.shape) if spec["bf16"] else x
-    units, seconds = 0, 0.0
-    while seconds < 10.0 and units < H:
-        t0 = time.perf_counter()
-        out, _, _ = oracle.mha_fwd(data, T, H, dtype, (0, 1), (units, units + 1))
+    work = (14.0 if spec["backward"] else 4.0) * D * causal_pairs(T)
+
+    def run(i):
+        head = i % H
+        out, _, _ = oracle.mha_fwd(data, T, H, dtype, (0, 1), (head, head + 1))
         if spec["backward"]:
-            oracle.mha_bwd(data, out, d_out, T, H, dtype, (0, 1), (units, units + 1))
-        seconds += time.perf_counter() - t0
-        units += 1
-    flops = (14.0 if spec["backward"] else 4.0) * D * causal_pairs(T) * units
-    return dict(value=round(flops / seconds / 1e12, 6), unit="TFLOP/s", cores=1, kind="port",
-                sample="%d of %d (sequence, head) units of the workload, %s, %.1f s of CPU time" % (
-                    units, B * H, "forward+backward" if spec["backward"] else "forward", seconds))
+            oracle.mha_bwd(data, out, d_out, T, H, dtype, (0, 1), (head, head + 1))
+        return work
+
+    return run, B * H, "(sequence, head) units, %s" % (
+        "forward+backward" if spec["backward"] else "forward")
 
 
-def measure(torch, w, steps, warmup):
+def cpu_units_gqa_prefill(spec):
+    import numpy as np
+    from oracle import pyoracle as oracle
+    T, qh, kh, d = spec["T"], spec["qh"], spec["kh"], spec["d"]
+    po = oracle.attention_params(qh, kh, d, 32, capacity=T)
+    rng = np.random.default_rng(2)
+    qg = oracle.bf16_round((0.5 * rng.standard_normal((T, qh, 2, d))).astype(np.float32))
+    k = oracle.bf16_round((0.5 * rng.standard_normal((T, kh, d))).astype(np.float32))
+    v = oracle.bf16_round((0.5 * rng.standard_normal((T, kh, d))).astype(np.float32))
+    qw, kw = values(np, d, 0.2, 0.3), values(np, d, 0.8, 0.4)
+    rows = 32   # query rows per unit, taken from evenly spread places of the sequence
+    blocks = T // rows
+
+    def run(i):
+        head = i % qh
+        block = (i * 37 + 11) % blocks
+        r0 = block * rows
+        oracle.gqa_sequence(po, qg, k, v, qw, kw, rows=(r0, r0 + rows), heads=(head, head + 1))
+        return 4.0 * d * sum(r + 1 for r in range(r0, r0 + rows))
+
+    return run, blocks * qh, "(head, %d query rows) units" % rows
+
+
+def cpu_units_gqa_decode(spec):
+    import numpy as np
+    from oracle import pyoracle as oracle
+    lengths, qh, kh, d = spec["lengths"], spec["qh"], spec["kh"], spec["d"]
+    po = oracle.attention_params(qh, kh, d, 32, capacity=max(lengths))
+    rng = np.random.default_rng(3)
+    longest = max(lengths)
+    keys = oracle.bf16_round(rng.standard_normal((kh, longest, d)).astype(np.float32))
+    vals = oracle.bf16_round(rng.standard_normal((kh, longest, d)).astype(np.float32))
+    q = oracle.bf16_round(rng.standard_normal((qh, d)).astype(np.float32))
+    gate = oracle.bf16_round(rng.standard_normal((qh, d)).astype(np.float32))
+
+    def run(i):
+        L = lengths[i % len(lengths)]
+        oracle.gqa_attend(po, q, gate, np.ascontiguousarray(keys[:, :L]),
+                          np.ascontiguousarray(vals[:, :L]))
+        return 2.0 * kh * d * 2 * L
+
+    return run, len(lengths), "sequences (attention over the cached rows, all heads)"
+
+
+def cpu_units_gdn_scan(spec):
+    import numpy as np
+    from oracle import pyoracle as oracle
+    T, H, dk, dv = spec["T"], spec["H"], spec["dk"], spec["dv"]
+    tokens = 2048   # tokens per unit: the first `tokens` of one head's chain
+    po = oracle.delta_params(H, H, dk, dv)
+    rng = np.random.default_rng(4)
+
+    def unit(x):
+        return x / np.sqrt((x * x).sum(-1, keepdims=True))
+
+    q = oracle.bf16_round(unit(rng.standard_normal((tokens, H, dk))).astype(np.float32))
+    k = oracle.bf16_round(unit(rng.standard_normal((tokens, H, dk))).astype(np.float32))
+    v = oracle.bf16_round(rng.standard_normal((tokens, H, dv)).astype(np.float32))
+    beta = (1.0 / (1.0 + np.exp(-rng.standard_normal((tokens, H))))).astype(np.float32)
+    g = (-np.log1p(np.exp(rng.standard_normal((tokens, H))))).astype(np.float32)
+    scale = 1.0 / math.sqrt(dk)
+    per_token = (2 * dk + 2 * dv) * 2.0 + 8.0
+
+    def run(i):
+        head = i % H
+        oracle.gdn_scan(po, q, k, v, g, beta, False, scale, heads=(head, head + 1))
+        return per_token * tokens
+
+    return run, 2 * H * (T // tokens), "(head, %d tokens) units of a chain" % tokens
+
+
+CPU_UNITS = {"mha": cpu_units_mha, "gqa_prefill": cpu_units_gqa_prefill,
+             "gqa_decode": cpu_units_gqa_decode, "gdn_scan": cpu_units_gdn_scan}
+
+
+def cpu_baseline(kind, spec, bound, budget):
+    """One thread (as the reference runs), then `threads` threads over
+    independent units (the oracle's C code runs outside the interpreter lock).
+    Rates are per unit of algorithmic work, so a sample needs no scaling."""
+    import concurrent.futures
+    run, total, what = CPU_UNITS[kind](spec)
+    divisor = 1e12 if bound == "mfma" else 1e9
+    unit = "TFLOP/s" if bound == "mfma" else "GB/s"
+    done, work, t0 = 0, 0.0, time.perf_counter()
+    while done < total and time.perf_counter() - t0 < budget:
+        work += run(done)
+        done += 1
+    seconds = time.perf_counter() - t0
+    threads = max(1, min(16, os.cpu_count() or 1))
+
+    def worker(first):
+        mine, i = 0.0, first
+        start = time.perf_counter()
+        while i < total and time.perf_counter() - start < budget:
+            mine += run(i)
+            i += threads
+        return mine, (i - first) // threads
+
+    t1 = time.perf_counter()
+    with concurrent.futures.ThreadPoolExecutor(max_workers=threads) as pool:
+        results = list(pool.map(worker, range(threads)))
+    wall = time.perf_counter() - t1
+    many_work = sum(r[0] for r in results)
+    many_units = sum(r[1] for r in results)
+    return dict(value=float("%.4g" % (work / seconds / divisor)), unit=unit, cores=1, kind="port",
+                sample="%d of %d %s of the workload in %.1f s" % (done, total, what, seconds),
+                threads=dict(cores=threads, value=float("%.4g" % (many_work / wall / divisor)),
+                             sample="%d units in %.1f s" % (many_units, wall)))
+
+
+def measure(torch, capi, w, steps, warmup):
     stream = torch.cuda.current_stream()
     for _ in range(warmup):
         w["step"]()
@@ -440,25 +583,41 @@ def measure(torch, w, steps, warmup):
         w["step"]()
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / steps
-    parts = {}
-    for name, fn, work in w["parts"]:
+    # Every buffer now holds what a complete step leaves, so any one kernel of
+    # the step can run alone on valid inputs.
+    kernels = {}
+    for name, fn, mask, work in w["kernels"]:
         pairs = []
-        for _ in range(steps):
-            start = torch.cuda.Event(enable_timing=True)
-            end = torch.cuda.Event(enable_timing=True)
-            start.record(stream)
+        with capi.only_kernels(0xffffffff if mask is None else mask):
             fn()
-            end.record(stream)
-            pairs.append((start, end))
-        torch.cuda.synchronize()
-        parts[name] = (sum(s.elapsed_time(e) for s, e in pairs) / len(pairs), work)
-    dominant = max(parts, key=lambda k: parts[k][0])
-    dom_ms, dom_work = parts[dominant]
+            torch.cuda.synchronize()
+            for _ in range(steps):
+                start = torch.cuda.Event(enable_timing=True)
+                end = torch.cuda.Event(enable_timing=True)
+                start.record(stream)
+                fn()
+                end.record(stream)
+                pairs.append((start, end))
+            torch.cuda.synchronize()
+        kernels[name] = (sum(s.elapsed_time(e) for s, e in pairs) / len(pairs), work)
+    w["step"]()   # leave complete results behind
+    torch.cuda.synchronize()
+    counted = {k: v for k, v in kernels.items() if v[1] is not None}
+    dominant = max(counted, key=lambda k: counted[k][0])
+    dom_ms, dom_work = counted[dominant]
     divisor = 1e12 if w["bound"] == "mfma" else 1e9
     value = w["work"] / (ms_per_step * 1e-3) / divisor
     achieved = dom_work / (dom_ms * 1e-3) / divisor
-    return dict(ms_per_step=ms_per_step, value=value, parts=parts, dominant=dominant,
+    return dict(ms_per_step=ms_per_step, value=value, kernels=kernels, dominant=dominant,
                 achieved=achieved, kernel_ms=dom_ms)
+
+
+def roofline(name, w, m):
+    return {"bound": w["bound"], "kernel": m["dominant"], "achieved": round(m["achieved"], 3),
+            "peak": w["peak"], "unit": "TFLOP/s" if w["bound"] == "mfma" else "GB/s",
+            "frac": round(m["achieved"] / w["peak"], 4),
+            "traffic": MEASURED_TRAFFIC_BYTES.get((name, m["dominant"])),
+            "kernel_ms": round(m["kernel_ms"], 4)}
 
 
 def main():
@@ -474,22 +633,17 @@ def main():
     capi.lib()
     head = "mha_train_bf16" if args.workload == "all" else args.workload
     w = WORKLOADS[head](torch, capi)
-    m = measure(torch, w, args.steps, args.warmup)
+    m = measure(torch, capi, w, args.steps, args.warmup)
     result = {
         "metric": w["metric"], "value": round(m["value"], 3), "unit": w["unit"], "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(m["ms_per_step"], 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": w["dtype"], "data": "synthetic", "config": w["config"],
-        "roofline": {"bound": w["bound"], "kernel": m["dominant"],
-                     "achieved": round(m["achieved"], 3), "peak": w["peak"],
-                     "unit": "TFLOP/s" if w["bound"] == "mfma" else "GB/s",
-                     "frac": round(m["achieved"] / w["peak"], 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get((head, m["dominant"])),
-                     "kernel_ms": round(m["kernel_ms"], 4)},
-        "parts_ms": {k: round(v[0], 4) for k, v in m["parts"].items()},
+        "roofline": roofline(head, w, m),
+        "kernels_ms": {k: round(v[0], 4) for k, v in m["kernels"].items()},
     }
     if not args.no_cpu_baseline and w["cpu"] is not None:
-        result["cpu_baseline"] = cpu_baseline_mha(w["cpu"][1])
+        result["cpu_baseline"] = cpu_baseline(w["cpu"][0], w["cpu"][1], w["bound"], args.cpu_seconds)
     if args.workload == "all":
         others = {}
         for name in NAMES:
@@ -498,10 +652,14 @@ def main():
             del w
             torch.cuda.empty_cache()
             w = WORKLOADS[name](torch, capi)
-            mm = measure(torch, w, max(args.steps // 2, 5), max(args.warmup // 2, 2))
+            mm = measure(torch, capi, w, args.steps, args.warmup)
             others[name] = {"metric": w["metric"], "value": round(mm["value"], 3), "unit": w["unit"],
-                            "ms_per_step": round(mm["ms_per_step"], 4), "bound": w["bound"],
-                            "frac_of_peak": round(mm["value"] / w["peak"], 4), "config": w["config"]}
+                            "ms_per_step": round(mm["ms_per_step"], 4), "dtype": w["dtype"],
+                            "config": w["config"], "roofline": roofline(name, w, mm),
+                            "kernels_ms": {k: round(v[0], 4) for k, v in mm["kernels"].items()}}
+            if not args.no_cpu_baseline and w["cpu"] is not None:
+                others[name]["cpu_baseline"] = cpu_baseline(w["cpu"][0], w["cpu"][1], w["bound"],
+                                                            args.cpu_seconds)
         result["workloads"] = others
     print(json.dumps(result))
 

@@ -516,6 +516,16 @@ int pluto_hip_dense_imported_forward_batch(void* stream, int storage,
  * process-wide state of the library; nothing else writes it. */
 int pluto_hip_test_force_generic(int enabled);
 
+/* Measurement hook: entry points that queue several kernels skip those whose
+ * class bit is cleared in `mask` (1 = the kernel that bounds the call: flash
+ * attention forward, key-owned attention backward, split-K decode, delta-net
+ * scan; 2 = the query-owned attention backward kernel; 4 = auxiliary kernels:
+ * preparation, tables, combines).  A benchmark runs the whole call once, then
+ * times one class with events around the call.  Returns the previous mask;
+ * the default, ~0u, runs everything.  Process-wide like the switch above, and
+ * like it written by nothing on the product path. */
+unsigned pluto_hip_test_kernel_classes(unsigned mask);
+
 #ifdef __cplusplus
 }
 #endif

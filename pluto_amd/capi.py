@@ -69,6 +69,7 @@ SIGNATURES = {
     "pluto_hip_error_name": (ctypes.c_char_p, [_I]),
     "pluto_hip_error_string": (ctypes.c_char_p, [_I]),
     "pluto_hip_test_force_generic": (_I, [_I]),
+    "pluto_hip_test_kernel_classes": (ctypes.c_uint, [ctypes.c_uint]),
     "pluto_hip_abi_version": (_I, []),
     "pluto_hip_target_arch": (ctypes.c_char_p, []),
     "pluto_hip_executor_create": (_I, [ctypes.POINTER(_VP)]),
@@ -172,6 +173,24 @@ class force_generic:
         return False
 
 
+MAIN_KERNEL, QUERY_KERNEL, AUXILIARY_KERNELS = 1, 2, 4
+
+
+class only_kernels:
+    """Context manager around the library's measurement hook: inside it the
+    multi-launch entry points queue only the kernel classes in `mask`."""
+
+    def __init__(self, mask):
+        self.mask = mask
+
+    def __enter__(self):
+        self.previous = lib().pluto_hip_test_kernel_classes(self.mask)
+
+    def __exit__(self, *exc):
+        lib().pluto_hip_test_kernel_classes(self.previous)
+        return False
+
+
 def check(code):
     if code != 0:
         l = lib()
@@ -197,16 +216,20 @@ def dtype_code(tensor):
 
 # ---- GPT-2 causal MHA ------------------------------------------------------
 
-def mha_forward(qkv, context_length, num_heads, stream=None):
+def mha_forward(qkv, context_length, num_heads, stream=None, into=None):
     """qkv [rows, 3E] (float32 or bfloat16, contiguous, on the GPU).
-    Returns (out [rows, E], maxima [rows/T*H, T], normalizers)."""
+    Returns (out [rows, E], maxima [rows/T*H, T], normalizers); `into` is an
+    earlier result whose three tensors are written again instead of new ones."""
     assert qkv.is_contiguous()
     rows, packed = qkv.shape
     E = packed // 3
-    out = torch.empty((rows, E), dtype=qkv.dtype, device=qkv.device)
-    stats = (max(rows // max(context_length, 1), 0) * num_heads, context_length)
-    maxima = torch.empty(stats, dtype=torch.float32, device=qkv.device)
-    normalizers = torch.empty(stats, dtype=torch.float32, device=qkv.device)
+    if into is not None:
+        out, maxima, normalizers = into
+    else:
+        out = torch.empty((rows, E), dtype=qkv.dtype, device=qkv.device)
+        stats = (max(rows // max(context_length, 1), 0) * num_heads, context_length)
+        maxima = torch.empty(stats, dtype=torch.float32, device=qkv.device)
+        normalizers = torch.empty(stats, dtype=torch.float32, device=qkv.device)
     check(lib().pluto_hip_mha_forward(stream or current_stream(), dtype_code(qkv),
                                       ptr(qkv), rows, context_length, num_heads, E,
                                       ptr(out), ptr(maxima), ptr(normalizers)))
@@ -296,17 +319,19 @@ def gqa_prefill_saved(p, length, cache, device="cuda"):
 
 
 def gqa_prefill(p, qg, k, v, q_norm, k_norm, cache, start_position=0, want_lse=False,
-                stream=None, want_probabilities=False, saved=None):
+                stream=None, want_probabilities=False, saved=None, out=None, workspace=None):
     """qg bf16 [T, qh, 2, d]; k, v bf16 [T, kh, d]; norms fp32 [d].
 
     want_probabilities appends fp32 [qh, T, start_position + T] to the result.
     saved: a gqa_prefill_saved(...) buffer to fill for the backward pass."""
     T = qg.shape[0]
-    out = torch.empty((T, p.query_heads, p.head_dim), dtype=torch.bfloat16, device=qg.device)
+    if out is None:
+        out = torch.empty((T, p.query_heads, p.head_dim), dtype=torch.bfloat16, device=qg.device)
     lse = (torch.empty((T, p.query_heads), dtype=torch.float32, device=qg.device)
            if want_lse else None)
     size = lib().pluto_hip_gqa_prefill_workspace_bytes(ctypes.byref(p), T)
-    workspace = torch.empty(max(size, 1), dtype=torch.uint8, device=qg.device)
+    if workspace is None:
+        workspace = torch.empty(max(size, 1), dtype=torch.uint8, device=qg.device)
     view = cache.view()
     check(lib().pluto_hip_gqa_prefill(stream or current_stream(), ctypes.byref(p), T,
                                       start_position, ptr(qg), ptr(k), ptr(v), ptr(q_norm),

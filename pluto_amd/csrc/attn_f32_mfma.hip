@@ -172,6 +172,7 @@ bool f32_forward_supported(const GenericForwardArgs& a) {
 int launch_f32_forward(hipStream_t stream, const GenericForwardArgs& a, int sequences) {
   const dim3 grid((a.q_rows + 31) / 32, a.query_heads, sequences);
   if (grid.y > 65535u || grid.z > 65535u) return PLUTO_HIP_EUNSUPPORTED;
+  if (!kernel_enabled(kMainKernel)) return 0;
   switch (a.head_dim) {
     case 32: f32_forward_kernel<32><<<grid, 64, 0, stream>>>(a); break;
     case 64: f32_forward_kernel<64><<<grid, 64, 0, stream>>>(a); break;

@@ -91,6 +91,17 @@ __device__ inline float wave_max(float v) {
 
 inline int launch_status() { return static_cast<int>(hipGetLastError()); }
 
+// Measurement hook (pluto_hip_test_kernel_classes): the launchers of the
+// specialised kernels ask whether their class is switched on, so that a
+// benchmark can time one kernel of a multi-launch entry point with events
+// around the call.  All classes are on unless a test or benchmark says so.
+enum KernelClass : unsigned {
+  kMainKernel = 1u,       // the kernel that bounds the call (flash, split-K, scan ...)
+  kQueryKernel = 2u,      // the query-owned half of the attention backward
+  kAuxiliaryKernel = 4u,  // preparation, tables, combines
+};
+bool kernel_enabled(KernelClass which);  // mha_capi.hip
+
 inline size_t align_up(size_t value, size_t alignment) {
   return (value + alignment - 1) / alignment * alignment;
 }

@@ -480,7 +480,8 @@ int launch_flash_backward(hipStream_t stream, const GenericBackwardArgs& a,
   if (tiles128 * units > 0x7fffffffLL) return PLUTO_HIP_EINVAL;
   const dim3 paired(static_cast<unsigned>(((tiles128 + 1) / 2) * units));
   const dim3 unpaired(static_cast<unsigned>(tiles128 * units));
-  if (dim == 64)
+  if (!kernel_enabled(kQueryKernel)) {
+  } else if (dim == 64)
     flash_dq_kernel<64, kDqPaired64><<<kDqPaired64 ? paired : unpaired, kThreads, 0, stream>>>(
         a, lse2, d_out_bf16);
   else
@@ -488,6 +489,7 @@ int launch_flash_backward(hipStream_t stream, const GenericBackwardArgs& a,
         a, lse2, d_out_bf16);
   status = launch_status();
   if (status != 0) return status;
+  if (!kernel_enabled(kMainKernel)) return 0;
   if (dim == 64)
     flash_dkv_kernel<64, kOtherPaired><<<kOtherPaired ? paired : unpaired, kThreads, 0, stream>>>(
         a, lse2, d_out_bf16);

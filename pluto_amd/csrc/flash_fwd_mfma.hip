@@ -409,6 +409,7 @@ int launch_flash_forward(hipStream_t stream, const FlashForwardArgs& a,
   const long long blocks = grid_blocks(a, 128, sequences, head_dim == 64);
   if (blocks <= 0 || blocks > 0x7fffffffLL) return PLUTO_HIP_EINVAL;
   const dim3 grid(static_cast<unsigned>(blocks));
+  if (!kernel_enabled(kMainKernel)) return 0;
   if (head_dim == 256)
     flash_forward_kernel<256, 1, 4><<<grid, 256, 0, stream>>>(a);
   else if (head_dim == 128)

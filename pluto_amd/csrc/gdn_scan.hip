@@ -791,9 +791,11 @@ int launch_gdn_chunked(hipStream_t stream, const GdnArgs& a) {
   const long long chunks = (a.length + C - 1) / C;
   const long long heads = static_cast<long long>(a.batch) * a.value_heads;
   if (heads * chunks > 0x7fffffffLL) return PLUTO_HIP_EINVAL;
-  gdn_chunk_prepare<<<static_cast<unsigned>(heads * chunks), 256, 0, stream>>>(a);
+  if (kernel_enabled(kAuxiliaryKernel))
+    gdn_chunk_prepare<<<static_cast<unsigned>(heads * chunks), 256, 0, stream>>>(a);
   int status = launch_status();
   if (status != 0) return status;
+  if (!kernel_enabled(kMainKernel)) return 0;
   gdn_chunk_scan<<<static_cast<unsigned>(heads * (SLICES / kScanGroup)), kScanThreads, 0, stream>>>(a);
   return launch_status();
 }

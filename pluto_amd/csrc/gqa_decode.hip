@@ -370,6 +370,7 @@ int launch_decode_fast(hipStream_t stream, const DecodeArgs& a, const DecodeBatc
   if (blocks <= 0 || blocks > 0x7fffffffLL) return PLUTO_HIP_EINVAL;
   if (a.split_tokens < 64 || a.split_tokens > kMaxSplit || a.split_tokens % 64 != 0)
     return PLUTO_HIP_EINVAL;
+  if (!kernel_enabled(kMainKernel)) return 0;
   switch (a.head_dim) {
     case 64: return launch_for_group<64>(stream, a, batch, group, static_cast<unsigned>(blocks));
     case 128: return launch_for_group<128>(stream, a, batch, group, static_cast<unsigned>(blocks));
@@ -380,6 +381,7 @@ int launch_decode_fast(hipStream_t stream, const DecodeArgs& a, const DecodeBatc
 
 int launch_decode_combine(hipStream_t stream, const DecodeCombineArgs& a,
                           const DecodeBatch& batch) {
+  if (!kernel_enabled(kAuxiliaryKernel)) return 0;
   decode_combine_kernel<<<batch.count * a.query_heads, 256, 0, stream>>>(a, batch);
   return launch_status();
 }

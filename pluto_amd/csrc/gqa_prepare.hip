@@ -259,6 +259,7 @@ int launch_rope_table(hipStream_t stream, int start_position, int length,
                       int rotary_dim, float theta, bool round, float* cosines,
                       float* sines) {
   const long long count = static_cast<long long>(length) * (rotary_dim / 2);
+  if (!kernel_enabled(kAuxiliaryKernel)) return 0;
   rope_table_kernel<<<static_cast<unsigned>((count + 255) / 256), 256, 0, stream>>>(
       start_position, length, rotary_dim, theta, round, cosines, sines);
   return launch_status();
@@ -268,6 +269,7 @@ int launch_prefill_prepare(hipStream_t stream, const PrefillPrepareArgs& a) {
   const long long units =
       static_cast<long long>(a.length) * (a.query_heads + a.key_value_heads);
   const int d = a.head_dim;
+  if (!kernel_enabled(kAuxiliaryKernel)) return 0;
   auto aligned = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
   const bool vectorised =
       a.round && a.q_out_dtype == PLUTO_HIP_BF16 && a.cache.dtype == PLUTO_HIP_BF16 &&
@@ -295,6 +297,7 @@ int launch_decode_prepare(hipStream_t stream, const DecodePrepareArgs& a,
                           const DecodeBatch& batch) {
   const long long units =
       static_cast<long long>(batch.count) * (a.query_heads + a.key_value_heads);
+  if (!kernel_enabled(kAuxiliaryKernel)) return 0;
   decode_prepare_kernel<<<static_cast<unsigned>((units + 3) / 4), 256, 0, stream>>>(a, batch);
   return launch_status();
 }

@@ -20,6 +20,13 @@ std::atomic<int> force_generic_flag{0};
 bool force_generic() { return force_generic_flag.load(std::memory_order_relaxed) != 0; }
 
 namespace {
+std::atomic<unsigned> kernel_class_mask{~0u};
+}
+bool kernel_enabled(KernelClass which) {
+  return (kernel_class_mask.load(std::memory_order_relaxed) & which) != 0;
+}
+
+namespace {
 
 int validate_mha(int dtype, int rows, int context_length, int num_heads,
                  int embedding_dim) {
@@ -71,6 +78,8 @@ extern "C" {
 int pluto_hip_test_force_generic(int enabled) {
   return force_generic_flag.exchange(enabled != 0 ? 1 : 0);
 }
+
+unsigned pluto_hip_test_kernel_classes(unsigned mask) { return kernel_class_mask.exchange(mask); }
 
 int pluto_hip_mha_forward(void* stream, int dtype, const void* qkv, int rows,
                           int context_length, int num_heads, int embedding_dim,
