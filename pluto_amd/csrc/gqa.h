@@ -34,8 +34,8 @@ struct PrefillPrepareArgs {
 
 // Per-launch slice of a decode batch, passed by value as a kernel argument.
 struct DecodeBatch {
-  int first = 0;  // index of the slice's first sequence in the full batch
   int count = 0;
+  int sequence[kDecodeBatchMax];  // index of entry i in the full batch
   int positions[kDecodeBatchMax];
   void* keys[kDecodeBatchMax];
   void* values[kDecodeBatchMax];
@@ -58,10 +58,20 @@ struct DecodePrepareArgs {
   bool round = true;
 };
 
+// The fused decode step (preparation of the new token, split-K attention over
+// the cache, combine and gate in the workgroup that finishes a (sequence, kv
+// head) last).
 struct DecodeArgs {
-  const uint16_t* q = nullptr;  // prepared queries, bf16 [batch, qh, d]
-  long long token_stride = 0, head_stride = 0;
-  int query_heads = 0, key_value_heads = 0, head_dim = 0;
+  const void* q_gate = nullptr;  // [batch, qh, 2, d]
+  const void* k = nullptr;       // [batch, kh, d]
+  const void* v = nullptr;
+  int io_dtype = PLUTO_HIP_F32;  // storage of q_gate, k, v and out
+  const float* q_norm = nullptr;
+  const float* k_norm = nullptr;
+  void* out = nullptr;  // [batch, qh, d]
+  long long token_stride = 0, head_stride = 0;  // of the bf16 caches
+  int query_heads = 0, key_value_heads = 0, head_dim = 0, rotary_dim = 0;
+  float epsilon = 1e-6f;
   int split_tokens = 512;
   float scale = 1.0f;
   // partial results of split-K block i (global index block_start[b] + j,
@@ -69,19 +79,12 @@ struct DecodeArgs {
   float* part_o = nullptr;
   float* part_m = nullptr;
   float* part_l = nullptr;
+  // one counter per (sequence, kv head) of the whole batch: zero when the
+  // kernel starts, and zero again when it ends
+  unsigned* arrivals = nullptr;
   long long block_base = 0;  // global index of this launch's first block
-};
-
-struct DecodeCombineArgs {
-  const float* part_o = nullptr;
-  const float* part_m = nullptr;
-  const float* part_l = nullptr;
-  long long block_base = 0;
-  const void* q_gate = nullptr;  // gate logits at [batch, qh, 1, :]
-  void* out = nullptr;           // [batch, qh, d]
-  int io_dtype = PLUTO_HIP_F32;
-  int query_heads = 0, key_value_heads = 0, head_dim = 0;
-  bool round = true;
+  // theta^(-2 f / rotary) for f < rotary / 2, evaluated on the host in FP64
+  double inverse_frequency[128];
 };
 
 int launch_rope_table(hipStream_t stream, int start_position, int length,
@@ -93,8 +96,9 @@ int launch_decode_prepare(hipStream_t stream, const DecodePrepareArgs& args,
 bool decode_fast_supported(int head_dim, int group);
 int launch_decode_fast(hipStream_t stream, const DecodeArgs& args,
                        const DecodeBatch& batch);
-int launch_decode_combine(hipStream_t stream, const DecodeCombineArgs& args,
-                          const DecodeBatch& batch);
+// Zeroes `count` arrival counters (a launch of its own: the fused kernel needs
+// them zero, and leaves them zero).
+int launch_decode_clear(hipStream_t stream, unsigned* arrivals, int count);
 // Two-pass probability rows (any dtype, any shape): row r of `rows` sees the
 // first `first_visible + r` cache rows; output fp32 [query_heads, rows,
 // row_width], zero beyond the visible prefix

@@ -427,6 +427,31 @@ int pluto_hip_gqa_prefill_probabilities(void* stream, const pluto_hip_attention_
       p->key_value_heads, p->head_dim, length, start_position + 1, width, scale, probabilities);
 }
 
+// Scratch of a decode call: arrival counters (one per sequence and kv head),
+// prepared queries (read by the any-shape kernels and the probabilities pass),
+// split-K partial results.
+struct DecodeLayout {
+  size_t arrivals, queries, part_o, part_m, part_l, total;
+};
+static DecodeLayout decode_layout(const pluto_hip_attention_params* p, int batch, long long blocks,
+                                  size_t arrivals_bytes) {
+  DecodeLayout l{};
+  const size_t heads = static_cast<size_t>(p->query_heads);
+  size_t at = 0;
+  auto take = [&](size_t bytes) {
+    const size_t offset = at;
+    at += align_up(bytes, 256);
+    return offset;
+  };
+  l.arrivals = take(arrivals_bytes);
+  l.queries = take(static_cast<size_t>(batch) * heads * p->head_dim * 4);
+  l.part_o = take(static_cast<size_t>(blocks) * heads * p->head_dim * 4);
+  l.part_m = take(static_cast<size_t>(blocks) * heads * 4);
+  l.part_l = take(static_cast<size_t>(blocks) * heads * 4);
+  l.total = at;
+  return l;
+}
+
 size_t pluto_hip_gqa_decode_workspace_bytes(const pluto_hip_attention_params* p, int batch,
                                             const int* positions, int split_tokens) {
   if (validate_params(p) != 0 || batch <= 0 || !positions) return 0;
@@ -435,11 +460,9 @@ size_t pluto_hip_gqa_decode_workspace_bytes(const pluto_hip_attention_params* p,
   for (int b = 0; b < batch; ++b)
     if (positions[b] < 0) return 0;
   const long long blocks = decode_blocks(batch, positions, split);
-  const size_t heads = static_cast<size_t>(p->query_heads);
-  size_t bytes = align_up(static_cast<size_t>(batch) * heads * p->head_dim * 4, 256);
-  bytes += align_up(static_cast<size_t>(blocks) * heads * p->head_dim * 4, 256);
-  bytes += 2 * align_up(static_cast<size_t>(blocks) * heads * 4, 256);
-  return bytes;
+  return decode_layout(p, batch, blocks,
+                       static_cast<size_t>(batch) * p->key_value_heads * sizeof(unsigned))
+      .total;
 }
 
 // Argument checks of the decode entry points; everything is rejected before
@@ -469,11 +492,16 @@ static int decode_check(const pluto_hip_attention_params* p, int batch, int io_d
   return 0;
 }
 
+// The fixed scratch starts with room for this many arrival counters; they are
+// zero when the library is loaded and every call leaves them zero.
+constexpr size_t kStaticArrivalBytes = 16384;
+
 static int decode_run(void* stream, const pluto_hip_attention_params* p, int batch, int io_dtype,
                       const void* q_gate, const void* k, const void* v, const float* q_norm,
                       const float* k_norm, const int* positions,
                       const pluto_hip_kv_cache_view* caches, void* out,
-                      float* const* probabilities, int split, void* workspace);
+                      float* const* probabilities, int split, void* workspace,
+                      const DecodeLayout& layout, bool clear_arrivals);
 
 int pluto_hip_gqa_decode(void* stream, const pluto_hip_attention_params* p, int batch,
                          int io_dtype, const void* q_gate, const void* k, const void* v,
@@ -485,10 +513,13 @@ int pluto_hip_gqa_decode(void* stream, const pluto_hip_attention_params* p, int 
   const int status =
       decode_check(p, batch, io_dtype, q_gate, k, v, q_norm, k_norm, positions, caches, out, split);
   if (status != 0) return status;
-  const size_t needed = pluto_hip_gqa_decode_workspace_bytes(p, batch, positions, split);
-  if (!workspace || workspace_bytes < needed) return PLUTO_HIP_EWORKSPACE;
+  const DecodeLayout layout =
+      decode_layout(p, batch, decode_blocks(batch, positions, split),
+                    static_cast<size_t>(batch) * p->key_value_heads * sizeof(unsigned));
+  if (!workspace || workspace_bytes < layout.total) return PLUTO_HIP_EWORKSPACE;
+  // whatever the workspace held: the counters are cleared by a launch of their own
   return decode_run(stream, p, batch, io_dtype, q_gate, k, v, q_norm, k_norm, positions, caches,
-                    out, probabilities, split, workspace);
+                    out, probabilities, split, workspace, layout, true);
 }
 
 size_t pluto_hip_gqa_decode_static_bytes(void) { return kStaticScratchBytes; }
@@ -507,111 +538,132 @@ int pluto_hip_gqa_decode_static(void* stream, const pluto_hip_attention_params* 
   int status =
       decode_check(p, batch, io_dtype, q_gate, k, v, q_norm, k_norm, positions, caches, out, split);
   if (status != 0) return status;
-  const size_t needed = pluto_hip_gqa_decode_workspace_bytes(p, batch, positions, split);
-  if (needed == 0) return PLUTO_HIP_EINVAL;
-  if (needed > kStaticScratchBytes) return PLUTO_HIP_ELIMIT;
+  if (static_cast<size_t>(batch) * p->key_value_heads * sizeof(unsigned) > kStaticArrivalBytes)
+    return PLUTO_HIP_ELIMIT;
+  const DecodeLayout layout =
+      decode_layout(p, batch, decode_blocks(batch, positions, split), kStaticArrivalBytes);
+  if (layout.total > kStaticScratchBytes) return PLUTO_HIP_ELIMIT;
   void* address = nullptr;
   status = static_scratch(&address);
   if (status != 0) return status;
+  // The counters at the head of the array are zero since the library was
+  // loaded and every call leaves them zero: nothing to clear, one launch.
   return decode_run(stream, p, batch, io_dtype, q_gate, k, v, q_norm, k_norm, positions, caches,
-                    out, probabilities, split, address);
+                    out, probabilities, split, address, layout, false);
 }
 
 static int decode_run(void* stream, const pluto_hip_attention_params* p, int batch, int io_dtype,
                       const void* q_gate, const void* k, const void* v, const float* q_norm,
                       const float* k_norm, const int* positions,
                       const pluto_hip_kv_cache_view* caches, void* out,
-                      float* const* probabilities, int split, void* workspace) {
+                      float* const* probabilities, int split, void* workspace,
+                      const DecodeLayout& layout, bool clear_arrivals) {
   int status = 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int qh = p->query_heads, kh = p->key_value_heads, d = p->head_dim;
   const int group = qh / kh;
   const bool round = p->round_to_bfloat16 != 0;
-  const long long blocks = decode_blocks(batch, positions, split);
   char* area = static_cast<char*>(workspace);
-  void* queries = area;
-  size_t offset = align_up(static_cast<size_t>(batch) * qh * d * 4, 256);
-  float* part_o = reinterpret_cast<float*>(area + offset);
-  offset += align_up(static_cast<size_t>(blocks) * qh * d * 4, 256);
-  float* part_m = reinterpret_cast<float*>(area + offset);
-  offset += align_up(static_cast<size_t>(blocks) * qh * 4, 256);
-  float* part_l = reinterpret_cast<float*>(area + offset);
+  void* queries = area + layout.queries;
 
   const pluto_hip_kv_cache_view& c0 = caches[0];
   bool fast = round && c0.dtype == PLUTO_HIP_BF16 && decode_fast_supported(d, group) &&
-              !force_generic() && c0.token_stride % 8 == 0 && c0.head_stride % 8 == 0;
+              p->rotary_dim / 2 <= 128 && !force_generic() && c0.token_stride % 8 == 0 &&
+              c0.head_stride % 8 == 0;
   for (int b = 0; b < batch && fast; ++b)
     fast = aligned16(caches[b].keys) && aligned16(caches[b].values);
   const int q_dtype = round ? PLUTO_HIP_BF16 : PLUTO_HIP_F32;
   const float scale = 1.0f / std::sqrt(static_cast<float>(d));
   const size_t io_bytes = element_bytes(io_dtype);
 
+  if (fast && clear_arrivals) {
+    status = launch_decode_clear(s, reinterpret_cast<unsigned*>(area + layout.arrivals),
+                                 batch * kh);
+    if (status != 0) return status;
+  }
   long long block_base = 0;
   for (int first = 0; first < batch; first += kDecodeBatchMax) {
     DecodeBatch slice;
-    slice.first = first;
     slice.count = batch - first < kDecodeBatchMax ? batch - first : kDecodeBatchMax;
     slice.block_start[0] = 0;
+    // Long sequences first: the workgroups that combine a sequence's blocks then
+    // run while shorter sequences are still streaming, not after everything
+    // else (insertion sort of at most kDecodeBatchMax entries, on the stack).
+    int order[kDecodeBatchMax];
     for (int i = 0; i < slice.count; ++i) {
-      slice.positions[i] = positions[first + i];
-      slice.keys[i] = caches[first + i].keys;
-      slice.values[i] = caches[first + i].values;
-      slice.block_start[i + 1] = slice.block_start[i] + (positions[first + i] + split) / split;
+      int at = i;
+      while (at > 0 && positions[order[at - 1]] < positions[first + i]) {
+        order[at] = order[at - 1];
+        --at;
+      }
+      order[at] = first + i;
     }
-    DecodePrepareArgs prep;
-    prep.q_gate = q_gate;
-    prep.k = k;
-    prep.v = v;
-    prep.io_dtype = io_dtype;
-    prep.q_norm = q_norm;
-    prep.k_norm = k_norm;
-    prep.q_out = queries;
-    prep.q_out_dtype = q_dtype;
-    prep.cache_dtype = c0.dtype;
-    prep.token_stride = c0.token_stride;
-    prep.head_stride = c0.head_stride;
-    prep.query_heads = qh;
-    prep.key_value_heads = kh;
-    prep.head_dim = d;
-    prep.rotary_dim = p->rotary_dim;
-    prep.epsilon = p->rms_norm_epsilon;
-    prep.theta = p->rope_theta;
-    prep.round = round;
-    status = launch_decode_prepare(s, prep, slice);
-    if (status != 0) return status;
+    for (int i = 0; i < slice.count; ++i) {
+      const int b = order[i];
+      slice.sequence[i] = b;
+      slice.positions[i] = positions[b];
+      slice.keys[i] = caches[b].keys;
+      slice.values[i] = caches[b].values;
+      slice.block_start[i + 1] = slice.block_start[i] + (positions[b] + split) / split;
+    }
+    if (!fast || probabilities) {
+      // the any-shape kernels and the probabilities pass read prepared queries
+      // (and the appended row) from memory
+      DecodePrepareArgs prep;
+      prep.q_gate = q_gate;
+      prep.k = k;
+      prep.v = v;
+      prep.io_dtype = io_dtype;
+      prep.q_norm = q_norm;
+      prep.k_norm = k_norm;
+      prep.q_out = queries;
+      prep.q_out_dtype = q_dtype;
+      prep.cache_dtype = c0.dtype;
+      prep.token_stride = c0.token_stride;
+      prep.head_stride = c0.head_stride;
+      prep.query_heads = qh;
+      prep.key_value_heads = kh;
+      prep.head_dim = d;
+      prep.rotary_dim = p->rotary_dim;
+      prep.epsilon = p->rms_norm_epsilon;
+      prep.theta = p->rope_theta;
+      prep.round = round;
+      status = launch_decode_prepare(s, prep, slice);
+      if (status != 0) return status;
+    }
     if (fast) {
       DecodeArgs a;
-      a.q = static_cast<const uint16_t*>(queries);
+      a.q_gate = q_gate;
+      a.k = k;
+      a.v = v;
+      a.io_dtype = io_dtype;
+      a.q_norm = q_norm;
+      a.k_norm = k_norm;
+      a.out = out;
       a.token_stride = c0.token_stride;
       a.head_stride = c0.head_stride;
       a.query_heads = qh;
       a.key_value_heads = kh;
       a.head_dim = d;
+      a.rotary_dim = p->rotary_dim;
+      a.epsilon = p->rms_norm_epsilon;
       a.split_tokens = split;
       a.scale = scale;
-      a.part_o = part_o;
-      a.part_m = part_m;
-      a.part_l = part_l;
+      a.part_o = reinterpret_cast<float*>(area + layout.part_o);
+      a.part_m = reinterpret_cast<float*>(area + layout.part_m);
+      a.part_l = reinterpret_cast<float*>(area + layout.part_l);
+      a.arrivals = reinterpret_cast<unsigned*>(area + layout.arrivals);
       a.block_base = block_base;
+      // the scalar specification's frequency, in FP64
+      // (cached_attention_ops_test.cc:66-67)
+      for (int f = 0; f < p->rotary_dim / 2; ++f)
+        a.inverse_frequency[f] =
+            std::pow(static_cast<double>(p->rope_theta), -2.0 * f / p->rotary_dim);
       status = launch_decode_fast(s, a, slice);
-      if (status != 0) return status;
-      DecodeCombineArgs c;
-      c.part_o = part_o;
-      c.part_m = part_m;
-      c.part_l = part_l;
-      c.block_base = block_base;
-      c.q_gate = q_gate;
-      c.out = out;
-      c.io_dtype = io_dtype;
-      c.query_heads = qh;
-      c.key_value_heads = kh;
-      c.head_dim = d;
-      c.round = round;
-      status = launch_decode_combine(s, c, slice);
       if (status != 0) return status;
     } else {
       for (int i = 0; i < slice.count; ++i) {
-        const int b = first + i;
+        const int b = slice.sequence[i];
         GenericForwardArgs a;
         const char* qbase = static_cast<const char*>(queries) +
                             static_cast<size_t>(b) * qh * d * element_bytes(q_dtype);
@@ -639,7 +691,7 @@ static int decode_run(void* stream, const pluto_hip_attention_params* p, int bat
     }
     if (probabilities) {
       for (int i = 0; i < slice.count; ++i) {
-        const int b = first + i;
+        const int b = slice.sequence[i];
         if (!probabilities[b]) continue;
         const char* qbase = static_cast<const char*>(queries) +
                             static_cast<size_t>(b) * qh * d * element_bytes(q_dtype);

@@ -1,13 +1,21 @@
-// Batched single-token GQA decode against a bf16 KV cache: split-K over blocks
-// of the sequence, tuned as an HBM streaming kernel.
+// Batched single-token GQA decode against a bf16 KV cache: one fused kernel,
+// split-K over blocks of the sequence, tuned as an HBM streaming kernel.
 //
-// Semantics: FullAttentionKernel (src/llm/layers/util/cached_attention_ops.cc:
-// 83-126) for every sequence of the batch.  One workgroup owns one
-// (sequence, kv head, block of `split_tokens` cache rows) and serves ALL query
-// heads of the group, so every K and V byte is read from HBM exactly once (the
-// reference launches one program per query head and streams the cache once per
-// head of the group).
+// Semantics: CachedAttentionStep (src/llm/layers/util/cached_attention_ops.cc:
+// 308-353: PrepareAttentionKernel :30-79, FullAttentionKernel :83-126) for
+// every sequence of the batch.  One workgroup owns one (sequence, kv head,
+// block of `split_tokens` cache rows) and serves ALL query heads of the group,
+// so every K and V byte is read from HBM exactly once (the reference launches
+// one program per query head and streams the cache once per head of the
+// group).
 //
+//   prepare Every workgroup normalises and rotates the group's query heads
+//           itself (a few hundred values; cheaper than a launch of its own)
+//           while its first cache rows are already travelling.  The
+//           workgroup that owns a sequence's last block also prepares the new
+//           K row and the V row, appends them to the cache and keeps a copy
+//           in LDS: it is the only one that needs them, and takes them from
+//           there.
 //   scores  S^T[token, head] = K[token, :] . q[head, :] with
 //           v_mfma_f32_16x16x32_bf16: the A operand (16 tokens x 32 channels) is
 //           loaded straight from global memory, 16 bytes per lane, the four
@@ -16,16 +24,21 @@
 //   values  O[head, :] += p[head, token] * V[token, :] on the vector ALU: 16
 //           bytes of V per lane, probabilities broadcast from LDS.  The kernel
 //           is bound by HBM, not by this arithmetic.
-// Partial (o, m, l) triples are written per block; a second kernel combines a
-// sequence's blocks in ascending order (fixed order: bitwise repeatable) and
-// applies bf16(bf16(core) * bf16(sigmoid(gate))).
+//   combine Partial (o, m, l) triples are written per block.  Workgroups count
+//           their arrivals per (sequence, kv head); the one that arrives last
+//           combines that pair's blocks in ascending order (a fixed order,
+//           whichever workgroup does it: bitwise repeatable), applies
+//           bf16(bf16(core) * bf16(sigmoid(gate))) and leaves the counter zero.
 #include "gqa.h"
+#include "gqa_rotate.h"
+#include "mfma_tile.h"
 
 namespace pluto_hip {
 namespace {
 
 constexpr int kMaxSplit = 512;
 constexpr int kThreads = 256;
+constexpr int kCombineChunk = 128;  // blocks combined per pass over the LDS weights
 
 __device__ inline bf16x8 load_bf16x8(const uint16_t* p) {
   return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p));
@@ -40,257 +53,545 @@ __device__ inline int find_sequence(const DecodeBatch& batch, int block) {
   return lo;
 }
 
-template <int D, int GROUP>
-__global__ void __launch_bounds__(kThreads)
-decode_split_kernel(DecodeArgs a, DecodeBatch batch) {
-  constexpr int KSTEPS = D / 32;
-  constexpr int LANES_PER_ROW = D / 8;     // phase 2: 16-byte pieces per V row
-  constexpr int ROWS_PER_PASS = 64 / LANES_PER_ROW;
-  // The probabilities (phases 1-2) and the per-wave partial outputs (after
-  // phase 2) share one LDS area, so that eight workgroups fit a compute unit.
-  constexpr int kProbFloats = kMaxSplit * 8, kOutFloats = 4 * GROUP * D;
-  __shared__ __attribute__((aligned(16))) float shared_area[kProbFloats > kOutFloats ? kProbFloats : kOutFloats];
-  float (*p_lds)[8] = reinterpret_cast<float (*)[8]>(shared_area);
-  float (*o_lds)[GROUP][D] = reinterpret_cast<float (*)[GROUP][D]>(shared_area);
-  __shared__ float wave_max[4][16];
-  __shared__ float wave_sum_lds[4][16];
+// Partial results travel between workgroups on different XCDs, each with an L2
+// of its own.  They are stored and loaded as device-scope relaxed atomics,
+// which go through to the memory side, so no L2 has to be written back or
+// invalidated wholesale (a device-scope fence does both, and costs more than
+// the rest of the kernel when four thousand workgroups issue one each).
+__device__ inline void store_shared(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ inline float load_shared(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
-  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+// Workgroup barrier that orders LDS traffic only: unlike __syncthreads() it
+// does not wait for the wave's outstanding global loads.
+__device__ inline void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+// One wave prepares one head vector (RMSNorm with (1 + w), split-half partial
+// RoPE, bf16 rounding points as in normalize_rotate) with a single round trip
+// to memory: every lane loads its D/64 channels and weights at once, the RoPE
+// partner comes from the LDS row the result is left in.  `row` receives the
+// bf16 bits; `cosine`/`sine` hold this lane's rounded table entries per slot.
+template <int D>
+__device__ inline void prepare_head(const void* base, long long offset, int dtype,
+                                    const float* weight, int rotary_dim, float epsilon,
+                                    const float (&cosine)[D / 64], const float (&sine)[D / 64],
+                                    uint16_t* row) {
+  constexpr int SLOTS = D / 64;
+  const int lane = threadIdx.x % 64;
+  float x[SLOTS], w[SLOTS];
+  if (dtype == PLUTO_HIP_BF16) {
+    const uint16_t* in = static_cast<const uint16_t*>(base) + offset;
+#pragma unroll
+    for (int i = 0; i < SLOTS; ++i) x[i] = bf16_bits_to_float(in[lane + 64 * i]);
+  } else {
+    const float* in = static_cast<const float*>(base) + offset;
+#pragma unroll
+    for (int i = 0; i < SLOTS; ++i) x[i] = in[lane + 64 * i];
+  }
+#pragma unroll
+  for (int i = 0; i < SLOTS; ++i) w[i] = weight[lane + 64 * i];
+  double square = 0.0;
+#pragma unroll
+  for (int i = 0; i < SLOTS; ++i) square += static_cast<double>(x[i] * x[i]);
+  square = wave_sum_f64(square);
+  const double inverse = 1.0 / sqrt(square / D + static_cast<double>(epsilon));
+  float normal[SLOTS];
+#pragma unroll
+  for (int i = 0; i < SLOTS; ++i) {
+    normal[i] = round_to_bf16(
+        static_cast<float>(x[i] * inverse * (1.0 + static_cast<double>(w[i]))));
+    row[lane + 64 * i] = static_cast<uint16_t>(__float_as_uint(normal[i]) >> 16);
+  }
+  // the wave's normalised row is in LDS before partners are read from it
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  __builtin_amdgcn_wave_barrier();
+  const int half = rotary_dim / 2;
+  float result[SLOTS];
+#pragma unroll
+  for (int i = 0; i < SLOTS; ++i) {
+    const int c = lane + 64 * i;
+    result[i] = normal[i];
+    if (c < rotary_dim) {
+      const float partner = bf16_bits_to_float(row[c < half ? c + half : c - half]);
+      const float a = round_to_bf16(normal[i] * cosine[i]);
+      const float b = round_to_bf16(partner * sine[i]);
+      result[i] = round_to_bf16(c < half ? a - b : a + b);
+    }
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  __builtin_amdgcn_wave_barrier();
+#pragma unroll
+  for (int i = 0; i < SLOTS; ++i)
+    row[lane + 64 * i] = static_cast<uint16_t>(__float_as_uint(result[i]) >> 16);
+}
+
+// What a workgroup knows about its (sequence, kv head, block).
+struct BlockContext {
+  int tid, wave, lane, hq, n;
+  int g, seq, position, length, t0, per_wave;
+  uint16_t* keys;    // this kv head's rows of the sequence's cache
+  uint16_t* values;
+  long long slot;    // where the block's partial results go
+};
+
+constexpr int kStageRows = 32;  // V rows per LDS stage of a wave: one contraction step
+
+// LDS of a workgroup: per wave two stages of 32 V rows (later reused for the
+// waves' partial outputs and the combine's block weights).
+template <int D>
+constexpr int value_area_bytes() { return 4 * 2 * kStageRows * D * 2; }
+
+// Prepare step, split-K attention over one block and the block's partial
+// results.  SPLIT: tokens per block when known at compile time (the loops
+// then have no branches the load scheduling would have to stop at), 0
+// otherwise.  LAST: the block holds the row this call appends; only then can
+// rows lie beyond the sequence, and only then is the new row needed (it is
+// taken from LDS, whatever the cache holds yet).
+//
+// Each wave owns a quarter of the block's tokens from the prepare step to the
+// end of phase 2 and waits for no other wave in between.
+//   phase 1  S^T[token, head] = K q^T for groups of 16 tokens, K rows straight
+//            from global memory into A operands.
+//   phase 2  O^T[channel, head] += V^T P^T for stages of 32 tokens
+//            (v_mfma_f32_16x16x32_bf16, one contraction step a stage).  V rows
+//            travel global -> LDS without registers (two stages a wave, the
+//            next one requested while this one is used) and are gathered into
+//            A operands by the LDS transpose read; P^T is the pair of score
+//            accumulators of the stage's two groups, so it needs no exchange.
+//            The contraction runs over (token 4q + e of the first group,
+//            e < 4; of the second group, e >= 4) for lane group q, in both
+//            operands.  Probabilities enter as bf16 hi + lo parts (two
+//            products), which keeps the FP32 arithmetic of the reference to
+//            about 2^-17.
+template <int D, int GROUP, int SPLIT, bool LAST>
+__device__ inline void decode_block(const DecodeArgs& a, const BlockContext& ctx,
+                                    unsigned char* value_area, float (*wave_max)[16],
+                                    float (*wave_sum_lds)[16], uint16_t (*q_lds)[D],
+                                    uint16_t (*new_row)[D]) {
+  constexpr int KSTEPS = D / 32;
+  constexpr int KCH = D / 8;                       // 16-byte chunks per row
+  constexpr int GROUPS = (SPLIT ? SPLIT : kMaxSplit) / 64;  // 16-token groups per wave at most
+  constexpr int STAGES = (GROUPS + 1) / 2;
+  constexpr int FILLS = kStageRows * KCH / 64;     // 16-byte fills per lane and stage
+  constexpr int kStageBytes = kStageRows * D * 2;
+  constexpr int CB = D / 16;                       // 16-channel blocks of O^T
+  float (*o_lds)[GROUP][D] = reinterpret_cast<float (*)[GROUP][D]>(value_area);
+  const int tid = ctx.tid, wave = ctx.wave, lane = ctx.lane, hq = ctx.hq, n = ctx.n;
+  const int g = ctx.g, seq = ctx.seq, position = ctx.position, length = ctx.length;
+  const int t0 = ctx.t0;
+  const int per_wave = SPLIT ? SPLIT / 4 : ctx.per_wave;
   const int kh = a.key_value_heads;
-  const int g = blockIdx.x % kh;
-  const int block = blockIdx.x / kh;
-  const int b = find_sequence(batch, block);
-  const int seq = batch.first + b;
-  const int length = batch.positions[b] + 1;
-  const int split = a.split_tokens;
-  const int t0 = (block - batch.block_start[b]) * split;
-  const int per_wave = split / 4;
-  const uint16_t* keys = static_cast<const uint16_t*>(batch.keys[b]) + g * a.head_stride;
-  const uint16_t* values = static_cast<const uint16_t*>(batch.values[b]) + g * a.head_stride;
+  const uint16_t* keys = ctx.keys;
   const float scale2 = a.scale * kLog2e;
+  const int groups = per_wave / 16;  // 16-token groups of this wave (<= GROUPS)
+  const int stages = (groups + 1) / 2;
+  const int wave_t0 = t0 + wave * per_wave;
+
+  // ---- the first two V stages are requested before anything else ----------
+  unsigned char* stage_base = value_area + wave * 2 * kStageBytes;
+  uint32_t fill_offset[FILLS];
+#pragma unroll
+  for (int i = 0; i < FILLS; ++i) fill_offset[i] = tile_fill_offset<D>(i * 64 + lane, a.token_stride);
+  auto fill = [&](int st) {
+    // rows beyond the sequence (LAST only) or beyond this call's reach read as
+    // zero: the descriptor ends with the last valid row
+    const int row0 = wave_t0 + kStageRows * st;
+    long long rows = kStageRows;
+    if constexpr (SPLIT == 0)  // a wave's quarter may end inside a stage
+      rows = min(rows, static_cast<long long>(per_wave) - kStageRows * st);
+    if constexpr (LAST) rows = min(rows, static_cast<long long>(length) - row0);
+    const uint32_t bytes =
+        rows <= 0 ? 0u : static_cast<uint32_t>(((rows - 1) * a.token_stride + D) * 2);
+    const int32x4 rsrc = make_rsrc(ctx.values + static_cast<long long>(row0) * a.token_stride, bytes);
+#pragma unroll
+    for (int i = 0; i < FILLS; ++i)
+      lds_fill<16>(rsrc, stage_base + (st & 1) * kStageBytes + i * 1024, fill_offset[i]);
+  };
+  fill(0);
+  if (1 < stages) fill(1);
+
+  // ---- then the first K rows ------------------------------------------------
+  // A operand row = lane % 16; rows beyond the valid prefix repeat its last row
+  auto k_token = [&](int grp) {
+    const int t = wave_t0 + 16 * grp + n;
+    return LAST ? min(t, length - 1) : t;
+  };
+  auto load_k = [&](int grp, bf16x8 (&dst)[KSTEPS]) {
+    // contraction step ks covers channels 32 ks .. 32 ks + 31: the four lanes
+    // of a token read one 64-byte sector per load
+    const uint16_t* row = keys + static_cast<long long>(k_token(grp)) * a.token_stride + 8 * hq;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) dst[ks] = load_bf16x8(row + 32 * ks);
+  };
+  bf16x8 k_rows[GROUPS][KSTEPS];
+#pragma unroll
+  for (int grp = 0; grp < GROUPS; ++grp)
+    if (grp < groups) load_k(grp, k_rows[grp]);
+
+  // ---- prepare: the group's queries, and the new cache row ----------------
+  {
+    // this lane's rotation table entries: channel c = lane + 64 i uses
+    // frequency c mod (rotary / 2)
+    const int half = a.rotary_dim / 2;
+    float cosine[D / 64], sine[D / 64];
+#pragma unroll
+    for (int i = 0; i < D / 64; ++i) {
+      const int c = lane + 64 * i;
+      cosine[i] = 1.0f;
+      sine[i] = 0.0f;
+      if (c < a.rotary_dim && (wave < GROUP || LAST)) {
+        const double angle =
+            static_cast<double>(position) * a.inverse_frequency[c < half ? c : c - half];
+        cosine[i] = round_to_bf16(static_cast<float>(cos(angle)));
+        sine[i] = round_to_bf16(static_cast<float>(sin(angle)));
+      }
+    }
+    for (int hh = wave; hh < GROUP; hh += 4)
+      prepare_head<D>(a.q_gate,
+                      (static_cast<long long>(seq) * a.query_heads + g * GROUP + hh) * 2 * D,
+                      a.io_dtype, a.q_norm, a.rotary_dim, a.epsilon, cosine, sine, q_lds[hh]);
+    if constexpr (LAST) {
+      // cached_attention_ops.cc:64-77: the rotated key and the rounded value
+      // become row `position` of the cache
+      const long long in = (static_cast<long long>(seq) * kh + g) * D;
+      const long long at = static_cast<long long>(position) * a.token_stride;
+      if (wave == 3) {
+        prepare_head<D>(a.k, in, a.io_dtype, a.k_norm, a.rotary_dim, a.epsilon, cosine, sine,
+                        new_row[0]);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_wave_barrier();
+        for (int c = lane; c < D; c += 64) ctx.keys[at + c] = new_row[0][c];
+      } else if (wave == 2) {
+        for (int c = lane; c < D; c += 64) {
+          const uint16_t bits = float_to_bf16_bits(load_element(a.v, in + c, a.io_dtype));
+          new_row[1][c] = bits;
+          ctx.values[at + c] = bits;
+        }
+      }
+    }
+    lds_barrier();
+  }
 
   // ---- phase 1: scores -------------------------------------------------
-  const int hq = lane / 16, n = lane % 16;
   bf16x8 qf[KSTEPS];
 #pragma unroll
   for (int ks = 0; ks < KSTEPS; ++ks) {
     uint4 bits = make_uint4(0, 0, 0, 0);
-    if (n < GROUP)
-      bits = *reinterpret_cast<const uint4*>(
-          a.q + (static_cast<long long>(seq) * a.query_heads + g * GROUP + n) * D +
-          32 * ks + 8 * hq);
+    if (n < GROUP) bits = *reinterpret_cast<const uint4*>(&q_lds[n][32 * ks + 8 * hq]);
     qf[ks] = __builtin_bit_cast(bf16x8, bits);
   }
-  // first batch of V rows for phase 2, requested now so that it travels while
-  // phase 1 computes (per_wave is a multiple of 16 rows, kBatch passes cover
-  // at most that)
-  constexpr int kBatch = 2;  // measured: 2 beats 1, 4, 8 and 16
-  const int sub = lane / LANES_PER_ROW, piece = lane % LANES_PER_ROW;
-  auto load_v = [&](int pass) {
-    const int token_local = wave * per_wave + pass * ROWS_PER_PASS + sub;
-    const int token = min(t0 + token_local, length - 1);
-    return *reinterpret_cast<const uint4*>(values + static_cast<long long>(token) * a.token_stride +
-                                           8 * piece);
-  };
-  uint4 v_next[kBatch];
+  bf16x8 k_new[KSTEPS];  // the appended row, as this lane would load it
+  if constexpr (LAST) {
 #pragma unroll
-  for (int i = 0; i < kBatch; ++i) v_next[i] = load_v(i);
-  const int groups = per_wave / 16;  // 16-token groups per wave (<= 8)
-  floatx4 s[kMaxSplit / 64];
+    for (int ks = 0; ks < KSTEPS; ++ks) k_new[ks] = load_bf16x8(&new_row[0][32 * ks + 8 * hq]);
+  }
+  floatx4 s[2 * STAGES];
   float local_max = kMasked;
 #pragma unroll
-  for (int grp = 0; grp < kMaxSplit / 64; ++grp) {
-    if (grp < groups) {
-      const int token_local = wave * per_wave + 16 * grp;
-      int token = t0 + token_local + n;  // A operand row = lane % 16
-      token = min(token, length - 1);    // stay inside the valid prefix
-      // contraction step ks covers channels 32 ks .. 32 ks + 31: the four lanes
-      // of a token read one 64-byte sector per load
-      const uint16_t* row = keys + static_cast<long long>(token) * a.token_stride + 8 * hq;
+  for (int grp = 0; grp < 2 * STAGES; ++grp) {
+    s[grp] = floatx4{kMasked, kMasked, kMasked, kMasked};
+    if (grp < GROUPS && grp < groups) {
       floatx4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks)
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(load_bf16x8(row + 32 * ks), qf[ks], acc,
-                                                      0, 0, 0);
+      for (int ks = 0; ks < KSTEPS; ++ks) {
+        bf16x8 k_use = k_rows[grp][ks];
+        if constexpr (LAST) k_use = k_token(grp) == position ? k_new[ks] : k_use;
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k_use, qf[ks], acc, 0, 0, 0);
+      }
       // accumulator register r = (token 4*hq + r of the group, head n)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const int t = t0 + token_local + 4 * hq + r;
-        const float v = t < length ? acc[r] * scale2 : kMasked;
+        const int t = wave_t0 + 16 * grp + 4 * hq + r;
+        const float v = (!LAST || t < length) ? acc[r] * scale2 : kMasked;
         acc[r] = v;
         local_max = fmaxf(local_max, v);
       }
       s[grp] = acc;
     }
   }
+  // Each wave normalises its quarter of the block by its own maximum.
   local_max = fmaxf(local_max, __shfl_xor(local_max, 16, 64));
   local_max = fmaxf(local_max, __shfl_xor(local_max, 32, 64));
   if (hq == 0) wave_max[wave][n] = local_max;
-  __syncthreads();
-  const float block_max = fmaxf(fmaxf(wave_max[0][n], wave_max[1][n]),
-                                fmaxf(wave_max[2][n], wave_max[3][n]));
+
+  // ---- phase 2: O^T += V^T P^T -------------------------------------------
+  floatx4 o_acc[CB];
+#pragma unroll
+  for (int cb = 0; cb < CB; ++cb) o_acc[cb] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
   float local_sum = 0.0f;
+  // transpose read of this lane: as a source it supplies row kk of its lane
+  // group's four rows, channels 4b .. 4b+3 of a 16-channel block
+  const int kk = (lane % 16) / 4, bsel = lane % 4;
+  int read_offset[2][CB];
 #pragma unroll
-  for (int grp = 0; grp < kMaxSplit / 64; ++grp) {
-    if (grp < groups) {
-      const int token_local = wave * per_wave + 16 * grp + 4 * hq;
+  for (int part = 0; part < 2; ++part) {
+    const int row = 16 * part + 4 * hq + kk;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const float p = __builtin_amdgcn_exp2f(s[grp][r] - block_max);
-        local_sum += p;
-        if (n < 8) p_lds[token_local + r][n] = p;
+    for (int cb = 0; cb < CB; ++cb)
+      read_offset[part][cb] =
+          (row * KCH + ((2 * cb + bsel / 2) ^ tile_swizzle(row))) * 16 + (bsel % 2) * 8;
+  }
+#pragma unroll
+  for (int st = 0; st < STAGES; ++st) {
+    if (st < stages) {
+      const unsigned char* stage = stage_base + (st & 1) * kStageBytes;
+      // this stage's rows have landed (the next stage's may still travel)
+      if (st + 1 < stages)
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(FILLS) : "memory");
+      else
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      if constexpr (LAST) {
+        const int local = position - (wave_t0 + kStageRows * st);
+        if (local >= 0 && local < kStageRows) {
+          // the appended V row: from LDS to its place in the stage
+          if (lane < KCH)
+            *reinterpret_cast<uint4*>(const_cast<unsigned char*>(stage) +
+                                      (local * KCH + (lane ^ tile_swizzle(local))) * 16) =
+                *reinterpret_cast<const uint4*>(&new_row[1][8 * lane]);
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
+      // P^T of the stage's two groups as hi + lo bf16 B operands
+      float p[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float score = s[2 * st + e / 4][e % 4];
+        // (a wave whose tokens all lie beyond the sequence has local_max ==
+        // kMasked: its probabilities are zero, not 2^0)
+        p[e] = score == kMasked ? 0.0f : __builtin_amdgcn_exp2f(score - local_max);
+        local_sum += p[e];
+      }
+      uint32_t hi[4], lo[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        hi[e] = pack_bf16(p[2 * e], p[2 * e + 1]);
+        lo[e] = pack_bf16(p[2 * e] - __uint_as_float(hi[e] << 16),
+                          p[2 * e + 1] - __uint_as_float(hi[e] & 0xffff0000u));
+      }
+      const bf16x8 p_hi = __builtin_bit_cast(bf16x8, make_uint4(hi[0], hi[1], hi[2], hi[3]));
+      const bf16x8 p_lo = __builtin_bit_cast(bf16x8, make_uint4(lo[0], lo[1], lo[2], lo[3]));
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb) {
+        const uint2 first = lds_transpose_read(stage, read_offset[0][cb]);
+        const uint2 second = lds_transpose_read(stage, read_offset[1][cb]);
+        const bf16x8 v_t =
+            __builtin_bit_cast(bf16x8, make_uint4(first.x, first.y, second.x, second.y));
+        o_acc[cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_t, p_hi, o_acc[cb], 0, 0, 0);
+        o_acc[cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_t, p_lo, o_acc[cb], 0, 0, 0);
+      }
+      // the stage after next takes this stage's place
+      if (st + 2 < stages) {
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_wave_barrier();
+        fill(st + 2);
       }
     }
   }
   local_sum += __shfl_xor(local_sum, 16, 64);
   local_sum += __shfl_xor(local_sum, 32, 64);
   if (hq == 0) wave_sum_lds[wave][n] = local_sum;
-  __syncthreads();
-
-  // ---- phase 2: O += p V ------------------------------------------------
-  float acc[GROUP][8];
+  __syncthreads();  // every wave is done with its V stages
+  // o_acc[cb][r] = O^T[channel 16 cb + 4 hq + r][head n]
+  if (n < GROUP) {
 #pragma unroll
-  for (int hh = 0; hh < GROUP; ++hh)
-#pragma unroll
-    for (int e = 0; e < 8; ++e) acc[hh][e] = 0.0f;
-  const int passes = per_wave / ROWS_PER_PASS;
-  // V rows travel in batches of kBatch loads per lane; a batch is requested
-  // while the previous one is consumed (the first one before phase 1's
-  // barriers, see above).
-  for (int first = 0; first < passes; first += kBatch) {
-    uint4 now[kBatch];
-#pragma unroll
-    for (int i = 0; i < kBatch; ++i) now[i] = v_next[i];
-    if (first + kBatch < passes) {
-#pragma unroll
-      for (int i = 0; i < kBatch; ++i) v_next[i] = load_v(first + kBatch + i);
-    }
-#pragma unroll
-    for (int i = 0; i < kBatch; ++i) {
-      if (first + i >= passes) break;  // narrow heads with the smallest split
-      const int token_local = wave * per_wave + (first + i) * ROWS_PER_PASS + sub;
-      const uint4 bits = now[i];
-      const float4 p0 = *reinterpret_cast<const float4*>(&p_lds[token_local][0]);
-      const float4 p1 = *reinterpret_cast<const float4*>(&p_lds[token_local][4]);
-      const float p[8] = {p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w};
-      const uint32_t w[4] = {bits.x, bits.y, bits.z, bits.w};
-      float v[8];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        v[2 * j] = __uint_as_float(w[j] << 16);
-        v[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
-      }
-#pragma unroll
-      for (int hh = 0; hh < GROUP; ++hh)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc[hh][e] += p[hh] * v[e];
-    }
-  }
-  // exchange stages outermost: the exchanges of a stage are in flight together
-#pragma unroll
-  for (int offset = LANES_PER_ROW; offset < 64; offset <<= 1) {
-    float other[GROUP][8];
-#pragma unroll
-    for (int hh = 0; hh < GROUP; ++hh)
-#pragma unroll
-      for (int e = 0; e < 8; ++e) other[hh][e] = __shfl_xor(acc[hh][e], offset, 64);
-#pragma unroll
-    for (int hh = 0; hh < GROUP; ++hh)
-#pragma unroll
-      for (int e = 0; e < 8; ++e) acc[hh][e] += other[hh][e];
-  }
-  __syncthreads();  // every wave is done with the probabilities
-  if (sub == 0) {
-#pragma unroll
-    for (int hh = 0; hh < GROUP; ++hh) {
-      float4 lo = make_float4(acc[hh][0], acc[hh][1], acc[hh][2], acc[hh][3]);
-      float4 hi = make_float4(acc[hh][4], acc[hh][5], acc[hh][6], acc[hh][7]);
-      *reinterpret_cast<float4*>(&o_lds[wave][hh][8 * piece]) = lo;
-      *reinterpret_cast<float4*>(&o_lds[wave][hh][8 * piece + 4]) = hi;
-    }
+    for (int cb = 0; cb < CB; ++cb)
+      *reinterpret_cast<float4*>(&o_lds[wave][n][16 * cb + 4 * hq]) =
+          make_float4(o_acc[cb][0], o_acc[cb][1], o_acc[cb][2], o_acc[cb][3]);
   }
   __syncthreads();
-  const long long slot = (a.block_base + block) * kh + g;
+  // the four waves' results, each relative to its own maximum, become the
+  // block's: o = sum_w o_w 2^(m_w - m), l likewise, m = max_w m_w
+  const long long slot = ctx.slot;
   for (int i = tid; i < GROUP * D; i += kThreads) {
     const int hh = i / D, c = i % D;
-    a.part_o[(slot * GROUP + hh) * D + c] =
-        (o_lds[0][hh][c] + o_lds[1][hh][c]) + (o_lds[2][hh][c] + o_lds[3][hh][c]);
+    const float m = fmaxf(fmaxf(wave_max[0][hh], wave_max[1][hh]),
+                          fmaxf(wave_max[2][hh], wave_max[3][hh]));
+    float w[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) w[q] = __builtin_amdgcn_exp2f(wave_max[q][hh] - m);
+    store_shared(&a.part_o[(slot * GROUP + hh) * D + c],
+                 (o_lds[0][hh][c] * w[0] + o_lds[1][hh][c] * w[1]) +
+                     (o_lds[2][hh][c] * w[2] + o_lds[3][hh][c] * w[3]));
   }
   if (tid < GROUP) {
-    a.part_m[slot * GROUP + tid] =
-        fmaxf(fmaxf(wave_max[0][tid], wave_max[1][tid]), fmaxf(wave_max[2][tid], wave_max[3][tid]));
-    a.part_l[slot * GROUP + tid] = (wave_sum_lds[0][tid] + wave_sum_lds[1][tid]) +
-                                   (wave_sum_lds[2][tid] + wave_sum_lds[3][tid]);
+    const float m = fmaxf(fmaxf(wave_max[0][tid], wave_max[1][tid]),
+                          fmaxf(wave_max[2][tid], wave_max[3][tid]));
+    float w[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) w[q] = __builtin_amdgcn_exp2f(wave_max[q][tid] - m);
+    store_shared(&a.part_m[slot * GROUP + tid], m);
+    store_shared(&a.part_l[slot * GROUP + tid],
+                 (wave_sum_lds[0][tid] * w[0] + wave_sum_lds[1][tid] * w[1]) +
+                     (wave_sum_lds[2][tid] * w[2] + wave_sum_lds[3][tid] * w[3]));
   }
 }
 
-// One workgroup (4 waves) per (sequence, query head).  Wave w folds the blocks
-// w, w+4, w+8, ... in ascending order, then the four partial results are added
-// in wave order: a fixed summation tree, hence bitwise repeatable.  Ends with
-// the sigmoid gate (cached_attention_ops.cc:119-125).
-__global__ void __launch_bounds__(256)
-decode_combine_kernel(DecodeCombineArgs a, DecodeBatch batch) {
-  __shared__ float wave_max_lds[4];
-  __shared__ float partial_o[4][256];
-  __shared__ float partial_l[4];
-  const int b = blockIdx.x / a.query_heads, head = blockIdx.x % a.query_heads;
-  const int seq = batch.first + b;
-  const int group = a.query_heads / a.key_value_heads;
-  const int g = head / group, hh = head % group;
-  const int D = a.head_dim;
-  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
-  const int first = batch.block_start[b], blocks = batch.block_start[b + 1] - first;
-  // partial results of block j live at slot0 + j * slot_step
-  const long long slot0 = ((a.block_base + first) * a.key_value_heads + g) * group + hh;
-  const long long slot_step = static_cast<long long>(a.key_value_heads) * group;
-  float maximum = kMasked;
-  for (int j = threadIdx.x; j < blocks; j += 256)
-    maximum = fmaxf(maximum, a.part_m[slot0 + j * slot_step]);
-  maximum = wave_max(maximum);
-  if (lane == 0) wave_max_lds[wave] = maximum;
-  __syncthreads();
-  maximum = fmaxf(fmaxf(wave_max_lds[0], wave_max_lds[1]), fmaxf(wave_max_lds[2], wave_max_lds[3]));
-  float normalizer = 0.0f;
-  float o[4] = {0.0f, 0.0f, 0.0f, 0.0f};  // head_dim <= 256 = 4 channels per lane
-  // four blocks per step: all loads of a step are issued before their use
-  for (int j0 = wave; j0 < blocks; j0 += 16) {
-    float bm[4], bl[4], bo[4][4];
+template <int D, int GROUP>
+__global__ void __launch_bounds__(kThreads)
+__attribute__((amdgpu_waves_per_eu(D == 256 ? 1 : 2, D == 256 ? 1 : 2)))
+decode_fused_kernel(DecodeArgs a, DecodeBatch batch) {
+  __shared__ __attribute__((aligned(1024))) unsigned char value_area[value_area_bytes<D>()];
+  float* shared_area = reinterpret_cast<float*>(value_area);
+  __shared__ float wave_max[4][16];
+  __shared__ float wave_sum_lds[4][16];
+  __shared__ __attribute__((aligned(16))) uint16_t q_lds[GROUP][D];  // prepared queries
+  __shared__ __attribute__((aligned(16))) uint16_t new_row[2][D];    // appended K and V rows
+  __shared__ int final_flag;
+
+  const int tid = threadIdx.x;
+  const int kh = a.key_value_heads;
+  const int g = blockIdx.x % kh;
+  const int block = blockIdx.x / kh;
+  const int b = find_sequence(batch, block);
+  const int seq = batch.sequence[b];
+  const int blocks_here = batch.block_start[b + 1] - batch.block_start[b];
+  const int j = block - batch.block_start[b];
+  BlockContext ctx;
+  ctx.tid = tid;
+  ctx.wave = tid / 64;
+  ctx.lane = tid % 64;
+  ctx.hq = ctx.lane / 16;
+  ctx.n = ctx.lane % 16;
+  ctx.g = g;
+  ctx.seq = seq;
+  ctx.position = batch.positions[b];
+  ctx.length = ctx.position + 1;
+  ctx.t0 = j * a.split_tokens;
+  ctx.per_wave = a.split_tokens / 4;
+  ctx.keys = static_cast<uint16_t*>(batch.keys[b]) + g * a.head_stride;
+  ctx.values = static_cast<uint16_t*>(batch.values[b]) + g * a.head_stride;
+  ctx.slot = (a.block_base + block) * kh + g;
+  const bool is_last = j == blocks_here - 1;  // this block holds row `position`
+  if (a.split_tokens == kMaxSplit) {
+    if (is_last)
+      decode_block<D, GROUP, kMaxSplit, true>(a, ctx, value_area, wave_max, wave_sum_lds, q_lds, new_row);
+    else
+      decode_block<D, GROUP, kMaxSplit, false>(a, ctx, value_area, wave_max, wave_sum_lds, q_lds, new_row);
+  } else {
+    if (is_last)
+      decode_block<D, GROUP, 0, true>(a, ctx, value_area, wave_max, wave_sum_lds, q_lds, new_row);
+    else
+      decode_block<D, GROUP, 0, false>(a, ctx, value_area, wave_max, wave_sum_lds, q_lds, new_row);
+  }
+
+  // ---- who combines: the workgroup of this (sequence, kv head) that arrives last
+  if (blocks_here > 1) {
+    // every store of this wave has been acknowledged by the memory side ...
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();  // ... and so has the whole workgroup's, before it is counted
+    if (tid == 0) {
+      unsigned* counter = a.arrivals + static_cast<long long>(seq) * kh + g;
+      const unsigned before = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED,
+                                                     __HIP_MEMORY_SCOPE_AGENT);
+      const bool final_one = before == static_cast<unsigned>(blocks_here - 1);
+      // nobody else touches the counter any more: leave it zero for the next call
+      if (final_one) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      final_flag = final_one ? 1 : 0;
+    }
+    __syncthreads();
+    if (!final_flag) return;
+    // the partial results are read below with device-scope loads, which do
+    // not take stale lines from this XCD's L2
+  } else {
+    __syncthreads();  // own partial results, read back below
+  }
+
+  // ---- combine: blocks in ascending order, kCombineChunk at a time --------
+  // LDS: m, l and then the weights of the chunk's blocks per head; running
+  // maximum, normalizer and rescale factor per head.
+  float* chunk_m = shared_area;                           // [kCombineChunk][GROUP]
+  float* chunk_l = shared_area + kCombineChunk * GROUP;   // [kCombineChunk][GROUP]
+  float* head_state = shared_area + 2 * kCombineChunk * GROUP;  // [3][GROUP]
+  static_assert((2 * kCombineChunk * GROUP + 3 * GROUP) * 4 <= value_area_bytes<D>());
+  static_assert(4 * GROUP * D * 4 <= value_area_bytes<D>());
+  constexpr int kOutputs = (GROUP * D + kThreads - 1) / kThreads;  // per thread
+  const long long first_slot = (a.block_base + batch.block_start[b]) * kh + g;
+  const long long slot_step = kh;  // consecutive blocks of one kv head
+  float o[kOutputs];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int j = j0 + 4 * u;
-      const bool valid = j < blocks;
-      const long long slot = slot0 + (valid ? j : j0) * slot_step;
-      bm[u] = valid ? a.part_m[slot] : kMasked;
-      bl[u] = a.part_l[slot];
+  for (int u = 0; u < kOutputs; ++u) o[u] = 0.0f;
+  if (tid < GROUP) {
+    head_state[0 * GROUP + tid] = kMasked;  // running maximum
+    head_state[1 * GROUP + tid] = 0.0f;     // running normalizer
+  }
+  for (int j0 = 0; j0 < blocks_here; j0 += kCombineChunk) {
+    const int count = min(kCombineChunk, blocks_here - j0);
+    __syncthreads();  // the previous chunk's weights are no longer read
+    for (int i = tid; i < count * GROUP; i += kThreads) {
+      const long long at = (first_slot + (j0 + i / GROUP) * slot_step) * GROUP + i % GROUP;
+      chunk_m[i] = load_shared(&a.part_m[at]);
+      chunk_l[i] = load_shared(&a.part_l[at]);
+    }
+    __syncthreads();
+    if (tid < GROUP) {
+      const float old_max = head_state[0 * GROUP + tid];
+      float maximum = old_max;
+      for (int jj = 0; jj < count; ++jj) maximum = fmaxf(maximum, chunk_m[jj * GROUP + tid]);
+      const float rescale = __builtin_amdgcn_exp2f(old_max - maximum);
+      float normalizer = head_state[1 * GROUP + tid] * rescale;
+      for (int jj = 0; jj < count; ++jj) {
+        const float w = __builtin_amdgcn_exp2f(chunk_m[jj * GROUP + tid] - maximum);
+        normalizer += chunk_l[jj * GROUP + tid] * w;
+        chunk_m[jj * GROUP + tid] = w;  // from here on: the block's weight
+      }
+      head_state[0 * GROUP + tid] = maximum;
+      head_state[1 * GROUP + tid] = normalizer;
+      head_state[2 * GROUP + tid] = rescale;
+    }
+    __syncthreads();
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int c = lane + 64 * i;
-        bo[u][i] = c < D ? a.part_o[slot * D + c] : 0.0f;
+    for (int u = 0; u < kOutputs; ++u) {
+      const int i = tid + u * kThreads;
+      if (i < GROUP * D) o[u] *= head_state[2 * GROUP + i / D];
+    }
+    // eight blocks per step: their loads are issued before their use
+    for (int jj = 0; jj < count; jj += 8) {
+      float part[8][kOutputs];
+#pragma unroll
+      for (int step = 0; step < 8; ++step) {
+        const int block_j = min(jj + step, count - 1);
+        const float* base = a.part_o + (first_slot + (j0 + block_j) * slot_step) * GROUP * D;
+#pragma unroll
+        for (int u = 0; u < kOutputs; ++u) {
+          const int i = tid + u * kThreads;
+          part[step][u] = i < GROUP * D ? load_shared(&base[i]) : 0.0f;
+        }
+      }
+#pragma unroll
+      for (int step = 0; step < 8; ++step) {
+        if (jj + step < count) {
+#pragma unroll
+          for (int u = 0; u < kOutputs; ++u) {
+            const int i = tid + u * kThreads;
+            if (i < GROUP * D) o[u] += part[step][u] * chunk_m[(jj + step) * GROUP + i / D];
+          }
+        }
       }
     }
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const float w = j0 + 4 * u < blocks ? __builtin_amdgcn_exp2f(bm[u] - maximum) : 0.0f;
-      normalizer += bl[u] * w;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) o[i] += bo[u][i] * w;
-    }
   }
+  // gate: cached_attention_ops.cc:119-125
 #pragma unroll
-  for (int i = 0; i < 4; ++i) partial_o[wave][lane + 64 * i] = o[i];
-  if (lane == 0) partial_l[wave] = normalizer;
-  __syncthreads();
-  const int c = threadIdx.x;
-  if (c >= D) return;
-  const float total = ((partial_l[0] + partial_l[1]) + partial_l[2]) + partial_l[3];
-  const float sum = ((partial_o[0][c] + partial_o[1][c]) + partial_o[2][c]) + partial_o[3][c];
-  const float core = sum / total;
-  const long long at = static_cast<long long>(seq) * a.query_heads + head;
-  const float logit = load_element(a.q_gate, (at * 2 + 1) * D + c, a.io_dtype);
-  const float sigmoid = 1.0f / (1.0f + expf(-logit));
-  const float value = a.round ? round_to_bf16(round_to_bf16(core) * round_to_bf16(sigmoid))
-                              : core * sigmoid;
-  store_element(a.out, at * D + c, a.io_dtype, value);
+  for (int u = 0; u < kOutputs; ++u) {
+    const int i = tid + u * kThreads;
+    if (i >= GROUP * D) continue;
+    const int hh = i / D, c = i % D;
+    const float core = o[u] / head_state[1 * GROUP + hh];
+    const long long at = static_cast<long long>(seq) * a.query_heads + g * GROUP + hh;
+    const float logit = load_element(a.q_gate, (at * 2 + 1) * D + c, a.io_dtype);
+    const float sigmoid = 1.0f / (1.0f + expf(-logit));
+    store_element(a.out, at * D + c, a.io_dtype,
+                  round_to_bf16(round_to_bf16(core) * round_to_bf16(sigmoid)));
+  }
+}
+
+__global__ void __launch_bounds__(256) decode_clear_kernel(unsigned* arrivals, int count) {
+  for (int i = blockIdx.x * 256 + threadIdx.x; i < count; i += gridDim.x * 256) arrivals[i] = 0u;
 }
 
 // Two-pass probability rows for inspection: one workgroup per (query head,
@@ -345,11 +646,11 @@ template <int D>
 int launch_for_group(hipStream_t stream, const DecodeArgs& a, const DecodeBatch& batch,
                      int group, unsigned blocks) {
   switch (group) {
-    case 1: decode_split_kernel<D, 1><<<blocks, kThreads, 0, stream>>>(a, batch); break;
-    case 2: decode_split_kernel<D, 2><<<blocks, kThreads, 0, stream>>>(a, batch); break;
-    case 4: decode_split_kernel<D, 4><<<blocks, kThreads, 0, stream>>>(a, batch); break;
-    case 6: decode_split_kernel<D, 6><<<blocks, kThreads, 0, stream>>>(a, batch); break;
-    case 8: decode_split_kernel<D, 8><<<blocks, kThreads, 0, stream>>>(a, batch); break;
+    case 1: decode_fused_kernel<D, 1><<<blocks, kThreads, 0, stream>>>(a, batch); break;
+    case 2: decode_fused_kernel<D, 2><<<blocks, kThreads, 0, stream>>>(a, batch); break;
+    case 4: decode_fused_kernel<D, 4><<<blocks, kThreads, 0, stream>>>(a, batch); break;
+    case 6: decode_fused_kernel<D, 6><<<blocks, kThreads, 0, stream>>>(a, batch); break;
+    case 8: decode_fused_kernel<D, 8><<<blocks, kThreads, 0, stream>>>(a, batch); break;
     default: return PLUTO_HIP_EUNSUPPORTED;
   }
   return launch_status();
@@ -370,6 +671,7 @@ int launch_decode_fast(hipStream_t stream, const DecodeArgs& a, const DecodeBatc
   if (blocks <= 0 || blocks > 0x7fffffffLL) return PLUTO_HIP_EINVAL;
   if (a.split_tokens < 64 || a.split_tokens > kMaxSplit || a.split_tokens % 64 != 0)
     return PLUTO_HIP_EINVAL;
+  if (a.rotary_dim / 2 > 128) return PLUTO_HIP_EUNSUPPORTED;
   if (!kernel_enabled(kMainKernel)) return 0;
   switch (a.head_dim) {
     case 64: return launch_for_group<64>(stream, a, batch, group, static_cast<unsigned>(blocks));
@@ -379,10 +681,9 @@ int launch_decode_fast(hipStream_t stream, const DecodeArgs& a, const DecodeBatc
   }
 }
 
-int launch_decode_combine(hipStream_t stream, const DecodeCombineArgs& a,
-                          const DecodeBatch& batch) {
+int launch_decode_clear(hipStream_t stream, unsigned* arrivals, int count) {
   if (!kernel_enabled(kAuxiliaryKernel)) return 0;
-  decode_combine_kernel<<<batch.count * a.query_heads, 256, 0, stream>>>(a, batch);
+  decode_clear_kernel<<<(count + 255) / 256, 256, 0, stream>>>(arrivals, count);
   return launch_status();
 }
 
