@@ -139,12 +139,13 @@ struct BlockContext {
   long long slot;    // where the block's partial results go
 };
 
-constexpr int kStageRows = 32;  // V rows per LDS stage of a wave: one contraction step
+constexpr int kStageRows = 16;  // V rows per LDS stage of a wave: one contraction step
+constexpr int kStages = 3;      // stages per wave: one in use, the others travelling
 
-// LDS of a workgroup: per wave two stages of 32 V rows (later reused for the
-// waves' partial outputs and the combine's block weights).
+// LDS of a workgroup: per wave kStages stages of 16 V rows (later reused for
+// the waves' partial outputs and the combine's block weights).
 template <int D>
-constexpr int value_area_bytes() { return 4 * 2 * kStageRows * D * 2; }
+constexpr int value_area_bytes() { return 4 * kStages * kStageRows * D * 2; }
 
 // Prepare step, split-K attention over one block and the block's partial
 // results.  SPLIT: tokens per block when known at compile time (the loops
@@ -157,17 +158,15 @@ constexpr int value_area_bytes() { return 4 * 2 * kStageRows * D * 2; }
 // end of phase 2 and waits for no other wave in between.
 //   phase 1  S^T[token, head] = K q^T for groups of 16 tokens, K rows straight
 //            from global memory into A operands.
-//   phase 2  O^T[channel, head] += V^T P^T for stages of 32 tokens
-//            (v_mfma_f32_16x16x32_bf16, one contraction step a stage).  V rows
-//            travel global -> LDS without registers (two stages a wave, the
-//            next one requested while this one is used) and are gathered into
-//            A operands by the LDS transpose read; P^T is the pair of score
-//            accumulators of the stage's two groups, so it needs no exchange.
-//            The contraction runs over (token 4q + e of the first group,
-//            e < 4; of the second group, e >= 4) for lane group q, in both
-//            operands.  Probabilities enter as bf16 hi + lo parts (two
-//            products), which keeps the FP32 arithmetic of the reference to
-//            about 2^-17.
+//   phase 2  O^T[channel, head] += V^T P^T for stages of 16 tokens
+//            (v_mfma_f32_16x16x16_bf16, one contraction step a stage).  V rows
+//            travel global -> LDS without registers (kStages stages a wave,
+//            the later ones requested while this one is used) and are gathered
+//            into A operands by the LDS transpose read; P^T is the group's
+//            score accumulator (lane group q holds tokens 4q .. 4q+3, the
+//            contraction slots of both operands), so it needs no exchange.
+//            Probabilities enter as bf16 hi + lo parts (two products), which
+//            keeps the FP32 arithmetic of the reference to about 2^-17.
 template <int D, int GROUP, int SPLIT, bool LAST>
 __device__ inline void decode_block(const DecodeArgs& a, const BlockContext& ctx,
                                     unsigned char* value_area, float (*wave_max)[16],
@@ -176,7 +175,7 @@ __device__ inline void decode_block(const DecodeArgs& a, const BlockContext& ctx
   constexpr int KSTEPS = D / 32;
   constexpr int KCH = D / 8;                       // 16-byte chunks per row
   constexpr int GROUPS = (SPLIT ? SPLIT : kMaxSplit) / 64;  // 16-token groups per wave at most
-  constexpr int STAGES = (GROUPS + 1) / 2;
+  constexpr int kAhead = 4;  // K groups requested before they are used
   constexpr int FILLS = kStageRows * KCH / 64;     // 16-byte fills per lane and stage
   constexpr int kStageBytes = kStageRows * D * 2;
   constexpr int CB = D / 16;                       // 16-channel blocks of O^T
@@ -189,11 +188,10 @@ __device__ inline void decode_block(const DecodeArgs& a, const BlockContext& ctx
   const uint16_t* keys = ctx.keys;
   const float scale2 = a.scale * kLog2e;
   const int groups = per_wave / 16;  // 16-token groups of this wave (<= GROUPS)
-  const int stages = (groups + 1) / 2;
   const int wave_t0 = t0 + wave * per_wave;
 
   // ---- the first two V stages are requested before anything else ----------
-  unsigned char* stage_base = value_area + wave * 2 * kStageBytes;
+  unsigned char* stage_base = value_area + wave * kStages * kStageBytes;
   uint32_t fill_offset[FILLS];
 #pragma unroll
   for (int i = 0; i < FILLS; ++i) fill_offset[i] = tile_fill_offset<D>(i * 64 + lane, a.token_stride);
@@ -210,10 +208,11 @@ __device__ inline void decode_block(const DecodeArgs& a, const BlockContext& ctx
     const int32x4 rsrc = make_rsrc(ctx.values + static_cast<long long>(row0) * a.token_stride, bytes);
 #pragma unroll
     for (int i = 0; i < FILLS; ++i)
-      lds_fill<16>(rsrc, stage_base + (st & 1) * kStageBytes + i * 1024, fill_offset[i]);
+      lds_fill<16>(rsrc, stage_base + (st % kStages) * kStageBytes + i * 1024, fill_offset[i]);
   };
-  fill(0);
-  if (1 < stages) fill(1);
+#pragma unroll
+  for (int st = 0; st < kStages; ++st)
+    if (st < groups) fill(st);
 
   // ---- then the first K rows ------------------------------------------------
   // A operand row = lane % 16; rows beyond the valid prefix repeat its last row
@@ -228,9 +227,9 @@ __device__ inline void decode_block(const DecodeArgs& a, const BlockContext& ctx
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) dst[ks] = load_bf16x8(row + 32 * ks);
   };
-  bf16x8 k_rows[GROUPS][KSTEPS];
+  bf16x8 k_rows[kAhead][KSTEPS];
 #pragma unroll
-  for (int grp = 0; grp < GROUPS; ++grp)
+  for (int grp = 0; grp < kAhead; ++grp)
     if (grp < groups) load_k(grp, k_rows[grp]);
 
   // ---- prepare: the group's queries, and the new cache row ----------------
@@ -290,19 +289,21 @@ __device__ inline void decode_block(const DecodeArgs& a, const BlockContext& ctx
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) k_new[ks] = load_bf16x8(&new_row[0][32 * ks + 8 * hq]);
   }
-  floatx4 s[2 * STAGES];
+  floatx4 s[GROUPS];
   float local_max = kMasked;
 #pragma unroll
-  for (int grp = 0; grp < 2 * STAGES; ++grp) {
+  for (int grp = 0; grp < GROUPS; ++grp) {
     s[grp] = floatx4{kMasked, kMasked, kMasked, kMasked};
-    if (grp < GROUPS && grp < groups) {
+    if (grp < groups) {
       floatx4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
       for (int ks = 0; ks < KSTEPS; ++ks) {
-        bf16x8 k_use = k_rows[grp][ks];
+        bf16x8 k_use = k_rows[grp % kAhead][ks];
         if constexpr (LAST) k_use = k_token(grp) == position ? k_new[ks] : k_use;
         acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k_use, qf[ks], acc, 0, 0, 0);
       }
+      // this group's registers take the rows of the group kAhead further on
+      if (grp + kAhead < groups) load_k(grp + kAhead, k_rows[grp % kAhead]);
       // accumulator register r = (token 4*hq + r of the group, head n)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
@@ -324,24 +325,28 @@ __device__ inline void decode_block(const DecodeArgs& a, const BlockContext& ctx
 #pragma unroll
   for (int cb = 0; cb < CB; ++cb) o_acc[cb] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
   float local_sum = 0.0f;
-  // transpose read of this lane: as a source it supplies row kk of its lane
-  // group's four rows, channels 4b .. 4b+3 of a 16-channel block
+  // transpose read of this lane: as a source it supplies row 4 hq + kk of the
+  // stage, channels 4b .. 4b+3 of a 16-channel block; it receives rows
+  // 4 hq .. 4 hq + 3 of channel 16 cb + lane % 16
   const int kk = (lane % 16) / 4, bsel = lane % 4;
-  int read_offset[2][CB];
-#pragma unroll
-  for (int part = 0; part < 2; ++part) {
-    const int row = 16 * part + 4 * hq + kk;
+  int read_offset[CB];
+  {
+    const int row = 4 * hq + kk;
 #pragma unroll
     for (int cb = 0; cb < CB; ++cb)
-      read_offset[part][cb] =
+      read_offset[cb] =
           (row * KCH + ((2 * cb + bsel / 2) ^ tile_swizzle(row))) * 16 + (bsel % 2) * 8;
   }
 #pragma unroll
-  for (int st = 0; st < STAGES; ++st) {
-    if (st < stages) {
-      const unsigned char* stage = stage_base + (st & 1) * kStageBytes;
-      // this stage's rows have landed (the next stage's may still travel)
-      if (st + 1 < stages)
+  for (int st = 0; st < GROUPS; ++st) {
+    if (st < groups) {
+      unsigned char* stage = stage_base + (st % kStages) * kStageBytes;
+      // this stage's rows have landed (those of the later stages may still
+      // travel: kStages - 1 of them unless the block ends first)
+      const int younger = min(kStages - 1, groups - 1 - st);
+      if (younger >= 2)
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * FILLS) : "memory");
+      else if (younger == 1)
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(FILLS) : "memory");
       else
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -350,46 +355,43 @@ __device__ inline void decode_block(const DecodeArgs& a, const BlockContext& ctx
         if (local >= 0 && local < kStageRows) {
           // the appended V row: from LDS to its place in the stage
           if (lane < KCH)
-            *reinterpret_cast<uint4*>(const_cast<unsigned char*>(stage) +
-                                      (local * KCH + (lane ^ tile_swizzle(local))) * 16) =
+            *reinterpret_cast<uint4*>(stage + (local * KCH + (lane ^ tile_swizzle(local))) * 16) =
                 *reinterpret_cast<const uint4*>(&new_row[1][8 * lane]);
           asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         }
       }
       __builtin_amdgcn_wave_barrier();
-      // P^T of the stage's two groups as hi + lo bf16 B operands
-      float p[8];
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const float score = s[2 * st + e / 4][e % 4];
-        // (a wave whose tokens all lie beyond the sequence has local_max ==
-        // kMasked: its probabilities are zero, not 2^0)
-        p[e] = score == kMasked ? 0.0f : __builtin_amdgcn_exp2f(score - local_max);
-        local_sum += p[e];
-      }
-      uint32_t hi[4], lo[4];
+      // P^T of the stage's group as hi + lo bf16 B operands
+      float p[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
+        const float score = s[st][e];
+        // (a wave whose tokens all lie beyond the sequence has local_max ==
+        // kMasked: its probabilities are zero, not 2^0)
+        p[e] = (LAST && score == kMasked) ? 0.0f : __builtin_amdgcn_exp2f(score - local_max);
+        local_sum += p[e];
+      }
+      uint32_t hi[2], lo[2];
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
         hi[e] = pack_bf16(p[2 * e], p[2 * e + 1]);
         lo[e] = pack_bf16(p[2 * e] - __uint_as_float(hi[e] << 16),
                           p[2 * e + 1] - __uint_as_float(hi[e] & 0xffff0000u));
       }
-      const bf16x8 p_hi = __builtin_bit_cast(bf16x8, make_uint4(hi[0], hi[1], hi[2], hi[3]));
-      const bf16x8 p_lo = __builtin_bit_cast(bf16x8, make_uint4(lo[0], lo[1], lo[2], lo[3]));
+      const shortx4 p_hi = __builtin_bit_cast(shortx4, make_uint2(hi[0], hi[1]));
+      const shortx4 p_lo = __builtin_bit_cast(shortx4, make_uint2(lo[0], lo[1]));
 #pragma unroll
       for (int cb = 0; cb < CB; ++cb) {
-        const uint2 first = lds_transpose_read(stage, read_offset[0][cb]);
-        const uint2 second = lds_transpose_read(stage, read_offset[1][cb]);
-        const bf16x8 v_t =
-            __builtin_bit_cast(bf16x8, make_uint4(first.x, first.y, second.x, second.y));
-        o_acc[cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_t, p_hi, o_acc[cb], 0, 0, 0);
-        o_acc[cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_t, p_lo, o_acc[cb], 0, 0, 0);
+        const shortx4 v_t =
+            __builtin_bit_cast(shortx4, lds_transpose_read(stage, read_offset[cb]));
+        o_acc[cb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(v_t, p_hi, o_acc[cb], 0, 0, 0);
+        o_acc[cb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(v_t, p_lo, o_acc[cb], 0, 0, 0);
       }
-      // the stage after next takes this stage's place
-      if (st + 2 < stages) {
+      // the stage kStages further on takes this stage's place
+      if (st + kStages < groups) {
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_wave_barrier();
-        fill(st + 2);
+        fill(st + kStages);
       }
     }
   }
@@ -434,7 +436,7 @@ __device__ inline void decode_block(const DecodeArgs& a, const BlockContext& ctx
 
 template <int D, int GROUP>
 __global__ void __launch_bounds__(kThreads)
-__attribute__((amdgpu_waves_per_eu(D == 256 ? 1 : 2, D == 256 ? 1 : 2)))
+__attribute__((amdgpu_waves_per_eu(D == 256 ? 1 : 3, D == 256 ? 1 : 3)))
 decode_fused_kernel(DecodeArgs a, DecodeBatch batch) {
   __shared__ __attribute__((aligned(1024))) unsigned char value_area[value_area_bytes<D>()];
   float* shared_area = reinterpret_cast<float*>(value_area);
