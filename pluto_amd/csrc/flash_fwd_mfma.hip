@@ -75,7 +75,12 @@ template <int D, int G, int WAVES>
 __global__ void __launch_bounds__(64 * WAVES)
 __attribute__((amdgpu_waves_per_eu(Config<D, G, WAVES>::kOccupancy,
                                    Config<D, G, WAVES>::kOccupancy)))
-flash_forward_kernel(FlashForwardArgs a) {
+flash_forward_kernel(FlashForwardArgs a_in, int unit_count) {
+  struct Args : FlashForwardArgs {
+    int unit_count;
+  } a;
+  static_cast<FlashForwardArgs&>(a) = a_in;
+  a.unit_count = unit_count;
   using C = Config<D, G, WAVES>;
   constexpr int KCH = C::KCH;
   constexpr int KS = D / 16;   // contraction steps of S^T
@@ -106,10 +111,20 @@ flash_forward_kernel(FlashForwardArgs a) {
     head = (logical / pairs) % a.query_heads;
     seq = logical / (pairs * a.query_heads);
   } else {
-    const int units = gridDim.x / q_tiles;  // (sequence, head) pairs
-    pair = q_tiles - 1 - blockIdx.x / units;
-    head = (blockIdx.x % units) % a.query_heads;
-    seq = (blockIdx.x % units) / a.query_heads;
+    // The `group` query heads that share a (sequence, kv head) at one query
+    // tile form a unit u; XCD x works on u = x, x + 8, ... in that order, so
+    // the heads that stream the same K/V rows do so from the same L2 at the
+    // same time.  u counts query tiles from the heaviest (last) down, kv heads
+    // fastest; the grid is padded to a multiple of 8 units.
+    const int kv_heads = a.query_heads / a.group;
+    const int kv_units = a.unit_count / q_tiles;  // (sequence, kv head) pairs
+    const int xcd = blockIdx.x % 8, slot = blockIdx.x / 8;
+    const int u = 8 * (slot / a.group) + xcd;
+    if (u >= a.unit_count) return;
+    pair = q_tiles - 1 - u / kv_units;
+    const int kv_unit = u % kv_units;
+    head = (kv_unit % kv_heads) * a.group + slot % a.group;
+    seq = kv_unit / kv_heads;
   }
   const int kv_head = head / a.group;
 
@@ -406,16 +421,21 @@ bool flash_forward_supported(const FlashForwardArgs& a, int head_dim) {
 int launch_flash_forward(hipStream_t stream, const FlashForwardArgs& a,
                          int head_dim, int sequences) {
   if (!flash_forward_supported(a, head_dim)) return PLUTO_HIP_EUNSUPPORTED;
-  const long long blocks = grid_blocks(a, 128, sequences, head_dim == 64);
-  if (blocks <= 0 || blocks > 0x7fffffffLL) return PLUTO_HIP_EINVAL;
+  long long blocks = grid_blocks(a, 128, sequences, head_dim == 64);
+  // unpaired schedule: units of `group` heads, dealt to the 8 XCDs
+  const long long q_tiles = (a.q_rows + 127) / 128;
+  const long long units = q_tiles * sequences * (a.query_heads / a.group);
+  if (head_dim != 64) blocks = (units + 7) / 8 * 8 * a.group;
+  if (blocks <= 0 || blocks > 0x7fffffffLL || units > 0x7fffffffLL) return PLUTO_HIP_EINVAL;
   const dim3 grid(static_cast<unsigned>(blocks));
+  const int unit_count = static_cast<int>(units);
   if (!kernel_enabled(kMainKernel)) return 0;
   if (head_dim == 256)
-    flash_forward_kernel<256, 1, 4><<<grid, 256, 0, stream>>>(a);
+    flash_forward_kernel<256, 1, 4><<<grid, 256, 0, stream>>>(a, unit_count);
   else if (head_dim == 128)
-    flash_forward_kernel<128, 1, 4><<<grid, 256, 0, stream>>>(a);
+    flash_forward_kernel<128, 1, 4><<<grid, 256, 0, stream>>>(a, unit_count);
   else
-    flash_forward_kernel<64, 1, 4><<<grid, 256, 0, stream>>>(a);
+    flash_forward_kernel<64, 1, 4><<<grid, 256, 0, stream>>>(a, unit_count);
   return launch_status();
 }
 
