@@ -6,7 +6,7 @@ matrix-core kernels."""
 import numpy as np
 import pytest
 
-from tests.util import assert_close, assert_close_bf16
+from tests.util import assert_close, assert_close_bf16_gradient
 
 pytestmark = pytest.mark.gpu
 
@@ -93,7 +93,7 @@ def test_matrix_core_kernels_match_oracle(capi, shape):
     T, qh, kh, d, rot = shape
     got, want, _, _ = run_case(capi, T, qh, kh, d, rot, True, seed=T + d)
     for name in ("dqg", "dk", "dv", "dq_norm", "dk_norm"):
-        assert_close_bf16(got[name], want[name], "%s T%d d%d" % (name, T, d))
+        assert_close_bf16_gradient(got[name], want[name], "%s T%d d%d" % (name, T, d))
 
 
 @pytest.mark.parametrize("shape", [(200, 8, 2, 64, 32), (333, 6, 2, 128, 64)])
@@ -119,7 +119,7 @@ def test_state_saved_by_forward_gives_the_recomputed_gradients(capi, shape):
         # only in where K and V are read from
         np.testing.assert_allclose(value.cpu().numpy(), got[name], rtol=1e-5, atol=1e-6,
                                    err_msg=name)
-        assert_close_bf16(value.cpu().numpy(), want[name], "%s T%d d%d" % (name, T, d))
+        assert_close_bf16_gradient(value.cpu().numpy(), want[name], "%s T%d d%d" % (name, T, d))
 
 
 def test_saved_state_is_refused_where_none_is_kept(capi):

@@ -7,7 +7,8 @@ import os
 import numpy as np
 import pytest
 
-from tests.util import assert_close, assert_close_bf16, from_bf16_bits, to_bf16_bits
+from tests.util import (assert_close, assert_close_bf16, assert_close_bf16_gradient,
+                        beyond_reference_tolerance, from_bf16_bits, to_bf16_bits)
 
 pytestmark = pytest.mark.gpu
 
@@ -60,6 +61,8 @@ def check(capi, oracle, T, H, E, B, bf16, seed, qk_scale=1.0):
     got = run_device(capi, x, d_out, T, H, bf16)
     want = run_oracle(oracle, x, d_out, T, H, bf16)
     tag = "T%d H%d E%d B%d %s" % (T, H, E, B, "bf16" if bf16 else "fp32")
+    # peaked scores leave most gradients tiny next to the few large ones
+    gradient_outliers = 2e-2 if qk_scale > 1 else 2e-3
     lse_got = got[1] + np.log(got[2])
     lse_want = want[1] + np.log(want[2])
     # the saved maximum itself is part of the layer state (attention.cc:161-168), not only
@@ -68,7 +71,7 @@ def check(capi, oracle, T, H, E, B, bf16, seed, qk_scale=1.0):
     if bf16:
         assert_close_bf16(got[0], want[0], tag + " out")
         assert_close(lse_got, lse_want, 1e-3, tag + " lse")
-        assert_close_bf16(got[3], want[3], tag + " d_qkv")
+        assert_close_bf16_gradient(got[3], want[3], tag + " d_qkv", outliers=gradient_outliers)
         return
     # peaked scores: the reference's own tolerance (attention_reference_test.cc:56-73)
     rel = 2e-3 if qk_scale > 1 else FP32_REL
@@ -109,6 +112,36 @@ def test_three_odd_heads(capi, oracle):
 def test_production_context_one_head(capi, oracle, bf16):
     # attention_reference_test.cc:171-176: T=1024, one 64-wide head
     check(capi, oracle, 1024, 1, 64, 1, bf16, seed=9)
+
+
+REFERENCE_BF16_CASES = [(33, 2, 64, 2), (33, 2, 128, 2), (65, 2, 64, 2), (65, 2, 128, 2),
+                        (65, 2, 256, 2), (1024, 1, 64, 1)]
+
+
+@pytest.mark.parametrize("T,H,E,B", REFERENCE_BF16_CASES)
+def test_reference_device_tolerance_on_its_bf16_cases(capi, oracle, T, H, E, B):
+    """The reference's own device-vs-CPU test (attention_reference_test.cc:19-73) with
+    its inputs (0.35 sin + 0.05 cos; upstream gradient 0.2 cos) and its bounds,
+    2e-3 + 2e-3|x| forward and 3e-3 + 3e-3|x| backward, on the bf16 cases whose heads
+    the matrix-core kernels serve.  The reference keeps P in FP32; these kernels
+    round P, dS and dO to bf16 for the matrix cores, so a fraction of the elements
+    could lie beyond the reference's bound; on the reference's inputs none does."""
+    index = np.arange(B * T * 3 * E, dtype=np.float32)
+    x = (np.float32(0.35) * np.sin(index * np.float32(0.071)) +
+         np.float32(0.05) * np.cos(index * np.float32(0.19))).astype(np.float32).reshape(B * T, 3 * E)
+    index = np.arange(B * T * E, dtype=np.float32)
+    d_out = (np.float32(0.2) * np.cos(index * np.float32(0.13))).astype(np.float32).reshape(B * T, E)
+    got = run_device(capi, x, d_out, T, H, True)
+    want = run_oracle(oracle, x, d_out, T, H, True)
+    forward = beyond_reference_tolerance(got[0], want[0], 2e-3, 2e-3)
+    backward = beyond_reference_tolerance(got[3], want[3], 3e-3, 3e-3)
+    print("T%d H%d E%d B%d: %.3f %% of the outputs beyond 2e-3 + 2e-3|x| (max-abs %.2e), "
+          "%.3f %% of the gradients beyond 3e-3 + 3e-3|x| (max-abs %.2e)" % (
+              T, H, E, B, 100 * forward, np.abs(got[0] - want[0]).max(), 100 * backward,
+              np.abs(got[3] - want[3]).max()))
+    assert forward == 0.0 and backward == 0.0
+    assert_close_bf16(got[0], want[0], "reference case out")
+    assert_close_bf16_gradient(got[3], want[3], "reference case d_qkv")
 
 
 def test_mfma_heads_of_128(capi, oracle):
@@ -221,7 +254,7 @@ def test_config2_gpt2_small_forward_backward_bf16(capi, oracle):
         g = d_qkv[rows].cpu().numpy()
         for part, name in ((0, "dQ"), (1, "dK"), (2, "dV")):
             c = slice(part * E + head * D, part * E + (head + 1) * D)
-            assert_close_bf16(g[:, c], want_g[rows, c], tag + name)
+            assert_close_bf16_gradient(g[:, c], want_g[rows, c], tag + name)
     with capi.force_generic():
         out2, m2, n2 = capi.mha_forward(xt, T, H)
         d2 = capi.mha_backward(xt, out2, gt, m2, n2, T, H)
@@ -230,7 +263,7 @@ def test_config2_gpt2_small_forward_backward_bf16(capi, oracle):
     g1, g2 = d_qkv.cpu().numpy(), d2.cpu().numpy()
     for part, name in ((0, "dQ"), (1, "dK"), (2, "dV")):
         c = slice(part * E, (part + 1) * E)
-        assert_close_bf16(g1[:, c], g2[:, c], "config 2 %s vs fp32-arithmetic kernel" % name)
+        assert_close_bf16_gradient(g1[:, c], g2[:, c], "config 2 %s vs fp32-arithmetic kernel" % name)
 
 
 def test_rejects_bad_arguments_before_any_work(capi):
