@@ -3,6 +3,8 @@
 // src/llm/layers/util/cached_attention_ops_test.cc, cached_attention_test.cc,
 // qwen_attention_test.cc and sequence_delta_net_test.cc.
 #include <algorithm>
+#include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <limits>
 
@@ -368,9 +370,14 @@ StatusOr<std::shared_ptr<BlockParameter>> Parameter(hip::Executor& executor,
 }
 
 TEST(QwenAttentionTest, ForwardMatchesCachedAttentionAndCausalHook) {
-  // qwen_attention_test.cc:155-228.  The sequence path (flash tiles) and the
-  // cached path (split-K) sum in different orders, so outputs agree to one
-  // bf16 ulp instead of bitwise.
+  // qwen_attention_test.cc:155-228.  The reference compares the two paths bit
+  // for bit.  Here the sequence path (flash tiles, bf16 probabilities) and the
+  // cached path (split-K, FP32-accurate probabilities) sum in different
+  // orders, so bf16(core) can land on either side of a rounding boundary and
+  // the gated product bf16(bf16(core) * bf16(gate)) then moves by up to two
+  // units in the last place in general.  On the reference's own cases the two
+  // paths do agree bit for bit, and that is what is asserted, as in the
+  // reference (the counts are printed).
   auto executor = NewExecutor();
   for (int d : {3, 256, 128}) {
     FullAttentionParameters p;
@@ -419,6 +426,7 @@ TEST(QwenAttentionTest, ForwardMatchesCachedAttentionAndCausalHook) {
       ASSERT_TRUE(cache.ok());
       auto cached_layer = QwenAttentionLayer::Create(*executor, p, *qw, *kw, 1, cache->get());
       ASSERT_TRUE(cached_layer.ok());
+      int differing = 0, compared = 0, worst = 0;
       for (int row = 0; row < length; ++row) {
         auto qi = Upload<BFloat16>(*executor, {qg.begin() + row * 4 * d, qg.begin() + (row + 1) * 4 * d});
         auto ki = Upload<BFloat16>(*executor, {k.begin() + row * d, k.begin() + (row + 1) * d});
@@ -427,10 +435,21 @@ TEST(QwenAttentionTest, ForwardMatchesCachedAttentionAndCausalHook) {
         ASSERT_TRUE(output.ok());
         EXPECT_EQ((*cache)->position(), row + 1);
         const auto expected = Read<BFloat16>(output->outputs[0]);
-        for (int c = 0; c < 2 * d; ++c)
-          EXPECT_NEAR(actual[row * 2 * d + c], expected[c], 2e-4 + 1.6e-2 * std::fabs(expected[c]))
-              << "d=" << d << " row=" << row << " c=" << c;
+        for (int c = 0; c < 2 * d; ++c) {
+          // bf16 bit patterns as integers that count representable values
+          auto ordered = [](BFloat16 bits) {
+            return (bits & 0x8000) ? -static_cast<int>(bits & 0x7fff) : static_cast<int>(bits);
+          };
+          const int ulps = std::abs(ordered(actual[row * 2 * d + c]) - ordered(expected[c]));
+          EXPECT_LE(ulps, 2) << "d=" << d << " row=" << row << " c=" << c;
+          differing += ulps != 0;
+          worst = std::max(worst, ulps);
+          ++compared;
+        }
       }
+      std::printf("sequence vs cached path, d=%d: %d of %d outputs differ, by at most %d bf16 ulp\n",
+                  d, differing, compared, worst);
+      EXPECT_EQ(differing, 0);
     }
   }
 }
