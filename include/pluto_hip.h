@@ -526,6 +526,19 @@ int pluto_hip_test_force_generic(int enabled);
  * like it written by nothing on the product path. */
 unsigned pluto_hip_test_kernel_classes(unsigned mask);
 
+/* Which family of kernels the calling thread's most recent compute call chose
+ * (the entry points fall back to the any-shape kernels when a shape, stride
+ * or alignment rules the specialised ones out; tests assert that the
+ * configurations the library is built for do not).  Thread-local. */
+#define PLUTO_HIP_PATH_NONE 0
+#define PLUTO_HIP_PATH_GENERIC 1      /* any shape, FP32 arithmetic */
+#define PLUTO_HIP_PATH_MATRIX_F32 2   /* FP32 storage on the FP32 matrix cores */
+#define PLUTO_HIP_PATH_FLASH 3        /* bf16 flash attention on the matrix cores */
+#define PLUTO_HIP_PATH_SPLIT_K 4      /* fused split-K decode */
+#define PLUTO_HIP_PATH_CHUNKED 5      /* chunked delta-net (forward scan or backward) */
+#define PLUTO_HIP_PATH_RECURRENCE 6   /* token-by-token delta-net */
+int pluto_hip_test_last_path(void);
+
 #ifdef __cplusplus
 }
 #endif

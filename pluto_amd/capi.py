@@ -70,6 +70,7 @@ SIGNATURES = {
     "pluto_hip_error_string": (ctypes.c_char_p, [_I]),
     "pluto_hip_test_force_generic": (_I, [_I]),
     "pluto_hip_test_kernel_classes": (ctypes.c_uint, [ctypes.c_uint]),
+    "pluto_hip_test_last_path": (_I, []),
     "pluto_hip_abi_version": (_I, []),
     "pluto_hip_target_arch": (ctypes.c_char_p, []),
     "pluto_hip_executor_create": (_I, [ctypes.POINTER(_VP)]),
@@ -174,6 +175,13 @@ class force_generic:
 
 
 MAIN_KERNEL, QUERY_KERNEL, AUXILIARY_KERNELS = 1, 2, 4
+(PATH_NONE, PATH_GENERIC, PATH_MATRIX_F32, PATH_FLASH, PATH_SPLIT_K, PATH_CHUNKED,
+ PATH_RECURRENCE) = range(7)
+
+
+def last_path():
+    """Kernel family the calling thread's most recent compute call chose."""
+    return lib().pluto_hip_test_last_path()
 
 
 class only_kernels:

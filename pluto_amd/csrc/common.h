@@ -101,6 +101,8 @@ enum KernelClass : unsigned {
   kAuxiliaryKernel = 4u,  // preparation, tables, combines
 };
 bool kernel_enabled(KernelClass which);  // mha_capi.hip
+// Records the kernel family a compute call chose (pluto_hip_test_last_path).
+void note_path(int path);  // mha_capi.hip
 
 inline size_t align_up(size_t value, size_t alignment) {
   return (value + alignment - 1) / alignment * alignment;

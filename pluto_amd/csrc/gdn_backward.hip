@@ -612,6 +612,7 @@ int launch_gdn_backward(hipStream_t stream, const pluto_hip_delta_params* p, int
                         const float* norm, const float* dy, float* dqkv, float* dz, float* da,
                         float* db, float* d_conv_weight, float* d_a_log, float* d_dt_bias,
                         float* d_norm, void* workspace) {
+  note_path(use_chunks(p) ? PLUTO_HIP_PATH_CHUNKED : PLUTO_HIP_PATH_RECURRENCE);
   const size_t T = static_cast<size_t>(length);
   const int kh = p->key_heads, vh = p->value_heads, kd = p->key_head_dim, vd = p->value_head_dim;
   const int channels = 2 * kh * kd + vh * vd, kernel = p->conv_kernel_dim;

@@ -102,8 +102,10 @@ int pluto_hip_gdn_scan(void* stream, const pluto_hip_delta_params* p, int batch,
   if (!force_generic() && workspace != nullptr && gdn_chunked_supported(a, 64)) {
     const size_t needed = pluto_hip_gdn_scan_workspace_bytes(p, batch, length, 64);
     if (workspace_bytes < needed) return PLUTO_HIP_EWORKSPACE;
+    note_path(PLUTO_HIP_PATH_CHUNKED);
     return launch_gdn_chunked(s, a);
   }
+  note_path(PLUTO_HIP_PATH_RECURRENCE);
   return launch_gdn_recurrence(s, a, PLUTO_HIP_BF16);
 }
 
@@ -178,7 +180,9 @@ int pluto_hip_gdn_layer_forward(void* stream, const pluto_hip_delta_params* p, i
   g.normalize_qk = 1;  // sequence_delta_net.cc:84-85
   g.round_output = round;
   g.q_scale = 1.0f / std::sqrt(static_cast<float>(kd));
-  if (round && !force_generic() && gdn_chunked_supported(g, 64))
+  const bool chunked = round && !force_generic() && gdn_chunked_supported(g, 64);
+  note_path(chunked ? PLUTO_HIP_PATH_CHUNKED : PLUTO_HIP_PATH_RECURRENCE);
+  if (chunked)
     status = launch_gdn_chunked(s, g);
   else
     status = launch_gdn_recurrence(s, g, mid_dtype);

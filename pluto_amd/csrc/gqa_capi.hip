@@ -269,7 +269,10 @@ int pluto_hip_gqa_prefill(void* stream, const pluto_hip_attention_params* p, int
     f.query_heads = qh;
     f.group = qh / kh;
     f.scale = scale;
-    if (flash_forward_supported(f, d)) return launch_flash_forward(s, f, d, 1);
+    if (flash_forward_supported(f, d)) {
+      note_path(PLUTO_HIP_PATH_FLASH);
+      return launch_flash_forward(s, f, d, 1);
+    }
     if (saved) return PLUTO_HIP_EUNSUPPORTED;
   }
   GenericForwardArgs a;
@@ -290,6 +293,7 @@ int pluto_hip_gqa_prefill(void* stream, const pluto_hip_attention_params* p, int
   a.head_dim = d;
   a.scale = scale;
   a.round_to_bf16 = round;
+  note_path(PLUTO_HIP_PATH_GENERIC);
   return launch_generic_forward(s, a, 1);
 }
 
@@ -575,6 +579,7 @@ static int decode_run(void* stream, const pluto_hip_attention_params* p, int bat
   const int q_dtype = round ? PLUTO_HIP_BF16 : PLUTO_HIP_F32;
   const float scale = 1.0f / std::sqrt(static_cast<float>(d));
   const size_t io_bytes = element_bytes(io_dtype);
+  note_path(fast ? PLUTO_HIP_PATH_SPLIT_K : PLUTO_HIP_PATH_GENERIC);
 
   if (fast && clear_arrivals) {
     status = launch_decode_clear(s, reinterpret_cast<unsigned*>(area + layout.arrivals),

@@ -22,6 +22,10 @@ bool force_generic() { return force_generic_flag.load(std::memory_order_relaxed)
 namespace {
 std::atomic<unsigned> kernel_class_mask{~0u};
 }
+namespace {
+thread_local int last_path = PLUTO_HIP_PATH_NONE;
+}
+void note_path(int path) { last_path = path; }
 bool kernel_enabled(KernelClass which) {
   return (kernel_class_mask.load(std::memory_order_relaxed) & which) != 0;
 }
@@ -81,6 +85,8 @@ int pluto_hip_test_force_generic(int enabled) {
 
 unsigned pluto_hip_test_kernel_classes(unsigned mask) { return kernel_class_mask.exchange(mask); }
 
+int pluto_hip_test_last_path(void) { return last_path; }
+
 int pluto_hip_mha_forward(void* stream, int dtype, const void* qkv, int rows,
                           int context_length, int num_heads, int embedding_dim,
                           void* out, float* maxima, float* normalizers) {
@@ -110,12 +116,18 @@ int pluto_hip_mha_forward(void* stream, int dtype, const void* qkv, int rows,
     f.query_heads = H;
     f.group = 1;
     f.scale = 1.0f / std::sqrt(static_cast<float>(D));
-    if (flash_forward_supported(f, D))
+    if (flash_forward_supported(f, D)) {
+      note_path(PLUTO_HIP_PATH_FLASH);
       return launch_flash_forward(s, f, D, sequences);
+    }
   }
   const GenericForwardArgs a =
       packed_forward_args(dtype, qkv, rows, T, H, E, out, maxima, normalizers);
-  if (!force_generic() && f32_forward_supported(a)) return launch_f32_forward(s, a, sequences);
+  if (!force_generic() && f32_forward_supported(a)) {
+    note_path(PLUTO_HIP_PATH_MATRIX_F32);
+    return launch_f32_forward(s, a, sequences);
+  }
+  note_path(PLUTO_HIP_PATH_GENERIC);
   return launch_generic_forward(s, a, sequences);
 }
 
@@ -184,9 +196,11 @@ int pluto_hip_mha_backward(void* stream, int dtype, const void* qkv,
     const size_t stats =
         align_up(static_cast<size_t>(rows) * num_heads * sizeof(float), 256);
     char* scratch = static_cast<char*>(workspace);
+    note_path(PLUTO_HIP_PATH_FLASH);
     return launch_flash_backward(s, a, reinterpret_cast<float*>(scratch + stats),
                                  reinterpret_cast<uint16_t*>(scratch + 2 * stats));
   }
+  note_path(PLUTO_HIP_PATH_GENERIC);
   return launch_generic_backward(s, a);
 }
 

@@ -161,6 +161,50 @@ def test_chunked_and_token_by_token_kernels_agree(capi):
         assert_close(chunked[name], sequential[name], 2e-4, name)
 
 
+def test_long_sequence_two_heads_matches_oracle(capi):
+    """T=2048 (32 chunks), two 128 x 128 heads: the length bench.py times, at a head
+    count the scalar oracle finishes in seconds.  The chunked kernels treat heads
+    independently (one workgroup row per head)."""
+    shape = (2048, 2, 2, 128, 128, 4)
+    got, want, _, _ = run(capi, shape, False, seed=5)
+    assert capi.last_path() == capi.PATH_CHUNKED
+    for name in want:
+        assert_close(got[name], want[name], 2e-4, "%s %s" % (name, shape))
+
+
+def test_benchmarked_shape_against_token_by_token_kernels(capi):
+    """The shape bench.py times (T=2048, sixteen 128 x 128 heads, every parameter
+    trains): the chunked kernels against the token-by-token kernels of the same
+    library, FP32 both."""
+    shape = (2048, 16, 16, 128, 128, 4)
+    T, kh, vh, kd, vd, K = shape
+    p = capi.delta_params(key_heads=kh, value_heads=vh, key_head_dim=kd, value_head_dim=vd,
+                          conv_kernel_dim=K, round_to_bfloat16=False)
+    c = make_case(T, kh, vh, kd, vd, K, seed=4)
+    bf = torch.bfloat16
+    args = (p, dev(c["qkv"], bf), dev(c["z"], bf), dev(c["a"], bf), dev(c["b"], bf), dev(c["conv"]),
+            dev(c["a_log"]), dev(c["dt_bias"]), dev(c["norm"]), dev(c["dy"]))
+    channels = 2 * kh * kd + vh * vd
+
+    def once():
+        grads = dict(conv_weight=torch.zeros(channels, K, device="cuda"),
+                     a_log=torch.zeros(vh, device="cuda"), dt_bias=torch.zeros(vh, device="cuda"),
+                     norm=torch.zeros(vd, device="cuda"))
+        out = capi.gdn_layer_backward(*args, parameter_grads=grads)
+        torch.cuda.synchronize()
+        named = dict(zip(("dqkv", "dz", "da", "db"), out))
+        named.update(grads)
+        return {k: v.cpu().numpy() for k, v in named.items()}
+
+    chunked = once()
+    assert capi.last_path() == capi.PATH_CHUNKED
+    with capi.force_generic():
+        sequential = once()
+        assert capi.last_path() == capi.PATH_RECURRENCE
+    for name in sequential:
+        assert_close(chunked[name], sequential[name], 2e-4, name)
+
+
 def test_rejects_bad_arguments(capi):
     import ctypes
     p = capi.delta_params(key_heads=1, value_heads=2, key_head_dim=4, value_head_dim=6,

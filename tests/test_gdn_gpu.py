@@ -145,6 +145,7 @@ def test_config5_chunked_scan(capi, oracle):
     dq, dk, dv, dg, db = dev(q, bf), dev(k, bf), dev(v, bf), dev(g), dev(beta)
     state = dev(state0.astype(np.float32))
     out = capi.gdn_scan(p, dq, dk, dv, dg, db, state, q_scale=scale, chunk=64)
+    assert capi.last_path() == capi.PATH_CHUNKED
     torch.cuda.synchronize()
     got, got_state = out.float().cpu().numpy(), state.cpu().numpy()
     # CPU recurrence on whole (sequence, head) chains (they are independent)

@@ -122,6 +122,66 @@ def test_state_saved_by_forward_gives_the_recomputed_gradients(capi, shape):
         assert_close_bf16_gradient(value.cpu().numpy(), want[name], "%s T%d d%d" % (name, T, d))
 
 
+def test_long_sequence_with_saved_state_matches_oracle(capi):
+    """T=1024, one kv group of six 128-wide heads (the grouping of the benchmarked
+    shape): eight query tiles, so the unpaired heaviest-first grid, with the block
+    the forward pass saves.  Every gradient against the oracle."""
+    T, qh, kh, d, rot = 1024, 6, 1, 128, 32
+    got, want, args, _ = run_case(capi, T, qh, kh, d, rot, True, seed=77)
+    assert capi.last_path() == capi.PATH_FLASH
+    p, qg, k, v, qw, kw_, dy = args
+    cache = capi.KvCache(T, kh, d)
+    saved = capi.gqa_prefill_saved(p, T, cache)
+    capi.gqa_prefill(p, qg, k, v, qw, kw_, cache, saved=saved)
+    dq_norm, dk_norm = torch.zeros(d, device="cuda"), torch.zeros(d, device="cuda")
+    dqg, dk, dv = capi.gqa_prefill_backward(p, qg, k, v, qw, kw_, dy, dq_norm=dq_norm,
+                                            dk_norm=dk_norm, saved=saved)
+    torch.cuda.synchronize()
+    assert capi.last_path() == capi.PATH_FLASH
+    with_saved = dict(dqg=dqg, dk=dk, dv=dv, dq_norm=dq_norm, dk_norm=dk_norm)
+    for name, value in with_saved.items():
+        assert_close_bf16_gradient(got[name], want[name], "%s T%d self-contained" % (name, T))
+        assert_close_bf16_gradient(value.cpu().numpy(), want[name], "%s T%d saved" % (name, T))
+
+
+def test_benchmarked_shape_against_fp32_kernels(capi):
+    """The shape bench.py times (T=8192, 24 query / 4 kv heads of 128, saved block):
+    the matrix-core kernels against the any-shape FP32-arithmetic kernels of the same
+    library.  The CPU oracle would need an hour for this length; it covers the same
+    kernels at T=1024 above."""
+    T, qh, kh, d, rot = 8192, 24, 4, 128, 32
+    p = capi.attention_params(query_heads=qh, key_value_heads=kh, head_dim=d, rotary_dim=rot,
+                              capacity=T, round_to_bfloat16=True)
+    gen = torch.Generator(device="cuda").manual_seed(2)
+    bf = torch.bfloat16
+    qg = (0.5 * torch.randn((T, qh, 2, d), generator=gen, device="cuda")).to(bf)
+    k = (0.5 * torch.randn((T, kh, d), generator=gen, device="cuda")).to(bf)
+    v = (0.5 * torch.randn((T, kh, d), generator=gen, device="cuda")).to(bf)
+    dy = torch.randn((T, qh, d), generator=gen, device="cuda")
+    qw, kw_ = dev(values(d, 0.2, 0.3)), dev(values(d, 0.8, 0.4))
+
+    def once(saved):
+        dq_norm, dk_norm = torch.zeros(d, device="cuda"), torch.zeros(d, device="cuda")
+        dqg, dk, dv = capi.gqa_prefill_backward(p, qg, k, v, qw, kw_, dy, dq_norm=dq_norm,
+                                                dk_norm=dk_norm, saved=saved)
+        torch.cuda.synchronize()
+        return dict(dqg=dqg, dk=dk, dv=dv, dq_norm=dq_norm, dk_norm=dk_norm)
+
+    cache = capi.KvCache(T, kh, d)
+    saved = capi.gqa_prefill_saved(p, T, cache)
+    capi.gqa_prefill(p, qg, k, v, qw, kw_, cache, saved=saved)
+    fast = once(saved)
+    assert capi.last_path() == capi.PATH_FLASH
+    with capi.force_generic():
+        slow = once(None)
+        assert capi.last_path() == capi.PATH_GENERIC
+    for name in fast:
+        # (fifty million elements: the tail of the per-element error reaches further
+        # than in the small cases; the max-norm bound still holds for every element)
+        assert_close_bf16_gradient(fast[name].cpu().numpy(), slow[name].cpu().numpy(),
+                                   "%s T%d vs fp32-arithmetic kernels" % (name, T), far=50.0)
+
+
 def test_saved_state_is_refused_where_none_is_kept(capi):
     T, qh, kh, d, rot = 16, 2, 1, 32, 8
     kw = dict(query_heads=qh, key_value_heads=kh, head_dim=d, rotary_dim=rot, capacity=T,

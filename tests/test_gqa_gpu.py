@@ -272,6 +272,7 @@ def test_config3_prefill_8192(capi, oracle):
     bf = torch.bfloat16
     dq, dk, dv = dev(qg, bf), dev(k, bf), dev(v, bf)
     out = capi.gqa_prefill(p, dq, dk, dv, dev(qw), dev(kw_), cache)
+    assert capi.last_path() == capi.PATH_FLASH
     torch.cuda.synchronize()
     got = out.float().cpu().numpy()
     # oracle on sampled whole rows (every row is an independent softmax)
@@ -314,6 +315,7 @@ def test_config4_batched_decode(capi, oracle):
     bf = torch.bfloat16
     out = capi.gqa_decode(p, dev(q_gate, bf), dev(k, bf), dev(v, bf), dev(qw), dev(kw_), caches,
                           split_tokens=512, advance=False)
+    assert capi.last_path() == capi.PATH_SPLIT_K
     torch.cuda.synchronize()
     got = out.float().cpu().numpy()
     assert np.all(np.isfinite(got))  # rows >= length are NaN poisoned and never read

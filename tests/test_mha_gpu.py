@@ -223,6 +223,7 @@ def test_config1_gpt2_small_forward_fp32(capi, oracle):
     x = rng.standard_normal((B * T, 3 * E)).astype(np.float32)
     xt = torch.from_numpy(x).cuda()
     out, maxima, normalizers = capi.mha_forward(xt, T, H)
+    assert capi.last_path() == capi.PATH_MATRIX_F32   # not the any-shape kernel
     want, wm, wn = oracle.mha_fwd(x, T, H)
     assert_close(out.cpu().numpy(), want, FP32_REL, "config 1 out")
     assert_close((maxima + normalizers.log()).cpu().numpy(), wm + np.log(wn), 1e-4, "config 1 lse")
@@ -238,7 +239,9 @@ def test_config2_gpt2_small_forward_backward_bf16(capi, oracle):
     d_out = rng.standard_normal((B * T, E)).astype(np.float32)
     xt, gt = device_inputs(x, d_out, True)
     out, maxima, normalizers = capi.mha_forward(xt, T, H)
+    assert capi.last_path() == capi.PATH_FLASH
     d_qkv = capi.mha_backward(xt, out, gt, maxima, normalizers, T, H)
+    assert capi.last_path() == capi.PATH_FLASH
     D = E // H
     units = [(0, 0), (7, 5), (15, 11)]
     bits = to_bf16_bits(oracle, x)
@@ -258,6 +261,7 @@ def test_config2_gpt2_small_forward_backward_bf16(capi, oracle):
     with capi.force_generic():
         out2, m2, n2 = capi.mha_forward(xt, T, H)
         d2 = capi.mha_backward(xt, out2, gt, m2, n2, T, H)
+        assert capi.last_path() == capi.PATH_GENERIC
         torch.cuda.synchronize()
     assert_close_bf16(out.float().cpu().numpy(), out2.float().cpu().numpy(), "config 2 out vs fp32-arithmetic kernel")
     g1, g2 = d_qkv.cpu().numpy(), d2.cpu().numpy()
