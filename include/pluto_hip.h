@@ -429,14 +429,21 @@ int pluto_hip_gdn_step(void* stream, const pluto_hip_delta_params* p,
  * recurrent_states[s] ([batch, vh, kd, vd]); qkv [batch, channels], z and
  * output [batch, vh*vd], a and b [batch, vh]; the weights are shared.  Row s
  * of the result is bit for bit what pluto_hip_gdn_step gives for sequence s
- * alone. */
+ * alone.
+ *   io_dtype  PLUTO_HIP_F32 or PLUTO_HIP_BF16: the element type of qkv, z, a,
+ *             b and output.  With bf16 the step reads the layer's activations
+ *             and writes its result directly, which replaces the four ToFloat
+ *             launches and the ToBFloat16 launch of DeltaNetLayer::fwd_impl
+ *             (src/llm/layers/delta_net.cc:70-102) with nothing: the result is
+ *             bit for bit the FP32 step's output cast to bf16.  The states stay
+ *             FP32. */
 int pluto_hip_gdn_step_batch(void* stream, const pluto_hip_delta_params* p,
-                             int batch, float* conv_states,
-                             float* recurrent_states, const float* qkv,
-                             const float* z, const float* a, const float* b,
+                             int batch, int io_dtype, float* conv_states,
+                             float* recurrent_states, const void* qkv,
+                             const void* z, const void* a, const void* b,
                              const float* conv_weight, const float* a_log,
                              const float* dt_bias, const float* norm,
-                             float* output, void* workspace,
+                             void* output, void* workspace,
                              size_t workspace_bytes);
 
 /* FullyConnectedLayer, trainable path: the projections either side of the

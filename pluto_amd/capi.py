@@ -128,7 +128,7 @@ SIGNATURES = {
     "pluto_hip_gdn_step_workspace_bytes": (_SZ, [ctypes.POINTER(DeltaParams)]),
     "pluto_hip_gdn_step": (_I, [_VP, ctypes.POINTER(DeltaParams)] + [_VP] * 11 + [_VP, _SZ]),
     "pluto_hip_gdn_step_batch_workspace_bytes": (_SZ, [ctypes.POINTER(DeltaParams), _I]),
-    "pluto_hip_gdn_step_batch": (_I, [_VP, ctypes.POINTER(DeltaParams), _I] + [_VP] * 11 +
+    "pluto_hip_gdn_step_batch": (_I, [_VP, ctypes.POINTER(DeltaParams), _I, _I] + [_VP] * 11 +
                                  [_VP, _SZ]),
     "pluto_hip_dense_workspace_bytes": (_SZ, [_I, _I, _I, _I]),
     "pluto_hip_dense_forward": (_I, [_VP, _I, _VP, _VP, _VP, _I, _I, _I, _VP, _VP, _SZ]),
@@ -533,9 +533,10 @@ class DeltaNetStep:
                 ptr(qkv), ptr(z), ptr(a), ptr(b), ptr(conv_weight), ptr(a_log), ptr(dt_bias),
                 ptr(norm), ptr(out), ptr(self.workspace), self.workspace.numel()))
             return out
-        out = torch.empty((self.batch, width), device=qkv.device)
+        # activations and result are FP32 or bf16, all of one type
+        out = torch.empty((self.batch, width), device=qkv.device, dtype=qkv.dtype)
         check(lib().pluto_hip_gdn_step_batch(
-            stream or current_stream(), ctypes.byref(p), self.batch, ptr(self.conv),
+            stream or current_stream(), ctypes.byref(p), self.batch, dtype_code(qkv), ptr(self.conv),
             ptr(self.state), ptr(qkv), ptr(z), ptr(a), ptr(b), ptr(conv_weight), ptr(a_log),
             ptr(dt_bias), ptr(norm), ptr(out), ptr(self.workspace), self.workspace.numel()))
         return out

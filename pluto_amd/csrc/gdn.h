@@ -57,16 +57,17 @@ int launch_gdn_conv_sequence(hipStream_t stream, const void* input, int in_dtype
 // One token per sequence against that sequence's [channels, kernel] shift
 // register (input, output [batch, channels]; state [batch, channels, kernel]):
 // ConvolutionKernel, src/llm/layers/util/cached_attention_ops.cc:180-203.
-int launch_gdn_conv_step(hipStream_t stream, const float* input, const float* weight, int batch,
-                         int channels, int kernel, bool round, float* state, float* output);
+int launch_gdn_conv_step(hipStream_t stream, const void* input, int in_dtype, const float* weight,
+                         int batch, int channels, int kernel, bool round, float* state,
+                         float* output);
 // Gates, one token of the recurrence and the output norm/gate of `batch`
 // sequences in one launch, for key and value widths up to 128 (step_kernel).
 bool gdn_step_fused_supported(int key_dim, int value_dim);
-int launch_gdn_step_fused(hipStream_t stream, const float* convolved, const float* z,
-                          const float* a, const float* b, const float* a_log,
+int launch_gdn_step_fused(hipStream_t stream, const float* convolved, const void* z,
+                          const void* a, const void* b, int io_dtype, const float* a_log,
                           const float* dt_bias, const float* norm, int batch, int key_heads,
                           int value_heads, int key_dim, int value_dim, float epsilon, bool round,
-                          float* state, float* out);
+                          float* state, void* out);
 // g = -exp(A_log) softplus(a + dt_bias), beta = round(sigmoid(b)):
 // sequence_delta_net.cc:88-96.
 int launch_gdn_gates(hipStream_t stream, const void* a, const void* b, int in_dtype,

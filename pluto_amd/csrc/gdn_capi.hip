@@ -247,14 +247,15 @@ size_t pluto_hip_gdn_step_workspace_bytes(const pluto_hip_delta_params* p) {
 }
 
 int pluto_hip_gdn_step_batch(void* stream, const pluto_hip_delta_params* p, int batch,
-                             float* conv_states, float* recurrent_states, const float* qkv,
-                             const float* z, const float* a, const float* b,
+                             int io_dtype, float* conv_states, float* recurrent_states,
+                             const void* qkv, const void* z, const void* a, const void* b,
                              const float* conv_weight, const float* a_log, const float* dt_bias,
-                             const float* norm, float* output, void* workspace,
+                             const float* norm, void* output, void* workspace,
                              size_t workspace_bytes) {
   int status = validate_delta(p);
   if (status != 0) return status;
   if (batch <= 0) return PLUTO_HIP_EINVAL;
+  if (io_dtype != PLUTO_HIP_F32 && io_dtype != PLUTO_HIP_BF16) return PLUTO_HIP_EUNSUPPORTED;
   // cached_attention_ops.cc:405-408
   if (!conv_states || !recurrent_states || !qkv || !z || !a || !b || !conv_weight || !a_log ||
       !dt_bias || !norm || !output)
@@ -274,14 +275,13 @@ int pluto_hip_gdn_step_batch(void* stream, const pluto_hip_delta_params* p, int 
   float* beta = reinterpret_cast<float*>(scratch + offset);
   offset += align_up(n * vh * 4, 256);
   float* core = reinterpret_cast<float*>(scratch + offset);
-  status = launch_gdn_conv_step(s, qkv, conv_weight, batch, channels, p->conv_kernel_dim, round,
-                                conv_states, convolved);
+  status = launch_gdn_conv_step(s, qkv, io_dtype, conv_weight, batch, channels,
+                                p->conv_kernel_dim, round, conv_states, convolved);
   if (status != 0) return status;
   if (!force_generic() && gdn_step_fused_supported(kd, vd))
-    return launch_gdn_step_fused(s, convolved, z, a, b, a_log, dt_bias, norm, batch, kh, vh, kd, vd,
-                                 p->rms_norm_epsilon, round, recurrent_states, output);
-  status =
-      launch_gdn_gates(s, a, b, PLUTO_HIP_F32, a_log, dt_bias, batch, vh, round, log_decay, beta);
+    return launch_gdn_step_fused(s, convolved, z, a, b, io_dtype, a_log, dt_bias, norm, batch, kh,
+                                 vh, kd, vd, p->rms_norm_epsilon, round, recurrent_states, output);
+  status = launch_gdn_gates(s, a, b, io_dtype, a_log, dt_bias, batch, vh, round, log_decay, beta);
   if (status != 0) return status;
   GdnArgs g;
   g.q = reinterpret_cast<const uint16_t*>(convolved);
@@ -304,9 +304,9 @@ int pluto_hip_gdn_step_batch(void* stream, const pluto_hip_delta_params* p, int 
   g.q_scale = 1.0f / std::sqrt(static_cast<float>(kd));
   status = launch_gdn_recurrence(s, g, PLUTO_HIP_F32);
   if (status != 0) return status;
-  return launch_gdn_output(s, core, PLUTO_HIP_F32, z, PLUTO_HIP_F32, norm,
+  return launch_gdn_output(s, core, PLUTO_HIP_F32, z, io_dtype, norm,
                            static_cast<long long>(batch) * vh, vd, p->rms_norm_epsilon, round,
-                           output, PLUTO_HIP_F32);
+                           output, io_dtype);
 }
 
 int pluto_hip_gdn_step(void* stream, const pluto_hip_delta_params* p, float* conv_state,
@@ -314,7 +314,7 @@ int pluto_hip_gdn_step(void* stream, const pluto_hip_delta_params* p, float* con
                        const float* a, const float* b, const float* conv_weight,
                        const float* a_log, const float* dt_bias, const float* norm,
                        float* output, void* workspace, size_t workspace_bytes) {
-  return pluto_hip_gdn_step_batch(stream, p, 1, conv_state, recurrent_state, qkv, z, a, b,
+  return pluto_hip_gdn_step_batch(stream, p, 1, PLUTO_HIP_F32, conv_state, recurrent_state, qkv, z, a, b,
                                   conv_weight, a_log, dt_bias, norm, output, workspace,
                                   workspace_bytes);
 }

@@ -33,14 +33,13 @@ conv_sequence_kernel(const void* input, int in_dtype, const float* __restrict__ 
 }
 
 __global__ void __launch_bounds__(128)
-conv_step_kernel(const float* __restrict__ input, const float* __restrict__ weight,
+conv_step_kernel(const void* __restrict__ input, int in_dtype, const float* __restrict__ weight,
                  int channels, int kernel, bool round, float* __restrict__ state,
                  float* __restrict__ output) {
   const int c = blockIdx.x * 128 + threadIdx.x;
   if (c >= channels) return;
   // blockIdx.y: the sequence, each with its own shift registers and row
   const long long sequence = blockIdx.y;
-  input += sequence * channels;
   output += sequence * channels;
   float* taps = state + (sequence * channels + c) * kernel;
   const float* w = weight + static_cast<long long>(c) * kernel;
@@ -52,7 +51,7 @@ conv_step_kernel(const float* __restrict__ input, const float* __restrict__ weig
     sum += previous * w[tap];
     taps[tap] = previous;
   }
-  const float current = maybe_round(input[c], round);
+  const float current = maybe_round(load_element(input, sequence * channels + c, in_dtype), round);
   taps[kernel - 1] = current;
   sum = maybe_round(sum + current * w[kernel - 1], round);
   output[c] = maybe_round(sum / (1.0f + expf(-sum)), round);
@@ -114,19 +113,20 @@ output_kernel(const void* core, int core_dtype, const void* z, int z_dtype,
 // 64 half + 63 of its column.
 struct StepArgs {
   const float* convolved = nullptr;  // [batch, channels] q | k | v after conv + SiLU
-  const float* z = nullptr;          // [batch, vh * vd]
-  const float* a = nullptr;          // [batch, vh]
-  const float* b = nullptr;
+  const void* z = nullptr;           // [batch, vh * vd], fp32 or bf16 (template argument)
+  const void* a = nullptr;           // [batch, vh]
+  const void* b = nullptr;
   const float* a_log = nullptr;
   const float* dt_bias = nullptr;
   const float* norm = nullptr;
   float* state = nullptr;            // [batch, vh, kd, vd]
-  float* out = nullptr;              // [batch, vh * vd]
+  void* out = nullptr;               // [batch, vh * vd], same type as z
   int kh = 0, vh = 0, kd = 0, vd = 0;
   float epsilon = 1e-6f;
   bool round = true;
 };
 
+template <int IO>
 __global__ void __launch_bounds__(256)
 step_kernel(StepArgs a) {
   __shared__ float ks[128], qs[128];
@@ -156,14 +156,15 @@ step_kernel(StepArgs a) {
     qs[tid] = tid < kd ? qv : 0.0f;
   }
   const float value = token[2 * a.kh * kd + head * vd + column_read];
-  const float gate = a.z[(static_cast<size_t>(seq) * a.vh + head) * vd + column_read];
+  const float gate =
+      load_element(a.z, (static_cast<long long>(seq) * a.vh + head) * vd + column_read, IO);
   const float weight = a.norm[column_read];
   const size_t scalar = static_cast<size_t>(seq) * a.vh + head;
-  const float alpha = a.a[scalar] + a.dt_bias[head];
+  const float alpha = load_element(a.a, scalar, IO) + a.dt_bias[head];
   // stable softplus: no overflow for strongly positive time steps
   const float softplus = fmaxf(alpha, 0.0f) + log1pf(expf(-fabsf(alpha)));
   const float decay = __expf(-expf(a.a_log[head]) * softplus);
-  const float beta = maybe_round(1.0f / (1.0f + expf(-a.b[scalar])), a.round);
+  const float beta = maybe_round(1.0f / (1.0f + expf(-load_element(a.b, scalar, IO))), a.round);
   __syncthreads();
   // 1e-6 inside the root: cached_attention_ops.cc:224-228
   float kk = 1e-6f, qq = 1e-6f;
@@ -207,7 +208,10 @@ step_kernel(StepArgs a) {
   const float normalized = maybe_round(core * inverse, a.round);
   const float affine = maybe_round(normalized * weight, a.round);
   const float result = affine * (gate / (1.0f + expf(-gate)));
-  a.out[(static_cast<size_t>(seq) * a.vh + head) * vd + column] = maybe_round(result, a.round);
+  // a bf16 result is rounded once, by the store: the FP32 step followed by the
+  // layer's cast (delta_net.cc:97-101) gives the same bits with or without the flag
+  store_element(a.out, (static_cast<long long>(seq) * a.vh + head) * vd + column, IO,
+                IO == PLUTO_HIP_BF16 ? result : maybe_round(result, a.round));
 }
 
 }  // namespace
@@ -216,11 +220,11 @@ bool gdn_step_fused_supported(int key_dim, int value_dim) {
   return key_dim <= 128 && value_dim <= 128;
 }
 
-int launch_gdn_step_fused(hipStream_t stream, const float* convolved, const float* z,
-                          const float* a, const float* b, const float* a_log,
+int launch_gdn_step_fused(hipStream_t stream, const float* convolved, const void* z,
+                          const void* a, const void* b, int io_dtype, const float* a_log,
                           const float* dt_bias, const float* norm, int batch, int key_heads,
                           int value_heads, int key_dim, int value_dim, float epsilon, bool round,
-                          float* state, float* out) {
+                          float* state, void* out) {
   StepArgs s;
   s.convolved = convolved;
   s.z = z;
@@ -237,7 +241,10 @@ int launch_gdn_step_fused(hipStream_t stream, const float* convolved, const floa
   s.vd = value_dim;
   s.epsilon = epsilon;
   s.round = round;
-  step_kernel<<<batch * value_heads, 256, 0, stream>>>(s);
+  if (io_dtype == PLUTO_HIP_BF16)
+    step_kernel<PLUTO_HIP_BF16><<<batch * value_heads, 256, 0, stream>>>(s);
+  else
+    step_kernel<PLUTO_HIP_F32><<<batch * value_heads, 256, 0, stream>>>(s);
   return launch_status();
 }
 
@@ -250,10 +257,11 @@ int launch_gdn_conv_sequence(hipStream_t stream, const void* input, int in_dtype
   return launch_status();
 }
 
-int launch_gdn_conv_step(hipStream_t stream, const float* input, const float* weight, int batch,
-                         int channels, int kernel, bool round, float* state, float* output) {
+int launch_gdn_conv_step(hipStream_t stream, const void* input, int in_dtype, const float* weight,
+                         int batch, int channels, int kernel, bool round, float* state,
+                         float* output) {
   conv_step_kernel<<<dim3((channels + 127) / 128, batch), 128, 0, stream>>>(
-      input, weight, channels, kernel, round, state, output);
+      input, in_dtype, weight, channels, kernel, round, state, output);
   return launch_status();
 }
 

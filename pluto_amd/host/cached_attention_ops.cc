@@ -147,11 +147,23 @@ StatusOr<std::unique_ptr<DeltaNetState>> DeltaNetState::Create(hip::Executor& ex
 Status DeltaNetState::Step(const float* qkv, const float* z, const float* a, const float* b,
                            const float* conv_weight, const float* a_log, const float* dt_bias,
                            const float* norm_weight, float* output) {
+  return StepAs(PLUTO_HIP_F32, qkv, z, a, b, conv_weight, a_log, dt_bias, norm_weight, output);
+}
+
+Status DeltaNetState::StepBFloat16(const void* qkv, const void* z, const void* a, const void* b,
+                                   const float* conv_weight, const float* a_log,
+                                   const float* dt_bias, const float* norm_weight, void* output) {
+  return StepAs(PLUTO_HIP_BF16, qkv, z, a, b, conv_weight, a_log, dt_bias, norm_weight, output);
+}
+
+Status DeltaNetState::StepAs(int io_dtype, const void* qkv, const void* z, const void* a,
+                             const void* b, const float* conv_weight, const float* a_log,
+                             const float* dt_bias, const float* norm_weight, void* output) {
   if (!qkv || !z || !a || !b || !conv_weight || !a_log || !dt_bias || !norm_weight || !output)
     return InvalidArgumentError("DeltaNet requires non-null device pointers");
   const pluto_hip_delta_params abi = ToAbi(parameters_);
   return hip::HipStatus(
-      pluto_hip_gdn_step_batch(executor_.stream(), &abi, batch_,
+      pluto_hip_gdn_step_batch(executor_.stream(), &abi, batch_, io_dtype,
                                static_cast<float*>(convolution_state_.data()),
                                static_cast<float*>(recurrent_state_.data()), qkv, z, a, b,
                                conv_weight, a_log, dt_bias, norm_weight, output, workspace_.data(),

@@ -88,6 +88,12 @@ class DeltaNetState final {
   Status Step(const float* qkv, const float* z, const float* a, const float* b,
               const float* conv_weight, const float* a_log, const float* dt_bias,
               const float* norm_weight, float* output);
+  // The same step on bf16 activations (qkv, z, a, b and output hold bf16
+  // elements; weights and both states stay FP32): what DeltaNetLayer feeds it,
+  // without the casts either side.  Output = the FP32 step's, rounded to bf16.
+  Status StepBFloat16(const void* qkv, const void* z, const void* a, const void* b,
+                      const float* conv_weight, const float* a_log, const float* dt_bias,
+                      const float* norm_weight, void* output);
   Status Reset();
 
  private:
@@ -96,6 +102,9 @@ class DeltaNetState final {
       : executor_(executor), parameters_(parameters), batch_(batch),
         convolution_state_(std::move(convolution_state)),
         recurrent_state_(std::move(recurrent_state)), workspace_(std::move(workspace)) {}
+  Status StepAs(int io_dtype, const void* qkv, const void* z, const void* a, const void* b,
+                const float* conv_weight, const float* a_log, const float* dt_bias,
+                const float* norm_weight, void* output);
   hip::Executor& executor_;
   DeltaNetParameters parameters_;
   int batch_;

@@ -277,10 +277,39 @@ def test_batched_step_rejects_bad_arguments(capi):
     x = torch.zeros(4096, device="cuda")
     px = capi.ptr(x)
     args = [px] * 11
-    assert lib.pluto_hip_gdn_step_batch(capi.current_stream(), ctypes.byref(p), 0, *args, px, size) != 0
-    assert lib.pluto_hip_gdn_step_batch(capi.current_stream(), ctypes.byref(p), 3, *args, px, 16) != 0
-    assert lib.pluto_hip_gdn_step_batch(capi.current_stream(), ctypes.byref(p), 3, None, *args[1:], px,
+    stream, f32 = capi.current_stream(), capi.F32
+    assert lib.pluto_hip_gdn_step_batch(stream, ctypes.byref(p), 0, f32, *args, px, size) != 0
+    assert lib.pluto_hip_gdn_step_batch(stream, ctypes.byref(p), 3, f32, *args, px, 16) != 0
+    assert lib.pluto_hip_gdn_step_batch(stream, ctypes.byref(p), 3, f32, None, *args[1:], px,
                                         size) != 0
+    assert lib.pluto_hip_gdn_step_batch(stream, ctypes.byref(p), 3, 77, *args, px, size) != 0
+
+
+@pytest.mark.parametrize("round_flag", [False, True])
+@pytest.mark.parametrize("dim", [5, 128])
+def test_bf16_step_is_the_fp32_step_between_casts(capi, dim, round_flag):
+    """io_dtype = bf16: what DeltaNetLayer::fwd_impl (delta_net.cc:70-102) computes
+    with four ToFloat launches before the FP32 step and one ToBFloat16 after it,
+    bit for bit, over several tokens (both states carry over) and five sequences."""
+    kh, vh, kd, vd = 2, 6, dim, (7 if dim == 5 else 128)
+    batch, steps = 5, 4
+    p = capi.delta_params(kh, vh, kd, vd, round_to_bfloat16=round_flag)
+    channels = 2 * kh * kd + vh * vd
+    w, a_log, dt, norm = layer_weights(kh, vh, kd, vd, 4)
+    dw, dal, ddt, dn = dev(w), dev(a_log), dev(dt), dev(norm)
+    direct = capi.DeltaNetStep(p, batch=batch)
+    through_casts = capi.DeltaNetStep(p, batch=batch)
+    rng = np.random.default_rng(10 * dim + round_flag)
+    bf = torch.bfloat16
+    for step in range(steps):
+        qkv, z, a, b = (dev(rng.standard_normal((batch, n)).astype(np.float32)).to(bf)
+                        for n in (channels, vh * vd, vh, vh))
+        got = direct.step(qkv, z, a, b, dw, dal, ddt, dn)
+        assert got.dtype == bf
+        want = through_casts.step(qkv.float(), z.float(), a.float(), b.float(), dw, dal, ddt, dn)
+        assert torch.equal(got, want.to(bf)), step
+    assert torch.equal(direct.state, through_casts.state)
+    assert torch.equal(direct.conv, through_casts.conv)
 
 
 @pytest.mark.parametrize("kh,vh,kd,vd,T,round_flag", [(2, 6, 5, 7, 9, False), (2, 6, 5, 7, 9, True),

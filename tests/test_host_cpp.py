@@ -38,7 +38,7 @@ def test_every_reference_class_has_cases(runner):
     suites = {name.split(".")[0] for name in listed}
     assert {"AttentionLayerTest", "AttentionOpsTest", "QwenAttentionTest", "SequenceDeltaNetTest",
             "KeyValueCacheTest", "BufferTest", "ExecutorTest", "PageLockedHostArrayTest",
-            "ActivationTypeCpu", "StatusCpu"} <= suites
+            "ActivationTypeCpu", "StatusCpu", "LayerHooksTest", "DeltaNetLayerTest"} <= suites
 
 
 @pytest.mark.gpu
