@@ -42,8 +42,8 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E (published)
 # kept as profiles/*_hbm_traffic.md.  None = not measured.
 MEASURED_TRAFFIC_BYTES = {
     ("mha_train_bf16", "flash_forward_kernel<64>"): 126.4e6,
-    ("gqa_prefill", "flash_forward_kernel<128>"): 347.7e6 + 50.3e6,
-    ("gqa_decode", "decode_split_kernel<128,6>"): 1028.3e6 + 12.6e6,
+    ("gqa_prefill", "flash_forward_kernel<128>"): 169.6e6 + 50.7e6,
+    ("gqa_decode", "decode_fused_kernel<128,6>"): 1044.3e6 + 13.0e6,
     ("gdn_scan", "gdn_chunk_prepare + gdn_chunk_scan"): 2105.3e6,
 }
 
@@ -51,7 +51,8 @@ NAMES = ["mha_train_bf16", "mha_fwd_fp32", "gqa_prefill", "gqa_decode", "gdn_sca
 # "copy" is a plain device copy of known size: the calibration case for the
 # FETCH_SIZE / WRITE_SIZE counters that `roofline.traffic` is derived from.
 # "gqa_prefill_bwd" and "gdn_layer_bwd" time the two sequence backward passes.
-EXTRA = ["copy", "gqa_prefill_bwd", "gdn_layer_bwd", "gdn_decode", "dense_qkv", "dense_imported"]
+EXTRA = ["copy", "gqa_prefill_bwd", "gdn_layer_bwd", "gdn_decode", "dense_qkv", "dense_imported",
+         "decode_block"]
 
 
 def parse_args():
@@ -275,8 +276,8 @@ def gqa_decode(torch, capi):
 
     work = 2.0 * kh * d * 2 * float(lengths.sum())   # K and V bytes of the valid prefix
     return dict(step=step,
-                kernels=[("decode_split_kernel<128,6>", step, capi.MAIN_KERNEL, work),
-                         ("prepare + combine", step, capi.AUXILIARY_KERNELS, None)],
+                kernels=[("decode_fused_kernel<128,6>", step, capi.MAIN_KERNEL, work),
+                         ("counter clear", step, capi.AUXILIARY_KERNELS, None)],
                 work=work,
                 metric="gqa_decode_hbm_gbs", unit="GB/s", dtype="bf16", bound="hbm",
                 peak=PEAK_HBM_GBS,
@@ -324,15 +325,16 @@ def gdn_decode(torch, capi):
     """One token of the gated delta-net layer for 32 sequences with their own
     states (the delta-net half of a batched decoder step): a row after the
     headline ones, not part of --workload all."""
-    batch, H, dk, dv, K = 32, 16, 128, 128, 4
-    p = capi.delta_params(H, H, dk, dv, K)
-    channels = 2 * H * dk + H * dv
+    batch, kh, H, dk, dv, K = 32, 16, 48, 128, 128, 4   # the model's 16 key / 48 value heads
+    p = capi.delta_params(kh, H, dk, dv, K)
+    channels = 2 * kh * dk + H * dv
     gen = torch.Generator(device="cuda").manual_seed(5)
+    bf = torch.bfloat16
     states = capi.DeltaNetStep(p, batch=batch)
-    qkv = torch.randn((batch, channels), generator=gen, device="cuda")
-    z = torch.randn((batch, H * dv), generator=gen, device="cuda")
-    a = torch.randn((batch, H), generator=gen, device="cuda")
-    b = torch.randn((batch, H), generator=gen, device="cuda")
+    qkv = torch.randn((batch, channels), generator=gen, device="cuda").to(bf)
+    z = torch.randn((batch, H * dv), generator=gen, device="cuda").to(bf)
+    a = torch.randn((batch, H), generator=gen, device="cuda").to(bf)
+    b = torch.randn((batch, H), generator=gen, device="cuda").to(bf)
     conv = 0.5 * torch.randn((channels, K), generator=gen, device="cuda")
     a_log = torch.zeros(H, device="cuda")
     dt_bias = torch.zeros(H, device="cuda")
@@ -346,8 +348,138 @@ def gdn_decode(torch, capi):
     return dict(step=step, kernels=[("whole call", step, None, work)], work=work,
                 metric="gdn_decode_step_hbm_gbs", unit="GB/s", dtype="f32", bound="hbm",
                 peak=PEAK_HBM_GBS,
-                config={"workload": "gated_delta_net_decode_step", "batch": batch, "heads": H,
-                        "d_k": dk, "d_v": dv, "conv_kernel": K, "state": "fp32, one per sequence"},
+                config={"workload": "gated_delta_net_decode_step", "batch": batch, "key_heads": kh,
+                        "value_heads": H, "d_k": dk, "d_v": dv, "conv_kernel": K,
+                        "activations": "bf16", "state": "fp32, one per sequence"},
+                cpu=None)
+
+
+def decode_block(torch, capi):
+    """The attention branches of one decoder step for 32 sequences at the model's
+    shape (CreateAttentionBranch, qwen/model.cc:174-274, lifted from batch one):
+    a full-attention branch (FP8 q|gate, k, v projections from the 5120-wide
+    residual stream, cached attention with 24 / 4 heads of 256 over contexts of
+    1024..32768 tokens, FP8 output projection) and a delta-net branch (FP8
+    q|k|v, z, a, b projections, the gated delta step with 16 / 48 heads of
+    128 x 128, FP8 output projection).  Bytes: every weight, every valid K/V row
+    and every state once.  A row after the headline ones, not part of
+    --workload all."""
+    import numpy as np
+    batch, width = 32, 5120
+    qh, kvh, d, capacity = 24, 4, 256, 32768
+    kh, vh, dk, dv, taps = 16, 48, 128, 128, 4
+    bf = torch.bfloat16
+    gen = torch.Generator(device="cuda").manual_seed(9)
+
+    def matrix(n_in, n_out):
+        w = torch.randint(0, 0x7e, (n_out, n_in), generator=gen, device="cuda", dtype=torch.uint8)
+        w |= torch.randint(0, 2, (n_out, n_in), generator=gen, device="cuda", dtype=torch.uint8) << 7
+        sc = (0.5 + torch.rand(((n_out + 127) // 128, (n_in + 127) // 128), generator=gen,
+                               device="cuda")) * (0.004 / math.sqrt(n_in / 5120))
+        size = lib_bytes(tokens=batch, input_dim=n_in)
+        return dict(w=w, s=sc, ws=torch.empty(size, dtype=torch.uint8, device="cuda"),
+                    bytes=float(w.numel() + sc.numel() * 4))
+
+    def lib_bytes(tokens, input_dim):
+        return max(capi.lib().pluto_hip_dense_imported_batch_workspace_bytes(tokens, input_dim), 1)
+
+    def project(m, x, out):
+        capi.dense_imported_forward_batch(capi.MATRIX_FP8_E4M3, m["w"], m["s"], x, m["ws"], out)
+
+    hidden = torch.randn((batch, width), generator=gen, device="cuda").to(bf)
+    # full attention
+    q, kv = qh * d, kvh * d
+    wq, wk, wv, wo = matrix(width, 2 * q), matrix(width, kv), matrix(width, kv), matrix(q, width)
+    p = capi.attention_params(qh, kvh, d, 64, capacity=capacity)
+    rng = np.random.default_rng(3)
+    lengths = (1024 + np.floor(rng.random(batch) * 31745)).astype(int)
+    caches = []
+    for L in lengths:
+        c = capi.KvCache(capacity, kvh, d)
+        c.keys[:, :L] = torch.randn((kvh, L, d), generator=gen, device="cuda").to(bf)
+        c.values[:, :L] = torch.randn((kvh, L, d), generator=gen, device="cuda").to(bf)
+        caches.append(c)
+    positions = [int(L - 1) for L in lengths]
+    qn = torch.from_numpy(values(np, d, 0.2, 0.3)).cuda()
+    kn = torch.from_numpy(values(np, d, 0.8, 0.4)).cuda()
+    q_gate = torch.empty((batch, qh, 2, d), dtype=bf, device="cuda")
+    k_new = torch.empty((batch, kvh, d), dtype=bf, device="cuda")
+    v_new = torch.empty((batch, kvh, d), dtype=bf, device="cuda")
+    attended = torch.empty((batch, qh, d), dtype=bf, device="cuda")
+    attention_out = torch.empty((batch, width), dtype=bf, device="cuda")
+    decode_ws = capi.gqa_decode_workspace(p, positions, 0)
+
+    def attention_in():
+        project(wq, hidden, q_gate.view(batch, -1))
+        project(wk, hidden, k_new.view(batch, -1))
+        project(wv, hidden, v_new.view(batch, -1))
+
+    def attention_core():
+        capi.gqa_decode(p, q_gate, k_new, v_new, qn, kn, caches, positions=positions,
+                        workspace=decode_ws, out=attended, advance=False)
+
+    def attention_project():
+        project(wo, attended.view(batch, -1), attention_out)
+
+    # delta-net
+    keys, vals = kh * dk, vh * dv
+    channels = 2 * keys + vals
+    wqkv, wz, wa, wb, wout = (matrix(width, channels), matrix(width, vals), matrix(width, vh),
+                              matrix(width, vh), matrix(vals, width))
+    dp = capi.delta_params(kh, vh, dk, dv, taps)
+    states = capi.DeltaNetStep(dp, batch=batch)
+    conv = 0.5 * torch.randn((channels, taps), generator=gen, device="cuda")
+    a_log, dt_bias, norm = (torch.zeros(vh, device="cuda"), torch.zeros(vh, device="cuda"),
+                            torch.ones(dv, device="cuda"))
+    qkv = torch.empty((batch, channels), dtype=bf, device="cuda")
+    z = torch.empty((batch, vals), dtype=bf, device="cuda")
+    a = torch.empty((batch, vh), dtype=bf, device="cuda")
+    b = torch.empty((batch, vh), dtype=bf, device="cuda")
+    delta_out = torch.empty((batch, width), dtype=bf, device="cuda")
+    mixed = [None]
+
+    def delta_in():
+        project(wqkv, hidden, qkv)
+        project(wz, hidden, z)
+        project(wa, hidden, a)
+        project(wb, hidden, b)
+
+    def delta_core():
+        mixed[0] = states.step(qkv, z, a, b, conv, a_log, dt_bias, norm)
+
+    def delta_project():
+        project(wout, mixed[0], delta_out)
+
+    def step():
+        attention_in()
+        attention_core()
+        attention_project()
+        delta_in()
+        delta_core()
+        delta_project()
+
+    kv_bytes = 2.0 * kvh * d * 2 * float(lengths.sum())
+    state_bytes = 2.0 * batch * (vh * dk * dv + channels * taps) * 4
+    in_a = wq["bytes"] + wk["bytes"] + wv["bytes"]
+    in_d = wqkv["bytes"] + wz["bytes"] + wa["bytes"] + wb["bytes"]
+    work = kv_bytes + state_bytes + in_a + in_d + wo["bytes"] + wout["bytes"]
+    return dict(step=step,
+                kernels=[("attention: q|gate, k, v projections", attention_in, None, in_a),
+                         ("attention: cached step (decode_fused_kernel<256,6>)", attention_core,
+                          None, kv_bytes),
+                         ("attention: output projection", attention_project, None, wo["bytes"]),
+                         ("delta-net: q|k|v, z, a, b projections", delta_in, None, in_d),
+                         ("delta-net: gated delta step", delta_core, None, state_bytes),
+                         ("delta-net: output projection", delta_project, None, wout["bytes"])],
+                work=work, metric="decoder_attention_branches_hbm_gbs", unit="GB/s", dtype="bf16",
+                bound="hbm", peak=PEAK_HBM_GBS,
+                config={"workload": "qwen_decoder_step_attention_branches", "batch": batch,
+                        "model_width": width, "projections": "fp8_e4m3, 128x128 fp32 block scales",
+                        "full_attention": {"query_heads": qh, "kv_heads": kvh, "head_dim": d,
+                                           "rotary_dim": 64, "sum_context": int(lengths.sum()),
+                                           "kv_cache": "bf16 head-major"},
+                        "delta_net": {"key_heads": kh, "value_heads": vh, "d_k": dk, "d_v": dv,
+                                      "conv_kernel": taps, "state": "fp32, one per sequence"}},
                 cpu=None)
 
 
@@ -428,7 +560,7 @@ def copy(torch, capi):
                         "bytes_written": n * 4}, cpu=None)
 
 
-WORKLOADS = {"copy": copy, "gdn_decode": gdn_decode, "dense_qkv": dense_qkv, "dense_imported": dense_imported, "mha_train_bf16": mha_train_bf16, "mha_fwd_fp32": mha_fwd_fp32,
+WORKLOADS = {"copy": copy, "gdn_decode": gdn_decode, "decode_block": decode_block, "dense_qkv": dense_qkv, "dense_imported": dense_imported, "mha_train_bf16": mha_train_bf16, "mha_fwd_fp32": mha_fwd_fp32,
              "gqa_prefill": gqa_prefill, "gqa_prefill_bwd": gqa_prefill_bwd, "gdn_layer_bwd": gdn_layer_bwd,
              "gqa_decode": gqa_decode,
              "gdn_scan": gdn_scan}

@@ -82,10 +82,11 @@ Status CachedAttentionStep(hip::Executor& executor, const FullAttentionParameter
   return cache.Advance();
 }
 
-Status CachedAttentionStepBatch(hip::Executor& executor, const FullAttentionParameters& p,
-                                Span<KeyValueCache* const> caches, const float* q_gate,
-                                const float* k, const float* v, const float* q_norm,
-                                const float* k_norm, float* output) {
+namespace {
+
+Status StepBatchAs(int io_dtype, hip::Executor& executor, const FullAttentionParameters& p,
+                   Span<KeyValueCache* const> caches, const void* q_gate, const void* k,
+                   const void* v, const float* q_norm, const float* k_norm, void* output) {
   if (caches.empty()) return InvalidArgumentError("attention batch must not be empty");
   if (!q_gate || !k || !v || !q_norm || !k_norm || !output)
     return InvalidArgumentError("attention requires non-null device pointers");
@@ -108,12 +109,28 @@ Status CachedAttentionStepBatch(hip::Executor& executor, const FullAttentionPara
       pluto_hip_gqa_decode_workspace_bytes(&abi, batch, positions.data(), 0);
   ASSIGN_OR_RETURN(auto workspace, hip::Buffer::Allocate(executor, workspace_bytes));
   RETURN_IF_ERROR(hip::HipStatus(
-      pluto_hip_gqa_decode(executor.stream(), &abi, batch, PLUTO_HIP_F32, q_gate, k, v, q_norm,
+      pluto_hip_gqa_decode(executor.stream(), &abi, batch, io_dtype, q_gate, k, v, q_norm,
                            k_norm, positions.data(), views.data(), output, nullptr, 0,
                            workspace.data(), workspace_bytes),
       "Qwen full attention"));
   for (KeyValueCache* cache : caches) RETURN_IF_ERROR(cache->Advance());
   return OkStatus();
+}
+
+}  // namespace
+
+Status CachedAttentionStepBatch(hip::Executor& executor, const FullAttentionParameters& p,
+                                Span<KeyValueCache* const> caches, const float* q_gate,
+                                const float* k, const float* v, const float* q_norm,
+                                const float* k_norm, float* output) {
+  return StepBatchAs(PLUTO_HIP_F32, executor, p, caches, q_gate, k, v, q_norm, k_norm, output);
+}
+
+Status CachedAttentionStepBatchBFloat16(hip::Executor& executor, const FullAttentionParameters& p,
+                                        Span<KeyValueCache* const> caches, const void* q_gate,
+                                        const void* k, const void* v, const float* q_norm,
+                                        const float* k_norm, void* output) {
+  return StepBatchAs(PLUTO_HIP_BF16, executor, p, caches, q_gate, k, v, q_norm, k_norm, output);
 }
 
 // src/llm/layers/util/cached_attention_ops.cc:369-399

@@ -54,6 +54,15 @@ Status CachedAttentionStepBatch(hip::Executor& executor,
                                 Span<KeyValueCache* const> caches, const float* q_gate,
                                 const float* k, const float* v, const float* q_norm,
                                 const float* k_norm, float* output);
+// The batched step on bf16 activations: q_gate, k, v and output hold bf16
+// elements, as the projections either side of the attention produce and take
+// them (what QwenAttentionLayer::CachedForward does for one sequence without
+// its casts).  The norm weights stay FP32.
+Status CachedAttentionStepBatchBFloat16(hip::Executor& executor,
+                                        const FullAttentionParameters& parameters,
+                                        Span<KeyValueCache* const> caches, const void* q_gate,
+                                        const void* k, const void* v, const float* q_norm,
+                                        const float* k_norm, void* output);
 
 struct DeltaNetParameters {
   int key_heads = 16;

@@ -65,6 +65,9 @@ class FullyConnectedLayer final : public Layer {
 
   int input_dim() const { return input_dim_; }
   int output_dim() const { return output_dim_; }
+  // Engaged for an imported matrix; weights() then holds the matrix and, for
+  // FP8, its block scales.
+  std::optional<MatrixStorage> imported_storage() const { return imported_storage_; }
 
  private:
   FullyConnectedLayer(hip::Executor& executor, int input_dim, int output_dim, DataType data_type,

@@ -12,9 +12,9 @@ QwenAttentionLayer::QwenAttentionLayer(hip::Executor& executor, FullAttentionPar
                                        std::shared_ptr<BlockParameter> q_norm,
                                        std::shared_ptr<BlockParameter> k_norm,
                                        int sequence_length, KeyValueCache* cache)
-    : executor_(executor), parameters_(p), q_norm_(std::move(q_norm)), k_norm_(std::move(k_norm)),
-      sequence_length_(sequence_length), weights_{q_norm_->value(), k_norm_->value()},
-      cache_(cache) {
+    : executor_(executor), parameters_(p), sequence_length_(sequence_length), cache_(cache),
+      q_norm_(std::move(q_norm)), k_norm_(std::move(k_norm)),
+      weights_{q_norm_->value(), k_norm_->value()} {
   const int64_t batch = ActivationType::kBatchDimension;
   input_types_ = {
       {DataType::BF16, {batch, sequence_length, 2LL * p.query_heads * p.head_dim}},

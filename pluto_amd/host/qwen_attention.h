@@ -1,21 +1,28 @@
-// Batch-one Qwen grouped-query attention: per-head Q/K RMSNorm, partial RoPE,
-// causal attention and sigmoid output gating -- QwenAttentionLayer of
-// src/llm/layers/qwen_attention.h:11-101 on MI355X.  Inputs are physical BF16
-// [T, query_heads, 2, head_dim] query/gate and [T, KV_heads, head_dim] K/V;
-// the output is BF16 [T, query_heads, head_dim].
+// QwenAttentionLayer, the class of src/llm/layers/qwen_attention.h:11-101 for
+// MI355X: grouped-query attention of one sequence with an RMS norm on every
+// query and key head, rotary embedding on the leading rotary_dim channels, a
+// causal softmax and a sigmoid gate on the output.
 //
-// A null cache selects stateless whole-sequence attention ("prefill"): one
-// prepare launch and one flash-attention launch over a private K/V scratch, for
-// any sequence length up to kMaximumSequenceLength (the reference stops at 128
-// because it materialises the quadratic probability tensor; here that tensor is
-// only produced when an attention_probabilities_hook asks for it).  Backward
-// through the sequence path is not part of this library and reports
-// Unimplemented.
+//   inputs   bf16 query|gate [T, query_heads, 2, head_dim], bf16 keys and bf16
+//            values [T, kv_heads, head_dim]
+//   output   bf16 [T, query_heads, head_dim]
 //
-// A nonnull cache selects single-token decoding and rejects backward.  The
-// cache is borrowed, must outlive the layer and must not be shared between
-// layers; its position advances even though fwd is const.  Reset it before a
-// new sequence or after any failed forward (including hooks).
+// Which of two modes a layer runs in is fixed at Create by the cache pointer
+// and by nothing else:
+//   no cache   the whole sequence at once, nothing persistent read or written.
+//              One prepare launch and one flash-attention launch over scratch
+//              keys/values, for up to kMaximumSequenceLength tokens (the
+//              reference stops at 128, where its [heads, T, T] probability
+//              tensor is still small; here that tensor exists only while an
+//              attention_probabilities_hook wants it).  bwd returns the
+//              gradients of all three inputs and adds the norm gradients of
+//              trainable norms.
+//   a cache    one token per fwd, appended to the borrowed KeyValueCache, whose
+//              position moves although fwd is const.  The cache must outlive
+//              the layer, belongs to this layer alone, and must be Reset before
+//              another sequence and after any fwd that failed (a failing hook
+//              counts).  bwd is rejected.
+// Calls on one layer must not overlap; the Executor outlives the layer.
 #pragma once
 
 #include <memory>
@@ -31,17 +38,16 @@ using FullAttentionParameters = cached_attention_ops::FullAttentionParameters;
 
 class QwenAttentionLayer final : public Layer {
  public:
-  // Bounds converted projection scratch for cached, single-token inference.
-  static constexpr int kMaximumDimension = 1048576;
-  static constexpr int kMaximumSequenceLength = 65535;
+  static constexpr int kMaximumDimension = 1048576;     // widest token row accepted
+  static constexpr int kMaximumSequenceLength = 65535;  // no-cache mode
 
-  // Shares resident FP32 norm parameters.  The cache pointer alone selects the
-  // execution mode; cached attention requires sequence_length == 1.
+  // Norm weights shared with their owner (an optimizer may train them); with a
+  // cache, sequence_length has to be 1.
   static StatusOr<std::unique_ptr<QwenAttentionLayer>> Create(
       hip::Executor& executor, FullAttentionParameters parameters,
       std::shared_ptr<BlockParameter> q_norm, std::shared_ptr<BlockParameter> k_norm,
       int sequence_length, KeyValueCache* cache = nullptr);
-  // Imports frozen FP32 norm buffers.
+  // Norm weights given as plain FP32 buffers: frozen, no gradient storage.
   static StatusOr<std::unique_ptr<QwenAttentionLayer>> Create(
       hip::Executor& executor, FullAttentionParameters parameters, Buffer q_norm, Buffer k_norm,
       int sequence_length, KeyValueCache* cache = nullptr);
@@ -61,26 +67,24 @@ class QwenAttentionLayer final : public Layer {
                                LayerHooks* hooks) const override;
   StatusOr<BufferVec> bwd_impl(hip::Executor& executor, Span<const Buffer> gradients,
                                BackwardState state, LayerHooks* hooks) override;
-  // Appends one token to the borrowed cache and optionally reports its
-  // [1, query_heads, 1, prefix_length] attention probabilities.
+  // the two modes of fwd_impl; CachedForward hands an installed probability
+  // hook one row per query head, [1, query_heads, 1, tokens so far]
   StatusOr<FwdResult> CachedForward(hip::Executor& executor, Span<const Buffer> inputs,
                                     LayerHooks* hooks) const;
-  // Whole causal sequence, without reading or updating any persistent cache.
   StatusOr<FwdResult> SequenceForward(hip::Executor& executor, Span<const Buffer> inputs,
                                       LayerHooks* hooks) const;
-
-  // Returns FP32 Q/gate, K and V gradients; accumulates norm gradients only
-  // into parameters that are active.
+  // FP32 gradients of query|gate, keys and values; a norm's gradient is added
+  // to its BlockParameter only while that parameter is being trained
   StatusOr<BufferVec> SequenceBackward(hip::Executor& executor, Span<const Buffer> gradients,
                                        BackwardState state);
 
+  std::vector<ActivationType> input_types_, output_types_;
   hip::Executor& executor_;
   FullAttentionParameters parameters_;
-  std::shared_ptr<BlockParameter> q_norm_, k_norm_;
   int sequence_length_;
-  Buffer weights_[2];     // Resident FP32 query/key norm values, in that order.
-  KeyValueCache* cache_;  // Nonowning; null means stateless sequence attention.
-  std::vector<ActivationType> input_types_, output_types_;
+  KeyValueCache* cache_;  // borrowed; null = whole-sequence mode
+  std::shared_ptr<BlockParameter> q_norm_, k_norm_;
+  Buffer weights_[2];  // the two norms' FP32 values, query norm first
 };
 
 }  // namespace pluto::llm

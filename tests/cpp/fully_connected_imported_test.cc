@@ -12,24 +12,9 @@ using testing::NewExecutor;
 using testing::Read;
 using testing::Upload;
 
-// Uploads raw elements of type T.
-template <class T>
-StatusOr<Buffer> UploadRaw(hip::Executor& executor, const std::vector<T>& values) {
-  ASSIGN_OR_RETURN(auto host, hip::PageLockedHostArray<T>::Allocate(executor, values.size()));
-  for (size_t i = 0; i < values.size(); ++i) host[i] = values[i];
-  ASSIGN_OR_RETURN(auto device, Buffer::Allocate(executor, values.size() * sizeof(T)));
-  RETURN_IF_ERROR(hip::HipStatus(pluto_hip_memcpy_async(executor.stream(), device.data(),
-                                                        host.data(), host.size_bytes(), 1),
-                                 "upload"));
-  RETURN_IF_ERROR(executor.Synchronize());
-  return device;
-}
+using testing::UploadRaw;
 
-std::vector<uint8_t> Fp8(const std::vector<float>& values) {
-  std::vector<uint8_t> codes(values.size());
-  for (size_t i = 0; i < values.size(); ++i) codes[i] = pluto_oracle_f32_to_fp8_e4m3(values[i]);
-  return codes;
-}
+std::vector<uint8_t> Fp8(const std::vector<float>& values) { return testing::Fp8Codes(values); }
 
 TEST(ImportedLinearTest, SharesAllStorageWithoutMastersOrGradients) {
   auto executor = NewExecutor();

@@ -61,6 +61,26 @@ StatusOr<hip::Buffer> Upload(hip::Executor& executor, const std::vector<float>& 
   return device;
 }
 
+// Uploads raw elements of type T (bf16 bit patterns, FP8 codes) and waits.
+template <class T>
+StatusOr<hip::Buffer> UploadRaw(hip::Executor& executor, const std::vector<T>& values) {
+  ASSIGN_OR_RETURN(auto host, hip::PageLockedHostArray<T>::Allocate(executor, values.size()));
+  for (size_t i = 0; i < values.size(); ++i) host[i] = values[i];
+  ASSIGN_OR_RETURN(auto device, hip::Buffer::Allocate(executor, values.size() * sizeof(T)));
+  RETURN_IF_ERROR(hip::HipStatus(
+      pluto_hip_memcpy_async(executor.stream(), device.data(), host.data(), host.size_bytes(), 1),
+      "upload"));
+  RETURN_IF_ERROR(executor.Synchronize());
+  return device;
+}
+
+// OCP FP8 E4M3 codes of the values, rounded as the oracle rounds.
+inline std::vector<uint8_t> Fp8Codes(const std::vector<float>& values) {
+  std::vector<uint8_t> codes(values.size());
+  for (size_t i = 0; i < values.size(); ++i) codes[i] = pluto_oracle_f32_to_fp8_e4m3(values[i]);
+  return codes;
+}
+
 // Reads a device buffer of element type T back as floats.
 template <class T>
 std::vector<float> Read(const hip::Buffer& buffer) {
