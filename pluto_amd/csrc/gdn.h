@@ -7,20 +7,16 @@
 namespace pluto_hip {
 
 // Scratch written by the chunk-parallel kernel for one 64-token chunk of one
-// (sequence, head), all in matrix-core register order:
-//   U      fp32 [4 token tiles][8 column slices][64 lanes][4]        32 KiB
-//   -W     bf16 [4 token tiles][4 key blocks][64 lanes][8]           16 KiB
-//   cQ     bf16 same shape (exp(c) * q_scale * Q)                    16 KiB
-//   A2     bf16 [4 token tiles][2 token blocks][64 lanes][8]          8 KiB
-//   Kt     bf16 [8 key tiles][2 token blocks][64 lanes][8]           16 KiB
-//   decay  fp32 exp(c_C)
-constexpr size_t kGdnOffsetU = 0;
-constexpr size_t kGdnOffsetW = 32768;
-constexpr size_t kGdnOffsetQ = 49152;
-constexpr size_t kGdnOffsetA2 = 65536;
-constexpr size_t kGdnOffsetKt = 73728;
-constexpr size_t kGdnOffsetDecay = 90112;
-constexpr size_t kGdnChunkBytes = 90368;
+// (sequence, head):
+//   T        bf16 [4 token tiles][2 token blocks][64 lanes][8]   8 KiB
+//            (I + A)^-1 in matrix-core operand order
+//   A2       bf16 same shape: M o (Q K^T) with every factor       8 KiB
+//   factors  fp32 [4][64]: beta, beta exp(c)/|k|, q_scale exp(c)/|q|,
+//            exp(c_C - c)/|k| per token; then exp(c_C)            2 KiB
+constexpr size_t kGdnOffsetT = 0;
+constexpr size_t kGdnOffsetA2 = 8192;
+constexpr size_t kGdnOffsetFactors = 16384;
+constexpr size_t kGdnChunkBytes = 18432;
 
 struct GdnArgs {
   // Row `token` (= sequence * T + t) of q starts at q + token * q_token_stride
