@@ -44,7 +44,7 @@ MEASURED_TRAFFIC_BYTES = {
     ("mha_train_bf16", "flash_forward_kernel<64>"): 126.4e6,
     ("gqa_prefill", "flash_forward_kernel<128>"): 169.6e6 + 50.7e6,
     ("gqa_decode", "decode_fused_kernel<128,6>"): 1044.3e6 + 13.0e6,
-    ("gdn_scan", "gdn_chunk_prepare + gdn_chunk_scan"): 1119.5e6,
+    ("gdn_scan", "gdn_chunk_prepare + gdn_chunk_scan"): 1052.6e6,
 }
 
 NAMES = ["mha_train_bf16", "mha_fwd_fp32", "gqa_prefill", "gqa_decode", "gdn_scan"]

@@ -8,15 +8,17 @@ namespace pluto_hip {
 
 // Scratch written by the chunk-parallel kernel for one 64-token chunk of one
 // (sequence, head):
-//   T        bf16 [4 token tiles][2 token blocks][64 lanes][8]   8 KiB
-//            (I + A)^-1 in matrix-core operand order
-//   A2       bf16 same shape: M o (Q K^T) with every factor       8 KiB
+//   T        bf16 [6 fragments][64 lanes][8]                     6 KiB
+//            (I + A)^-1 in matrix-core operand order: fragment (token tile i,
+//            token block kb) for (0,0) (1,0) (2,0) (2,1) (3,0) (3,1); the other
+//            two are zero, the matrix being lower triangular
+//   A2       bf16 same shape: M o (Q K^T) with every factor       6 KiB
 //   factors  fp32 [4][64]: beta, beta exp(c)/|k|, q_scale exp(c)/|q|,
 //            exp(c_C - c)/|k| per token; then exp(c_C)            2 KiB
 constexpr size_t kGdnOffsetT = 0;
-constexpr size_t kGdnOffsetA2 = 8192;
-constexpr size_t kGdnOffsetFactors = 16384;
-constexpr size_t kGdnChunkBytes = 18432;
+constexpr size_t kGdnOffsetA2 = 6144;
+constexpr size_t kGdnOffsetFactors = 12288;
+constexpr size_t kGdnChunkBytes = 14336;
 
 struct GdnArgs {
   // Row `token` (= sequence * T + t) of q starts at q + token * q_token_stride

@@ -20,12 +20,12 @@
 //
 // Kernel 1 (gdn_chunk_prepare, one workgroup per chunk, fully parallel): the
 // two Gram matrices on the matrix cores from the raw bf16 inputs, T by a block
-// forward substitution on the matrix cores, and 18 KiB per chunk written out:
+// forward substitution on the matrix cores, and 14 KiB per chunk written out:
 // T and M o (Q K^T) as bf16 matrix-core operands, and the per-token factors.
 // Kernel 2 (gdn_chunk_scan, one workgroup per (sequence, head, 16 state
 // columns)): walks the chunks with v_mfma_f32_16x16x32_bf16, the state in FP32
 // accumulator registers of one wave, a second wave computing the outputs, two
-// more streaming each chunk's 18 KiB and its raw K, Q and V rows into LDS.
+// more streaming each chunk's 14 KiB and its raw K, Q and V rows into LDS.
 // State columns are independent, which is what gives the sequential part
 // 8 x batch x heads way parallelism.
 #include "gdn.h"
@@ -284,11 +284,13 @@ gdn_chunk_prepare(GdnArgs a) {
   uint4* t_out = reinterpret_cast<uint4*>(out + kGdnOffsetT);
   uint4* a2_out = reinterpret_cast<uint4*>(out + kGdnOffsetA2);
   // T and M o (Q K^T) as matrix-core operands over tokens j: fragment
-  // f = 2*tile + kb, lane (hq, m) = row 16 tile + m, slot (hq, e) = column
-  // 32 kb + 16 (e / 4) + 4 hq + e % 4
-  for (int piece = tid; piece < 8 * 64; piece += 256) {
+  // (tile, kb), lane (hq, m) = row 16 tile + m, slot (hq, e) = column
+  // 32 kb + 16 (e / 4) + 4 hq + e % 4; the two fragments above the diagonal
+  // are zero and are not stored
+  for (int piece = tid; piece < 6 * 64; piece += 256) {
     const int f = piece / 64, l = piece % 64;
-    const int tile = f / 2, kb = f % 2, hq = l / 16, m = l % 16;
+    const int tile = f < 2 ? f : 2 + (f - 2) / 2, kb = f < 2 ? 0 : (f - 2) % 2;
+    const int hq = l / 16, m = l % 16;
     const int row = 16 * tile + m, lo = 32 * kb + 4 * hq;
     uint2 w0 = *reinterpret_cast<const uint2*>(&sm.t[row][lo]);
     uint2 w1 = *reinterpret_cast<const uint2*>(&sm.t[row][lo + 16]);
@@ -313,7 +315,7 @@ gdn_chunk_prepare(GdnArgs a) {
 }
 
 // LDS stage of the sequential kernel for one chunk: the chunk's scratch as it
-// sits in memory (T | A2 | factors, 18 KiB), the raw K and Q rows gathered
+// sits in memory (T | A2 | factors, 14 KiB), the raw K and Q rows gathered
 // into matrix-core operand order (16 KiB each), and the 16 value columns of the
 // workgroup's slice (2 KiB).
 constexpr int kStageScratch = 0;
@@ -373,7 +375,7 @@ struct ScanSources {
   uint32_t k_row_bytes, q_row_bytes, v_row_bytes;
 };
 
-// The direct-to-LDS loads of one chunk, 1 KiB each: 18 of scratch, 16 of K,
+// The direct-to-LDS loads of one chunk, 1 KiB each: 14 of scratch, 16 of K,
 // 16 of Q, 2 of V.  Loader wave LOADER of LOADERS issues every LOADERS-th.
 constexpr int kFillScratch = static_cast<int>(kGdnChunkBytes) / 1024;
 constexpr int kScanFillLoads = kFillScratch + 16 + 16 + 2;
@@ -444,12 +446,12 @@ constexpr int kScanAhead = 4;
 __device__ inline void scan_touch(const ScanSources& src, uint32_t dump_address, int chunk,
                                   int slice, int lane) {
   const uint32_t lane_bytes = static_cast<uint32_t>(lane) * 16u;
-  // scratch: 18 KiB / 8 = 2304 bytes, three loads (the last one runs into the
+  // scratch: 14 KiB / 8 = 1792 bytes, two loads (the second runs into the
   // next slice's share, or past the end of the scratch, where it reads zeros)
   const uint32_t scratch = static_cast<uint32_t>(chunk) * static_cast<uint32_t>(kGdnChunkBytes) +
                            static_cast<uint32_t>(slice) * (kGdnChunkBytes / SLICES) + lane_bytes;
 #pragma unroll
-  for (int i = 0; i < 3; ++i) lds_dma_16(src.scratch, dump_address, scratch + i * 1024, 0);
+  for (int i = 0; i < 2; ++i) lds_dma_16(src.scratch, dump_address, scratch + i * 1024, 0);
   // K and Q: eight token rows of 256 bytes each, four rows a load
   const uint32_t row = static_cast<uint32_t>(chunk) * C + 8 * slice + lane / 16;
   const uint32_t piece = (lane % 16) * 16u;
@@ -562,12 +564,12 @@ __device__ __forceinline__ void chain_step(const ScanContext ctx, const lds_byte
 #pragma unroll
       for (int j = 0; j < 4; ++j) f2[j] = factor_in[16 + 4 * j];
       t_reg[0] = t_in[0 * 64];
-      t_reg[1] = t_in[2 * 64];
-      t_reg[2] = t_in[4 * 64];
+      t_reg[1] = t_in[1 * 64];
+      t_reg[2] = t_in[2 * 64];
     } else if (i == 2) {
-      t_reg[3] = t_in[5 * 64];
-      t_reg[4] = t_in[6 * 64];
-      t_reg[5] = t_in[7 * 64];
+      t_reg[3] = t_in[3 * 64];
+      t_reg[4] = t_in[4 * 64];
+      t_reg[5] = t_in[5 * 64];
 #pragma unroll
       for (int j = 0; j < 4; ++j) f4[j] = factor_in[48 + 4 * j];
     }
@@ -684,12 +686,12 @@ __device__ __forceinline__ void output_step(const ScanContext ctx, int chunk, co
     }
     if (i == 1) {
       a2_reg[0] = a2_in[0 * 64];
-      a2_reg[1] = a2_in[2 * 64];
-      a2_reg[2] = a2_in[4 * 64];
+      a2_reg[1] = a2_in[1 * 64];
+      a2_reg[2] = a2_in[2 * 64];
     } else if (i == 2) {
-      a2_reg[3] = a2_in[5 * 64];
-      a2_reg[4] = a2_in[6 * 64];
-      a2_reg[5] = a2_in[7 * 64];
+      a2_reg[3] = a2_in[3 * 64];
+      a2_reg[4] = a2_in[4 * 64];
+      a2_reg[5] = a2_in[5 * 64];
 #pragma unroll
       for (int j = 0; j < 4; ++j) f3[j] = factor_in[32 + 4 * j];
     }
