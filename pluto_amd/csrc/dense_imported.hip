@@ -10,6 +10,8 @@
 // rows and reads them in 16-byte pieces (whenever rows start 16-byte aligned),
 // the token comes from the FP32 copy the first kernel leaves in the workspace;
 // all arithmetic is FP32, the 64 lane sums are added by a butterfly.
+#include <algorithm>
+
 #include "dense.h"
 
 namespace pluto_hip {
@@ -211,26 +213,34 @@ __global__ void __launch_bounds__(256) imported_matvec_kernel(MatVecArgs a) {
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(16))) float floatx16;
 
-// tokens as FP8 values in bf16 [tokens, n] and their group scales [tokens, n / 128]
+// Tokens as FP8 values in bf16 and their group scales [tokens, n / 128].  The
+// values are written in the order the matrix-core kernel reads them, so that
+// each of its loads is one contiguous KiB: [pass of 32 tokens][block of 128
+// columns][step j][lane = token % 32 + 32 h][8], the lane's elements being
+// columns 128 block + 64 h + 8 j .. + 7.
 __global__ void __launch_bounds__(kGroup)
 imported_token_fp8_kernel(const uint16_t* x, int n, uint16_t* values, float* scales) {
   __shared__ float largest[2];
-  x += static_cast<size_t>(blockIdx.y) * n;
-  values += static_cast<size_t>(blockIdx.y) * n;
-  const int i = blockIdx.x * kGroup + threadIdx.x;
+  const int token = blockIdx.y, block = blockIdx.x, c = threadIdx.x;
+  x += static_cast<size_t>(token) * n;
+  const int i = block * kGroup + c;
   const float v = i < n ? bf16_bits_to_float(x[i]) : 0.0f;
   const float mine = wave_max(fabsf(v));
   if (threadIdx.x % 64 == 0) largest[threadIdx.x / 64] = mine;
   __syncthreads();
   const float scale = fmaxf(largest[0], largest[1]) / 448.0f;
-  if (i < n) values[i] = float_to_bf16_bits(fp8_round(v / fmaxf(scale, 1e-12f)));
-  if (threadIdx.x == 0) scales[static_cast<size_t>(blockIdx.y) * gridDim.x + blockIdx.x] = scale;
+  const size_t pass = token / 32;
+  const int lane = token % 32 + 32 * (c / 64), step = (c % 64) / 8;
+  if (i < n)
+    values[(((pass * gridDim.x + block) * 8 + step) * 64 + lane) * 8 + c % 8] =
+        float_to_bf16_bits(fp8_round(v / fmaxf(scale, 1e-12f)));
+  if (threadIdx.x == 0) scales[static_cast<size_t>(token) * gridDim.x + block] = scale;
 }
 
 struct TileArgs {
   const void* weights = nullptr;
   const float* weight_scales = nullptr;  // FP8 only
-  const uint16_t* tokens = nullptr;      // bf16 [count, cols]
+  const uint16_t* tokens = nullptr;      // bf16 [count, cols]; FP8: one pass in operand order
   const float* token_scales = nullptr;   // FP8 only: [count, cols / 128]
   uint16_t* out = nullptr;               // [count, rows]
   int cols = 0, rows = 0, count = 0;     // count <= 32
@@ -244,7 +254,8 @@ __device__ inline uint32_t fp8_pair_to_bf16(uint32_t word) {
 
 constexpr int kTileWaves = 8;  // waves that split a tile's contraction
 
-template <bool FP8>
+// AHEAD (FP8 only): blocks of a wave whose weight loads are issued together.
+template <bool FP8, int AHEAD = 1>
 __global__ void __launch_bounds__(64 * kTileWaves) imported_tile_kernel(TileArgs a) {
   __shared__ float partial[kTileWaves - 1][16][64];
   const int lane = threadIdx.x % 64, n = lane % 32, h = lane / 32;
@@ -255,39 +266,70 @@ __global__ void __launch_bounds__(64 * kTileWaves) imported_tile_kernel(TileArgs
   const int groups = a.cols / kGroup;
   const unsigned char* w = static_cast<const unsigned char*>(a.weights) +
                            (static_cast<size_t>(row) * a.cols + 64 * h) * (FP8 ? 1 : 2);
-  const uint16_t* x = a.tokens + static_cast<size_t>(token) * a.cols + 64 * h;
+  // FP8: operand order, 1 KiB a step; otherwise the token's own row
+  const uint16_t* x = FP8 ? a.tokens + lane * 8 : a.tokens + static_cast<size_t>(token) * a.cols + 64 * h;
   const float* block_scale =
       FP8 ? a.weight_scales + static_cast<size_t>(row_base / kGroup) * groups : nullptr;
   const float* group_scale = FP8 ? a.token_scales + static_cast<size_t>(token) * groups : nullptr;
   floatx16 total;
 #pragma unroll
   for (int i = 0; i < 16; ++i) total[i] = 0.0f;
-  for (int g = wave; g < groups; g += kTileWaves) {
-    uint4 xs[8];
+  if constexpr (FP8) {
+    // A wave's weight rows are few bytes (64 a lane and block): the loads of
+    // AHEAD of its blocks (all of them for widths up to 8192) are issued before
+    // anything is waited for, so that the latency of HBM is paid once a batch
+    // and not once a block; the tokens (L2 hits) follow one block ahead of the
+    // products.  Blocks past the end repeat the last one (loads without
+    // branches) and are not added.
+    constexpr int kAhead = AHEAD;
+    for (int g0 = wave; g0 < groups; g0 += kTileWaves * kAhead) {
+      uint4 raw[kAhead][4];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) xs[j] = *reinterpret_cast<const uint4*>(x + g * kGroup + 8 * j);
-    if constexpr (FP8) {
-      uint4 raw[4];
+      for (int b = 0; b < kAhead; ++b) {
+        const int g = min(g0 + b * kTileWaves, groups - 1);
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-        raw[j] = *reinterpret_cast<const uint4*>(w + static_cast<size_t>(g) * kGroup + 16 * j);
-      floatx16 acc;
-#pragma unroll
-      for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const uint32_t lo = j % 2 == 0 ? raw[j / 2].x : raw[j / 2].z;
-        const uint32_t hi = j % 2 == 0 ? raw[j / 2].y : raw[j / 2].w;
-        const uint4 bits = make_uint4(fp8_pair_to_bf16<false>(lo), fp8_pair_to_bf16<true>(lo),
-                                      fp8_pair_to_bf16<false>(hi), fp8_pair_to_bf16<true>(hi));
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, bits),
-                                                      __builtin_bit_cast(bf16x8, xs[j]), acc, 0, 0,
-                                                      0);
+        for (int j = 0; j < 4; ++j)
+          raw[b][j] = *reinterpret_cast<const uint4*>(w + static_cast<size_t>(g) * kGroup + 16 * j);
       }
-      const float scale = block_scale[g] * group_scale[g];
+      uint4 xs[2][8];
 #pragma unroll
-      for (int i = 0; i < 16; ++i) total[i] += acc[i] * scale;
-    } else {
+      for (int j = 0; j < 8; ++j)
+        xs[0][j] = *reinterpret_cast<const uint4*>(x + (static_cast<size_t>(g0) * 8 + j) * 512);
+#pragma unroll
+      for (int b = 0; b < kAhead; ++b) {
+        const int g = g0 + b * kTileWaves;
+        if (b + 1 < kAhead) {
+          const int next = min(g + kTileWaves, groups - 1);
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            xs[(b + 1) % 2][j] =
+                *reinterpret_cast<const uint4*>(x + (static_cast<size_t>(next) * 8 + j) * 512);
+        }
+        floatx16 acc;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const uint32_t lo = j % 2 == 0 ? raw[b][j / 2].x : raw[b][j / 2].z;
+          const uint32_t hi = j % 2 == 0 ? raw[b][j / 2].y : raw[b][j / 2].w;
+          const uint4 bits = make_uint4(fp8_pair_to_bf16<false>(lo), fp8_pair_to_bf16<true>(lo),
+                                        fp8_pair_to_bf16<false>(hi), fp8_pair_to_bf16<true>(hi));
+          acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, bits),
+                                                        __builtin_bit_cast(bf16x8, xs[b % 2][j]),
+                                                        acc, 0, 0, 0);
+        }
+        // a block past the end contributes nothing (its scale is read in range)
+        const int in_range = min(g, groups - 1);
+        const float scale = g < groups ? block_scale[in_range] * group_scale[in_range] : 0.0f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) total[i] += acc[i] * scale;
+      }
+    }
+  } else {
+    for (int g = wave; g < groups; g += kTileWaves) {
+      uint4 xs[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) xs[j] = *reinterpret_cast<const uint4*>(x + g * kGroup + 8 * j);
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const uint4 bits =
@@ -320,6 +362,26 @@ __global__ void __launch_bounds__(64 * kTileWaves) imported_tile_kernel(TileArgs
     }
 }
 
+template <int AHEAD>
+void launch_fp8_tiles_ahead(hipStream_t s, const TileArgs& t, int blocks) {
+  imported_tile_kernel<true, AHEAD><<<blocks, 64 * kTileWaves, 0, s>>>(t);
+}
+
+// Picks AHEAD = blocks a wave owns, up to eight.
+void launch_fp8_tiles(hipStream_t s, const TileArgs& t, int blocks) {
+  const int groups = t.cols / kGroup;
+  switch (std::min(8, (groups + kTileWaves - 1) / kTileWaves)) {
+    case 1: return launch_fp8_tiles_ahead<1>(s, t, blocks);
+    case 2: return launch_fp8_tiles_ahead<2>(s, t, blocks);
+    case 3: return launch_fp8_tiles_ahead<3>(s, t, blocks);
+    case 4: return launch_fp8_tiles_ahead<4>(s, t, blocks);
+    case 5: return launch_fp8_tiles_ahead<5>(s, t, blocks);
+    case 6: return launch_fp8_tiles_ahead<6>(s, t, blocks);
+    case 7: return launch_fp8_tiles_ahead<7>(s, t, blocks);
+    default: return launch_fp8_tiles_ahead<8>(s, t, blocks);
+  }
+}
+
 // The matrix-core path takes bf16 and FP8 weights whose rows are whole
 // 128-element blocks; fewer than nine tokens are cheaper on the vector path.
 bool tile_path(int storage, int tokens, int input_dim) {
@@ -349,10 +411,20 @@ void launch_matvec(hipStream_t s, MatVecArgs a, int tokens) {
 
 }  // namespace
 
+namespace {
+size_t tile_values_bytes(int tokens, int input_dim) {
+  const size_t padded = (static_cast<size_t>(tokens) + 31) / 32 * 32;
+  return align_up(padded * input_dim * 2, 256);
+}
+}  // namespace
+
 size_t dense_imported_workspace_bytes(int tokens, int input_dim) {
-  // FP32 tokens (vector path), or their FP8 values in bf16 and the group
-  // scales (matrix-core path): the first is the larger
-  return align_up(static_cast<size_t>(tokens) * input_dim * sizeof(float), 256) + 256;
+  // FP32 tokens (vector path), or their FP8 values in bf16, in whole passes of
+  // 32 tokens, and the group scales (matrix-core path)
+  const size_t vector_path = align_up(static_cast<size_t>(tokens) * input_dim * sizeof(float), 256);
+  const size_t groups = (static_cast<size_t>(input_dim) + kGroup - 1) / kGroup;
+  const size_t tile_path = tile_values_bytes(tokens, input_dim) + align_up(tokens * groups * 4, 256);
+  return std::max(vector_path, tile_path) + 256;
 }
 
 int launch_dense_imported_forward(hipStream_t s, int storage, const void* weights,
@@ -370,8 +442,8 @@ int launch_dense_imported_forward(hipStream_t s, int storage, const void* weight
     t.rows = output_dim;
     if (fp8) {
       uint16_t* values = static_cast<uint16_t*>(workspace);
-      float* token_scales = reinterpret_cast<float*>(
-          static_cast<char*>(workspace) + align_up(static_cast<size_t>(tokens) * input_dim * 2, 256));
+      float* token_scales = reinterpret_cast<float*>(static_cast<char*>(workspace) +
+                                                     tile_values_bytes(tokens, input_dim));
       imported_token_fp8_kernel<<<groups, kGroup, 0, s>>>(static_cast<const uint16_t*>(input),
                                                           input_dim, values, token_scales);
       t.tokens = values;
@@ -382,7 +454,7 @@ int launch_dense_imported_forward(hipStream_t s, int storage, const void* weight
     for (int done = 0; done < tokens; done += 32) {
       t.count = tokens - done < 32 ? tokens - done : 32;
       if (fp8)
-        imported_tile_kernel<true><<<blocks, 64 * kTileWaves, 0, s>>>(t);
+        launch_fp8_tiles(s, t, blocks);
       else
         imported_tile_kernel<false><<<blocks, 64 * kTileWaves, 0, s>>>(t);
       t.tokens += static_cast<size_t>(32) * input_dim;
