@@ -430,25 +430,46 @@ flash_dkv_kernel(GenericBackwardArgs a, const float* __restrict__ lse2,
         }
       }
     }
-    if (key_row < T) {
-      float* dk = a.d_qkv + (seq_row0 + key_row) * 3 * E + E + head * D;
-      float* dv = dk + E;
+    // dK and dV leave through LDS so that every store instruction writes whole
+    // rows (16 lanes x 16 bytes): written straight from the accumulators, a
+    // lane's 16-byte pieces lie 9 KiB apart and each store touches 32 lines.
+    // One tensor at a time, 32 keys x D floats a wave, pieces swizzled by row.
+    __syncthreads();  // every wave is done with the tile stages
+    {
+      // 64 columns of one tensor at a time: 32 keys x 64 floats a wave, 32 KiB
+      static_assert(4 * 32 * 64 * 4 <= 2 * kStageBytes, "the stages hold one step of the workgroup");
+      constexpr int kPieces = 16;  // 16-byte pieces in 64 columns
+      float4* area = reinterpret_cast<float4*>(lds) + wave * 32 * kPieces;
+      const int out_piece = lane % kPieces, out_row = lane / kPieces;
 #pragma unroll
-      for (int db = 0; db < DB; ++db)
+      for (int step = 0; step < 2 * (D / 64); ++step) {
+        const int tensor = step / (D / 64), half = step % (D / 64);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          float4 kv, vv;
-          kv.x = dk_acc[db][4 * j + 0] * a.scale;
-          kv.y = dk_acc[db][4 * j + 1] * a.scale;
-          kv.z = dk_acc[db][4 * j + 2] * a.scale;
-          kv.w = dk_acc[db][4 * j + 3] * a.scale;
-          vv.x = dv_acc[db][4 * j + 0];
-          vv.y = dv_acc[db][4 * j + 1];
-          vv.z = dv_acc[db][4 * j + 2];
-          vv.w = dv_acc[db][4 * j + 3];
-          *reinterpret_cast<float4*>(dk + 32 * db + 8 * j + 4 * h) = kv;
-          *reinterpret_cast<float4*>(dv + 32 * db + 8 * j + 4 * h) = vv;
+        for (int d2 = 0; d2 < 2; ++d2)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const floatx16& acc = tensor == 0 ? dk_acc[2 * half + d2] : dv_acc[2 * half + d2];
+            const float factor = tensor == 0 ? a.scale : 1.0f;
+            float4 value;
+            value.x = acc[4 * j + 0] * factor;
+            value.y = acc[4 * j + 1] * factor;
+            value.z = acc[4 * j + 2] * factor;
+            value.w = acc[4 * j + 3] * factor;
+            const int piece = 8 * d2 + 2 * j + h;
+            area[n * kPieces + (piece ^ (n % kPieces))] = value;
+          }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the wave reads what its own lanes wrote
+        float* dst = a.d_qkv + (seq_row0 + k0 + 32 * wave) * 3 * E + (1 + tensor) * E + head * D +
+                     64 * half;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const int row = 4 * i + out_row;
+          const float4 value = area[row * kPieces + (out_piece ^ (row % kPieces))];
+          if (k0 + 32 * wave + row < T)
+            *reinterpret_cast<float4*>(dst + static_cast<long long>(row) * 3 * E + 4 * out_piece) = value;
         }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // before the area is overwritten
+      }
     }
     __syncthreads();  // the next pass refills a stage
   }
