@@ -11,6 +11,12 @@ D=64.  The default run (--workload all) appends the other four configurations
 of the path under "workloads", each with its own `roofline` and
 `cpu_baseline`; --workload NAME runs one workload alone.
 
+Each workload first runs untimed for --settle-seconds (0.3 s) of continuous
+work, then the W warm-up steps, then the K timed steps: the part reaches the
+clocks it sustains only after some 30 ms of work, and a training or serving
+loop lives in that state (the first 20 steps after an idle period run 10-15 %
+slower in the matrix-core kernels).  `config.settle_s` records the setting.
+
 Exactly one JSON line is printed.  `roofline` describes the kernel of the
 step that takes longest: its average duration is measured live with HIP
 events on the launch stream around calls that queue only that kernel (the
@@ -66,6 +72,9 @@ def parse_args():
     ap.add_argument("--cpu-seconds", type=float, default=5.0,
                     help="CPU time budget of each cpu_baseline leg")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--settle-seconds", type=float, default=0.3,
+                    help="untimed continuous running of each workload before its warm-up steps, "
+                         "so that the timed steps see the clocks the part sustains (0 = none)")
     ap.add_argument("--launch", default="eager", choices=["graph", "eager"],
                     help="graph: replay the timed steps from a HIP graph where the workload supports "
                          "it (measured: 0.232 instead of 0.235 ms for the training step, 0.203 "
@@ -739,8 +748,18 @@ def capture_step(torch, w):
     return graph
 
 
-def measure(torch, capi, w, steps, warmup, launch="eager"):
+def measure(torch, capi, w, steps, warmup, launch="eager", settle_seconds=0.0):
     stream = torch.cuda.current_stream()
+    # The part needs some 30 ms of continuous work to reach the clocks it then
+    # sustains (the matrix-core kernels run 10-15 % slower until then), far more
+    # than a handful of warm-up steps of 0.2 ms: the step first runs untimed
+    # for `settle_seconds`, then come the warm-up steps asked for.
+    settle_until = time.perf_counter() + settle_seconds
+    while time.perf_counter() < settle_until:
+        for _ in range(50):
+            w["step"]()
+        torch.cuda.synchronize()
+    w["config"]["settle_s"] = settle_seconds
     for _ in range(warmup):
         w["step"]()
     torch.cuda.synchronize()
@@ -805,7 +824,7 @@ def main():
     capi.lib()
     head = "mha_train_bf16" if args.workload == "all" else args.workload
     w = WORKLOADS[head](torch, capi)
-    m = measure(torch, capi, w, args.steps, args.warmup, args.launch)
+    m = measure(torch, capi, w, args.steps, args.warmup, args.launch, args.settle_seconds)
     result = {
         "metric": w["metric"], "value": round(m["value"], 3), "unit": w["unit"], "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(m["ms_per_step"], 4),
@@ -824,7 +843,7 @@ def main():
             del w
             torch.cuda.empty_cache()
             w = WORKLOADS[name](torch, capi)
-            mm = measure(torch, capi, w, args.steps, args.warmup, args.launch)
+            mm = measure(torch, capi, w, args.steps, args.warmup, args.launch, args.settle_seconds)
             others[name] = {"metric": w["metric"], "value": round(mm["value"], 3), "unit": w["unit"],
                             "ms_per_step": round(mm["ms_per_step"], 4), "dtype": w["dtype"],
                             "config": w["config"], "roofline": roofline(name, w, mm),
