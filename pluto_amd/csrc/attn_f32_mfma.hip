@@ -3,8 +3,13 @@
 // FlashAttentionForwardKernel (src/llm/layers/attention.cc:98-170), where
 // products and sums stay in FP32.
 //
-// One wave owns 32 query rows of one (sequence, head) and walks the visible
-// keys in tiles of 32.  As in the bf16 kernels the products are transposed,
+// A workgroup of four waves owns 32 query rows of one (sequence, head); wave w
+// walks the visible key tiles (32 keys each) w, w + 4, ... with its own running
+// maximum, sum and output, and wave 0 merges the four partial results through
+// LDS in wave order.  The FP32 matrix instruction is slow (64 cycles for
+// 32x32x2), a row block near the end of a sequence has many tiles and there
+// are few row blocks, so splitting the keys is what fills the machine.  As in
+// the bf16 kernels the products are transposed,
 // S^T = K Q^T and O^T = V^T P^T, so that a lane owns one query column: its row
 // maximum and sum are lane-local up to one exchange between the two lane
 // halves, and P^T leaves the accumulator in B-operand order.  The contraction
@@ -19,11 +24,16 @@
 namespace pluto_hip {
 namespace {
 
+constexpr int kKeySplit = 4;  // waves per workgroup, each taking every fourth key tile
+
 template <int D>
-__global__ void __launch_bounds__(64)
+__global__ void __launch_bounds__(64 * kKeySplit)
 f32_forward_kernel(GenericForwardArgs a) {
   constexpr int HALF = D / 2, DB = D / 32;
-  const int lane = threadIdx.x, h = lane / 32, n = lane % 32;
+  __shared__ float part_o[kKeySplit - 1][DB * 16][64];
+  __shared__ float part_max[kKeySplit - 1][64], part_sum[kKeySplit - 1][64];
+  const int lane = threadIdx.x % 64, h = lane / 32, n = lane % 32;
+  const int wave = threadIdx.x / 64;
   const int q0 = blockIdx.x * 32, head = blockIdx.y, seq = blockIdx.z;
   const int kv_head = head / a.group;
   const float* q_base = static_cast<const float*>(a.q.base) + seq * a.q.seq_stride +
@@ -62,20 +72,20 @@ f32_forward_kernel(GenericForwardArgs a) {
   float4 k_next[HALF / 4];
   {
     const float4* row = reinterpret_cast<const float4*>(
-        k_base + min(n, a.kv_rows - 1) * a.k.row_stride + h * HALF);
+        k_base + min(wave * 32 + n, a.kv_rows - 1) * a.k.row_stride + h * HALF);
 #pragma unroll
     for (int j = 0; j < HALF / 4; ++j) k_next[j] = row[j];
   }
-  for (int kt = 0; kt < key_tiles; ++kt) {
+  for (int kt = wave; kt < key_tiles; kt += kKeySplit) {
     float kf[HALF];
 #pragma unroll
     for (int j = 0; j < HALF / 4; ++j) {
       kf[4 * j] = k_next[j].x; kf[4 * j + 1] = k_next[j].y;
       kf[4 * j + 2] = k_next[j].z; kf[4 * j + 3] = k_next[j].w;
     }
-    if (kt + 1 < key_tiles) {
+    if (kt + kKeySplit < key_tiles) {
       const float4* row = reinterpret_cast<const float4*>(
-          k_base + min((kt + 1) * 32 + n, a.kv_rows - 1) * a.k.row_stride + h * HALF);
+          k_base + min((kt + kKeySplit) * 32 + n, a.kv_rows - 1) * a.k.row_stride + h * HALF);
 #pragma unroll
       for (int j = 0; j < HALF / 4; ++j) k_next[j] = row[j];
     }
@@ -122,6 +132,39 @@ f32_forward_kernel(GenericForwardArgs a) {
       for (int i = 0; i < 16; ++i)
         o[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(values[db][i], s[i], o[db], 0, 0, 0);
     }
+  }
+  // ---- merge: every wave's result is relative to its own maximum ------------
+  if (wave > 0) {
+    part_max[wave - 1][lane] = running_max;
+    part_sum[wave - 1][lane] = running_sum;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) part_o[wave - 1][db * 16 + i][lane] = o[db][i];
+  }
+  __syncthreads();
+  if (wave > 0) return;
+  {
+    float maximum = running_max;
+#pragma unroll
+    for (int w = 0; w < kKeySplit - 1; ++w) maximum = fmaxf(maximum, part_max[w][lane]);
+    // a wave without tiles contributes weight 2^(kMasked - maximum) = 0
+    const float own = __builtin_amdgcn_exp2f(running_max - maximum);
+    running_sum *= own;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) o[db][i] *= own;
+#pragma unroll
+    for (int w = 0; w < kKeySplit - 1; ++w) {
+      const float weight = __builtin_amdgcn_exp2f(part_max[w][lane] - maximum);
+      running_sum += part_sum[w][lane] * weight;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[db][i] += part_o[w][db * 16 + i][lane] * weight;
+    }
+    running_max = maximum;
   }
   if (query >= a.q_rows) return;
   const float normalizer = running_sum > 0.0f ? running_sum : 1.0f;
@@ -174,9 +217,9 @@ int launch_f32_forward(hipStream_t stream, const GenericForwardArgs& a, int sequ
   if (grid.y > 65535u || grid.z > 65535u) return PLUTO_HIP_EUNSUPPORTED;
   if (!kernel_enabled(kMainKernel)) return 0;
   switch (a.head_dim) {
-    case 32: f32_forward_kernel<32><<<grid, 64, 0, stream>>>(a); break;
-    case 64: f32_forward_kernel<64><<<grid, 64, 0, stream>>>(a); break;
-    case 128: f32_forward_kernel<128><<<grid, 64, 0, stream>>>(a); break;
+    case 32: f32_forward_kernel<32><<<grid, 64 * kKeySplit, 0, stream>>>(a); break;
+    case 64: f32_forward_kernel<64><<<grid, 64 * kKeySplit, 0, stream>>>(a); break;
+    case 128: f32_forward_kernel<128><<<grid, 64 * kKeySplit, 0, stream>>>(a); break;
     default: return PLUTO_HIP_EUNSUPPORTED;
   }
   return launch_status();
