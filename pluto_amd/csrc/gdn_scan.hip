@@ -77,18 +77,20 @@ __device__ inline void split_operand(const floatx4& first, const floatx4& second
   }
 }
 
-// 52 KiB, so that three workgroups share a compute unit's LDS: once the Gram
-// matrices are done the rows of K and Q make room for the two bf16 results.
+// 35 KiB, so that four workgroups share a compute unit's LDS (the kernel is a
+// chain of short, barrier-separated phases and lives on occupancy): once the
+// Gram matrices are done the rows of K make room for A, and A in turn for the
+// finished inverse; the rows of Q make room for the second bf16 result.
 struct ChunkSmem {
   union {
     uint16_t k[C][DK + 8];  // raw K rows (bf16)
-    uint16_t t[C][C + 8];   // later: (I + A)^-1, bf16
+    float a[C][C + 4];      // then: strictly lower triangular A (FP32) and the blocks of its solve
+    uint16_t t[C][C + 8];   // last: (I + A)^-1, bf16
   };
   union {
     uint16_t q[C][DK + 8];  // raw Q rows
     uint16_t a2[C][C + 8];  // later: M o (Q K^T) with all factors, bf16
   };
-  float a[C][C + 4];        // strictly lower triangular A (FP32), then the blocks of its solve
   float cum[C];             // inclusive cumulative log decay
   float beta[C];
   float inv_k[C];           // 1/|k| (or 1)
@@ -161,9 +163,12 @@ gdn_chunk_prepare(GdnArgs a) {
   {
     const int ti = wave / 2, tj = wave % 2;
     const int h = lane / 32, n = lane % 32;
-    float a2v[16];
+    float a2v[16], av[16];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) a2v[i] = 0.0f;
+    for (int i = 0; i < 16; ++i) {
+      a2v[i] = 0.0f;
+      av[i] = 0.0f;
+    }
     if (tj <= ti) {
       floatx16 gk, gq;
 #pragma unroll
@@ -185,19 +190,19 @@ gdn_chunk_prepare(GdnArgs a) {
       for (int i = 0; i < 16; ++i) {
         const int row = 32 * ti + 8 * (i / 4) + 4 * h + (i % 4);  // token i
         const float decay = __expf(fminf(sm.cum[row] - cum_j, 0.0f));
-        float av = 0.0f;
-        if (col < row) av = sm.beta[row] * decay * sm.inv_k[row] * inv_kj * gk[i];
+        if (col < row) av[i] = sm.beta[row] * decay * sm.inv_k[row] * inv_kj * gk[i];
         if (col <= row) a2v[i] = decay * sm.q_factor[row] * inv_kj * gq[i];
-        sm.a[row][col] = av;
       }
-    } else {
-      for (int i = lane; i < 32 * 32; i += 64) sm.a[32 * ti + i / 32][32 * tj + i % 32] = 0.0f;
     }
     __syncthreads();  // nobody reads the rows of K and Q any more
 #pragma unroll
-    for (int i = 0; i < 16; ++i)
-      sm.a2[32 * ti + 8 * (i / 4) + 4 * h + (i % 4)][32 * tj + n] = float_to_bf16_bits(a2v[i]);
+    for (int i = 0; i < 16; ++i) {
+      const int row = 32 * ti + 8 * (i / 4) + 4 * h + (i % 4);
+      sm.a[row][32 * tj + n] = av[i];  // the tile above the diagonal is zero
+      sm.a2[row][32 * tj + n] = float_to_bf16_bits(a2v[i]);
+    }
   }
+  __syncthreads();
 
   // ---- T = (I + A)^-1 by blocks of 16 rows on the matrix cores.  With T_b the
   // inverse of diagonal block b of I + A, block row b of the solve X of
@@ -271,6 +276,7 @@ gdn_chunk_prepare(GdnArgs a) {
       acc = mfma16(t_lo, r_hi, acc);
       x[b] = mfma16(t_hi, r_lo, acc);
     }
+    __syncthreads();  // every wave has read what it needs of A: T takes its place
 #pragma unroll
     for (int b = 0; b < 4; ++b)
 #pragma unroll
