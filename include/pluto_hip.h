@@ -527,8 +527,10 @@ int pluto_hip_test_force_generic(int enabled);
  * class bit is cleared in `mask` (1 = the kernel that bounds the call: flash
  * attention forward, key-owned attention backward, split-K decode, delta-net
  * scan; 2 = the query-owned attention backward kernel; 4 = auxiliary kernels:
- * preparation, tables, combines).  A benchmark runs the whole call once, then
- * times one class with events around the call.  Returns the previous mask;
+ * preparation, tables, combines; 16 = not a kernel: with this bit cleared the
+ * attention forward at head width 128 keeps to its four-wave kernel whatever
+ * the sequence length, which lets a test compare its two kernels).  A benchmark
+ * runs the whole call once, then times one class with events around the call.  Returns the previous mask;
  * the default, ~0u, runs everything.  Process-wide like the switch above, and
  * like it written by nothing on the product path. */
 unsigned pluto_hip_test_kernel_classes(unsigned mask);

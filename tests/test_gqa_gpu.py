@@ -291,6 +291,49 @@ def test_config3_prefill_8192(capi, oracle):
     assert_close_bf16(got, out2.float().cpu().numpy(), "config 3 vs fp32-arithmetic kernel")
 
 
+@pytest.mark.parametrize("lengths", [(1024,), (1301,), (1100, 1237)])
+def test_long_prefill_kernels_agree_bit_for_bit(capi, oracle, lengths):
+    # From 1024 rows on the forward at head width 128 runs its eight-wave kernel
+    # (two waves a SIMD one phase apart, 256-row tiles, three LDS stages).  It
+    # walks the keys in the same order with the same arithmetic as the four-wave
+    # kernel, so outputs, statistics and cache must be identical: whole tiles,
+    # a ragged last tile, and a second piece that continues a filled cache.
+    qh, kh, d = 6, 2, 128
+    total = sum(lengths)
+    kw = dict(query_heads=qh, key_value_heads=kh, head_dim=d, rotary_dim=32, capacity=total)
+    p, po = both_params(capi, oracle, **kw)
+    rng = np.random.default_rng(11)
+    qg, k, v = make_sequence(oracle, rng, total, qh, kh, d)
+    qw, kw_ = dev(values(d, 0.2, 0.3)), dev(values(d, 0.8, 0.4))
+    bf = torch.bfloat16
+    results = []
+    for mask in (0xffffffff, 0xffffffff & ~capi.PING_PONG):
+        cache = capi.KvCache(total, kh, d)
+        outs = []
+        with capi.only_kernels(mask):
+            start = 0
+            for length in lengths:
+                piece = slice(start, start + length)
+                outs.append(capi.gqa_prefill(p, dev(qg[piece], bf), dev(k[piece], bf),
+                                             dev(v[piece], bf), qw, kw_, cache,
+                                             start_position=start, want_lse=True))
+                assert capi.last_path() == capi.PATH_FLASH
+                start += length
+            torch.cuda.synchronize()
+        results.append((outs, cache))
+    (new, new_cache), (old, old_cache) = results
+    for (out_new, lse_new), (out_old, lse_old) in zip(new, old):
+        assert torch.equal(out_new, out_old)
+        assert torch.equal(lse_new, lse_old)
+    assert torch.equal(new_cache.keys, old_cache.keys)
+    assert torch.equal(new_cache.values, old_cache.values)
+    # and the last rows against the oracle
+    want = oracle.gqa_sequence(po, qg, k, v, values(d, 0.2, 0.3), values(d, 0.8, 0.4),
+                               rows=(total - 3, total))
+    got = new[-1][0].float().cpu().numpy()
+    assert_close_bf16(got[-3:], want["out"][total - 3:total], "last rows of the long prefill")
+
+
 def test_config4_batched_decode(capi, oracle):
     # batch 32, context length ~ U[1024, 32768] (seed 3), 24 query heads, 4 KV
     # heads, D=128, bf16 cache, split-K over 512-token blocks.
