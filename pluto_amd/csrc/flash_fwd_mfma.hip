@@ -399,8 +399,10 @@ flash_forward_kernel(FlashForwardArgs a_in, int unit_count) {
 // one instruction every four cycles, whatever its kind, and stalls on its own
 // dependencies, while the matrix pipe needs a new instruction only every 32.
 // Per 32-key block a wave has a matrix phase M(b) = { S^T of block b,
-// O^T += V^T P^T of block b-1 } and a vector phase V(b) = { LDS reads of the
-// operands of M(b+1), softmax of block b }.  Here a workgroup has eight waves,
+// O^T += V^T P^T of block b-1 } and a vector phase V(b) = { softmax of block b }.
+// The K operands of M(b+1) are read from LDS in the middle of V(b), the V^T
+// operands of M(b+1) at its own start (they are needed only after the S^T
+// chain).  Here a workgroup has eight waves,
 // two a SIMD; every phase ends with a workgroup barrier and the wave of a SIMD
 // that arrives second runs one phase behind the first, so that on every SIMD
 // one wave is in its matrix phase while the other is in its vector phase, and
@@ -409,9 +411,11 @@ flash_forward_kernel(FlashForwardArgs a_in, int unit_count) {
 // loop bounds are the workgroup's, only the work inside a phase is conditional.
 //
 // K/V tiles (64 keys = two blocks) rotate through three LDS stages.  Tile t is
-// read in V(2t-1) .. V(2t+1); tile t+3 takes its place and is requested right
-// after the barrier that ends the late waves' V(2t+1); its loads have six
-// phases to land before the barrier that precedes its first read.
+// read from V(2t-1) (K operands of its first block) to M(2t+2) (V^T operands
+// of its second); tile t+3 takes its place and is requested in M(2t+3) by
+// either kind of wave, after the barrier that ends the late waves' M(2t+2);
+// its first read is in V(2t+5), and the barrier before that phase is passed
+// only by waves whose own loads of the tile have landed.
 template <int D>
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 flash_forward_pingpong_kernel(FlashForwardArgs a_in, int unit_count) {
@@ -679,14 +683,12 @@ flash_forward_pingpong_kernel(FlashForwardArgs a_in, int unit_count) {
 
     // stage offsets of tiles t, t + 1, t + 2
     int cur = 0, nxt = kStageBytes, third = 2 * kStageBytes;
-    // One tile: V(2t), M(2t+1), V(2t+1), M(2t+2).  A matrix phase starts with
-    // the LDS reads of its own operands (the vector phase is the longer one and
-    // the matrix phase has issue slots to spare).  `conditional`: blocks may be
-    // masked or invisible to this wave (the diagonal tiles).
-    //   tile t is read in M(2t) .. M(2t+2); tile t+3 takes its place and is
-    //   requested in M(2t+3) by either kind of wave; its first read is in
-    //   M(2t+6), and the barrier before that phase is passed only by waves
-    //   whose own loads of the tile have landed.
+    // One tile: V(2t), M(2t+1), V(2t+1), M(2t+2).  `conditional`: blocks may be
+    // masked or invisible to this wave (the diagonal tiles).  Tile t+1 is first
+    // read in V(2t+1); the barrier before it ends the early waves' M(2t+1) and
+    // the late waves' V(2t), which is where each kind waits for its own loads
+    // of that tile.  Tile t+2 is requested in M(2t+1), into the stage tile t-1
+    // left with the late waves' M(2t).
     auto one_tile = [&](int t, bool conditional) {
       const bool m0 = !conditional || matters(2 * t);
       const bool m1 = !conditional || matters(2 * t + 1);
