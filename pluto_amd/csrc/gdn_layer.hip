@@ -109,8 +109,7 @@ output_kernel(const void* core, int core_dtype, const void* z, int z_dtype,
 // DeltaOutputKernel (cached_attention_ops.cc:205-272) with the gate
 // arithmetic of sequence_delta_net.cc:88-96 in one launch.  The state is read
 // and written exactly once, every load is issued before anything is waited
-// for: thread (half, column) = (tid / 128, tid % 128) owns rows 64 half ..
-// 64 half + 63 of its column.
+// for.
 struct StepArgs {
   const float* convolved = nullptr;  // [batch, channels] q | k | v after conv + SiLU
   const void* z = nullptr;           // [batch, vh * vd], fp32 or bf16 (template argument)
@@ -126,26 +125,34 @@ struct StepArgs {
   bool round = true;
 };
 
+// Threads per workgroup of step_kernel: thread (part, column) = (tid / 128,
+// tid % 128) owns rows 16 part .. 16 part + 15 of its column.  With 64 rows a
+// thread the kernel needed 272 registers, which left a compute unit four waves
+// that loaded, computed and stored in turn (60 us for 32 x 48 heads); sixteen
+// waves of 97 registers take 49 us.
+constexpr int kStepThreads = 1024;
+constexpr int kStepParts = kStepThreads / 128, kStepRows = 128 / kStepParts;
+
 template <int IO>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(kStepThreads)
 step_kernel(StepArgs a) {
   __shared__ float ks[128], qs[128];
-  __shared__ float halves[2][128];
+  __shared__ float partial[kStepParts][128];
   __shared__ float squares[2];
   const int bh = blockIdx.x, seq = bh / a.vh, head = bh % a.vh;
   const int key_head = head / (a.vh / a.kh);
   const int kd = a.kd, vd = a.vd;
-  const int tid = threadIdx.x, column = tid % 128, half = tid / 128;
+  const int tid = threadIdx.x, column = tid % 128, part = tid / 128;
   const int channels = 2 * a.kh * kd + a.vh * vd;
   const float* token = a.convolved + static_cast<size_t>(seq) * channels;
   float* state = a.state + static_cast<size_t>(bh) * kd * vd;
   const bool active = column < vd;
   const int column_read = active ? column : vd - 1;
   // the state slice: rows beyond the key width read the last row and count as zero
-  float s[64];
+  float s[kStepRows];
 #pragma unroll
-  for (int r = 0; r < 64; ++r) {
-    const int row = 64 * half + r;
+  for (int r = 0; r < kStepRows; ++r) {
+    const int row = kStepRows * part + r;
     const float value = state[min(row, kd - 1) * vd + column_read];
     s[r] = (row < kd && active) ? value : 0.0f;
   }
@@ -166,44 +173,62 @@ step_kernel(StepArgs a) {
   const float decay = __expf(-expf(a.a_log[head]) * softplus);
   const float beta = maybe_round(1.0f / (1.0f + expf(-load_element(a.b, scalar, IO))), a.round);
   __syncthreads();
-  // 1e-6 inside the root: cached_attention_ops.cc:224-228
-  float kk = 1e-6f, qq = 1e-6f;
-  for (int d = 0; d < 128; ++d) {
-    kk += ks[d] * ks[d];
-    qq += qs[d] * qs[d];
+  // the normalised key and the normalised, scaled query replace the raw ones
+  // in LDS (1e-6 inside the root: cached_attention_ops.cc:224-228)
+  float k_scaled = 0.0f, q_scaled = 0.0f;
+  if (tid < 128) {
+    float kk = 1e-6f, qq = 1e-6f;
+    for (int d = 0; d < 128; ++d) {
+      kk += ks[d] * ks[d];
+      qq += qs[d] * qs[d];
+    }
+    k_scaled = ks[tid] * rsqrtf(kk);
+    q_scaled = qs[tid] * (rsqrtf(qq) / sqrtf(static_cast<float>(kd)));
   }
-  const float k_factor = rsqrtf(kk);
-  const float q_factor = rsqrtf(qq) / sqrtf(static_cast<float>(kd));
+  __syncthreads();
+  if (tid < 128) {
+    ks[tid] = k_scaled;
+    qs[tid] = q_scaled;
+  }
+  __syncthreads();
   float prediction = 0.0f;
 #pragma unroll
-  for (int r = 0; r < 64; ++r) {
+  for (int r = 0; r < kStepRows; ++r) {
     s[r] *= decay;
-    prediction += s[r] * (ks[64 * half + r] * k_factor);
+    prediction += s[r] * ks[kStepRows * part + r];
   }
-  halves[half][column] = prediction;
+  partial[part][column] = prediction;
   __syncthreads();
-  const float delta = (value - (halves[0][column] + halves[1][column])) * beta;
+  float predicted = partial[0][column];
+#pragma unroll
+  for (int i = 1; i < kStepParts; ++i) predicted += partial[i][column];
+  const float delta = (value - predicted) * beta;
   __syncthreads();
   float output = 0.0f;
 #pragma unroll
-  for (int r = 0; r < 64; ++r) {
-    s[r] += (ks[64 * half + r] * k_factor) * delta;
-    output += s[r] * (qs[64 * half + r] * q_factor);
+  for (int r = 0; r < kStepRows; ++r) {
+    s[r] += ks[kStepRows * part + r] * delta;
+    output += s[r] * qs[kStepRows * part + r];
   }
 #pragma unroll
-  for (int r = 0; r < 64; ++r) {
-    const int row = 64 * half + r;
+  for (int r = 0; r < kStepRows; ++r) {
+    const int row = kStepRows * part + r;
     if (row < kd && active) state[row * vd + column] = s[r];
   }
-  halves[half][column] = output;
+  partial[part][column] = output;
   __syncthreads();
   // RMSNorm over the head's columns, then the SiLU(z) gate
   float core = 0.0f;
-  if (half == 0 && active) core = maybe_round(halves[0][column] + halves[1][column], a.round);
+  if (part == 0 && active) {
+    core = partial[0][column];
+#pragma unroll
+    for (int i = 1; i < kStepParts; ++i) core += partial[i][column];
+    core = maybe_round(core, a.round);
+  }
   const float square = wave_sum(core * core);
-  if (half == 0 && tid % 64 == 0) squares[tid / 64] = square;
+  if (part == 0 && tid % 64 == 0) squares[tid / 64] = square;
   __syncthreads();
-  if (half != 0 || !active) return;
+  if (part != 0 || !active) return;
   const float inverse = rsqrtf((squares[0] + squares[1]) / static_cast<float>(vd) + a.epsilon);
   const float normalized = maybe_round(core * inverse, a.round);
   const float affine = maybe_round(normalized * weight, a.round);
@@ -242,9 +267,9 @@ int launch_gdn_step_fused(hipStream_t stream, const float* convolved, const void
   s.epsilon = epsilon;
   s.round = round;
   if (io_dtype == PLUTO_HIP_BF16)
-    step_kernel<PLUTO_HIP_BF16><<<batch * value_heads, 256, 0, stream>>>(s);
+    step_kernel<PLUTO_HIP_BF16><<<batch * value_heads, kStepThreads, 0, stream>>>(s);
   else
-    step_kernel<PLUTO_HIP_F32><<<batch * value_heads, 256, 0, stream>>>(s);
+    step_kernel<PLUTO_HIP_F32><<<batch * value_heads, kStepThreads, 0, stream>>>(s);
   return launch_status();
 }
 
