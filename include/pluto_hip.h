@@ -44,7 +44,15 @@ extern "C" {
 const char* pluto_hip_error_name(int code);
 const char* pluto_hip_error_string(int code);
 
-/* Library/ABI version and the gfx target the kernels were compiled for. */
+/* Library/ABI version and the gfx target the kernels were compiled for.  The
+ * version changes whenever an existing signature, struct or workspace layout
+ * changes; a caller compares pluto_hip_abi_version() with the
+ * PLUTO_HIP_ABI_VERSION of the header it was built against.
+ *   2: pluto_hip_gdn_step_batch takes io_dtype and void* activations; the
+ *      decode workspace starts with the arrival counters;
+ *      pluto_hip_dense_imported_workspace_bytes grew.
+ *   3: pluto_hip_gqa_decode_static_reset added. */
+#define PLUTO_HIP_ABI_VERSION 3
 int pluto_hip_abi_version(void);
 const char* pluto_hip_target_arch(void);
 
@@ -297,10 +305,19 @@ int pluto_hip_gqa_decode(void* stream, const pluto_hip_attention_params* p,
  * 13 MiB.  All calls on one GPU share the array: calls that overlap there, on
  * whatever streams, race on it.  pluto_hip_gqa_decode_static_prepare looks
  * the array's device address up for the calling thread's current device (the
- * entry point does it itself on its first call there). */
+ * entry point does it itself on its first call there).
+ * The array starts with the split-K arrival counters; every call that runs to
+ * its end leaves them zero, which the next call relies on.  A call that
+ * returns an error after queueing work marks the device, and the next call
+ * there clears the counters first.  After anything else that may have left
+ * them non-zero (calls that overlapped on one GPU, a kernel that was aborted)
+ * queue pluto_hip_gqa_decode_static_reset(stream): one small fill kernel (no
+ * memset node, so it may be recorded into a graph) that zeroes them all;
+ * later calls on that stream then start clean. */
 #define PLUTO_HIP_GQA_DECODE_STATIC_BYTES (16u << 20)
 size_t pluto_hip_gqa_decode_static_bytes(void);
 int pluto_hip_gqa_decode_static_prepare(void);
+int pluto_hip_gqa_decode_static_reset(void* stream);
 int pluto_hip_gqa_decode_static(void* stream, const pluto_hip_attention_params* p,
                                 int batch, int io_dtype, const void* q_gate,
                                 const void* k, const void* v, const float* q_norm,
@@ -516,11 +533,12 @@ int pluto_hip_dense_imported_forward_batch(void* stream, int storage,
  * Test support.  No counterpart in the reference.
  * --------------------------------------------------------------------- */
 
-/* Routes every later call of this library, on any thread, through the
- * any-shape FP32-arithmetic kernels (enabled != 0) or back to normal kernel
- * selection (0), so that tests can compare the two implementations on the
- * device.  Returns the previous setting.  This switch is the only
- * process-wide state of the library; nothing else writes it. */
+/* Routes the later calls of the CALLING THREAD through the any-shape
+ * FP32-arithmetic kernels (enabled != 0) or back to normal kernel selection
+ * (0), so that tests can compare the two implementations on the device.
+ * Returns the thread's previous setting.  Thread-local, like the two hooks
+ * below: a thread that never calls them always gets normal kernel selection,
+ * and the library keeps no process-wide switches. */
 int pluto_hip_test_force_generic(int enabled);
 
 /* Measurement hook: entry points that queue several kernels skip those whose
@@ -531,7 +549,7 @@ int pluto_hip_test_force_generic(int enabled);
  * attention forward at head width 128 keeps to its four-wave kernel whatever
  * the sequence length, which lets a test compare its two kernels).  A benchmark
  * runs the whole call once, then times one class with events around the call.  Returns the previous mask;
- * the default, ~0u, runs everything.  Process-wide like the switch above, and
+ * the default, ~0u, runs everything.  Thread-local like the switch above, and
  * like it written by nothing on the product path. */
 unsigned pluto_hip_test_kernel_classes(unsigned mask);
 

@@ -112,6 +112,7 @@ SIGNATURES = {
                                   ctypes.POINTER(_VP), _I, _VP, _SZ]),
     "pluto_hip_gqa_decode_static_bytes": (_SZ, []),
     "pluto_hip_gqa_decode_static_prepare": (_I, []),
+    "pluto_hip_gqa_decode_static_reset": (_I, [_VP]),
     "pluto_hip_gqa_decode_static": (_I, [_VP, ctypes.POINTER(AttentionParams), _I, _I, _VP,
                                          _VP, _VP, _VP, _VP, ctypes.POINTER(_I),
                                          ctypes.POINTER(KvCacheView), _VP,

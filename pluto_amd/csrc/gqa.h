@@ -98,7 +98,8 @@ int launch_decode_fast(hipStream_t stream, const DecodeArgs& args,
                        const DecodeBatch& batch);
 // Zeroes `count` arrival counters (a launch of its own: the fused kernel needs
 // them zero, and leaves them zero).
-int launch_decode_clear(hipStream_t stream, unsigned* arrivals, int count);
+// `always`: also when the test-support kernel mask has switched auxiliary kernels off
+int launch_decode_clear(hipStream_t stream, unsigned* arrivals, int count, bool always = false);
 // Two-pass probability rows (any dtype, any shape): row r of `rows` sees the
 // first `first_visible + r` cache rows; output fp32 [query_heads, rows,
 // row_width], zero beyond the visible prefix

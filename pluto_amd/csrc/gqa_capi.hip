@@ -24,10 +24,14 @@ namespace {
 constexpr int kMaxDevices = 64;
 std::atomic<void*> static_scratch_address[kMaxDevices];
 std::mutex static_scratch_mutex;
+// Set when a call on the fixed scratch returned an error after it had queued
+// work: its kernels may leave arrival counters behind that are not zero, so
+// the next call on that device clears them first.
+std::atomic<bool> static_scratch_dirty[kMaxDevices];
 
 // Device address of `scratch` on the calling thread's current device, looked
 // up once per device.
-int static_scratch(void** address) {
+int static_scratch(void** address, int* device_out = nullptr) {
   int device = 0;
   hipError_t error = hipGetDevice(&device);
   if (error != hipSuccess) return static_cast<int>(error);
@@ -44,6 +48,7 @@ int static_scratch(void** address) {
     }
   }
   *address = known;
+  if (device_out) *device_out = device;
   return 0;
 }
 
@@ -497,7 +502,8 @@ static int decode_check(const pluto_hip_attention_params* p, int batch, int io_d
 }
 
 // The fixed scratch starts with room for this many arrival counters; they are
-// zero when the library is loaded and every call leaves them zero.
+// zero when the library is loaded and every call that runs to its end leaves
+// them zero.  pluto_hip_gqa_decode_static_reset re-zeroes them.
 constexpr size_t kStaticArrivalBytes = 16384;
 
 static int decode_run(void* stream, const pluto_hip_attention_params* p, int batch, int io_dtype,
@@ -548,12 +554,39 @@ int pluto_hip_gqa_decode_static(void* stream, const pluto_hip_attention_params* 
       decode_layout(p, batch, decode_blocks(batch, positions, split), kStaticArrivalBytes);
   if (layout.total > kStaticScratchBytes) return PLUTO_HIP_ELIMIT;
   void* address = nullptr;
-  status = static_scratch(&address);
+  int device = 0;
+  status = static_scratch(&address, &device);
   if (status != 0) return status;
   // The counters at the head of the array are zero since the library was
-  // loaded and every call leaves them zero: nothing to clear, one launch.
-  return decode_run(stream, p, batch, io_dtype, q_gate, k, v, q_norm, k_norm, positions, caches,
-                    out, probabilities, split, address, layout, false);
+  // loaded and every call that ran to its end left them zero: nothing to
+  // clear, one launch.  A call that failed after it had queued work may have
+  // left some behind; the first call after it clears them all.
+  if (static_scratch_dirty[device].exchange(false, std::memory_order_acq_rel)) {
+    status = launch_decode_clear(static_cast<hipStream_t>(stream),
+                                 static_cast<unsigned*>(address),
+                                 static_cast<int>(kStaticArrivalBytes / sizeof(unsigned)), true);
+    if (status != 0) {
+      static_scratch_dirty[device].store(true, std::memory_order_release);
+      return status;
+    }
+  }
+  status = decode_run(stream, p, batch, io_dtype, q_gate, k, v, q_norm, k_norm, positions, caches,
+                      out, probabilities, split, address, layout, false);
+  if (status != 0) static_scratch_dirty[device].store(true, std::memory_order_release);
+  return status;
+}
+
+int pluto_hip_gqa_decode_static_reset(void* stream) {
+  void* address = nullptr;
+  int device = 0;
+  const int status = static_scratch(&address, &device);
+  if (status != 0) return status;
+  // a fill kernel, not a memset: callers may record this into a graph
+  const int cleared = launch_decode_clear(
+      static_cast<hipStream_t>(stream), static_cast<unsigned*>(address),
+      static_cast<int>(kStaticArrivalBytes / sizeof(unsigned)), true);
+  if (cleared == 0) static_scratch_dirty[device].store(false, std::memory_order_release);
+  return cleared;
 }
 
 static int decode_run(void* stream, const pluto_hip_attention_params* p, int batch, int io_dtype,

@@ -21,9 +21,11 @@
 //           loaded straight from global memory, 16 bytes per lane, the four
 //           lanes of a token together one 64-byte sector per load;
 //           the group's heads are the (zero padded) 16 columns.
-//   values  O[head, :] += p[head, token] * V[token, :] on the vector ALU: 16
-//           bytes of V per lane, probabilities broadcast from LDS.  The kernel
-//           is bound by HBM, not by this arithmetic.
+//   values  O[head, :] += p[head, token] * V[token, :] on
+//           v_mfma_f32_16x16x16_bf16: V rows stream through 16-row LDS stages
+//           (buffer loads that write LDS directly), the probabilities enter as
+//           the sum of two bf16 numbers (hi + lo), which keeps the product to
+//           FP32 accuracy.  The kernel is bound by HBM, not by this arithmetic.
 //   combine Partial (o, m, l) triples are written per block.  Workgroups count
 //           their arrivals per (sequence, kv head); the one that arrives last
 //           combines that pair's blocks in ascending order (a fixed order,
@@ -683,8 +685,8 @@ int launch_decode_fast(hipStream_t stream, const DecodeArgs& a, const DecodeBatc
   }
 }
 
-int launch_decode_clear(hipStream_t stream, unsigned* arrivals, int count) {
-  if (!kernel_enabled(kAuxiliaryKernel)) return 0;
+int launch_decode_clear(hipStream_t stream, unsigned* arrivals, int count, bool always) {
+  if (!always && !kernel_enabled(kAuxiliaryKernel)) return 0;
   decode_clear_kernel<<<(count + 255) / 256, 256, 0, stream>>>(arrivals, count);
   return launch_status();
 }

@@ -1,7 +1,6 @@
 // C ABI of GPT-2 style causal multi-head attention: validation and kernel
 // selection.  The layer-level contract is that of AttentionLayer
 // (src/llm/layers/attention.cc:400-596).
-#include <atomic>
 #include <cmath>
 
 #include "attn_generic.h"
@@ -10,25 +9,21 @@
 
 namespace pluto_hip {
 
-// Test hook (pluto_hip_test_force_generic): routes everything through the
-// any-shape FP32-arithmetic kernels so the two implementations can be checked
-// against each other on the device.  The one process-wide switch of the
-// library; nothing on the product path writes it.
+// Test hooks.  pluto_hip_test_force_generic routes the calling thread's later
+// calls through the any-shape FP32-arithmetic kernels so that the two
+// implementations can be checked against each other on the device;
+// pluto_hip_test_kernel_classes masks kernel classes for measurements.  Both
+// are per thread: a thread that never calls them (every product caller) always
+// gets normal kernel selection, whatever a test thread of the same process has
+// set.  The library has no process-wide switches.
 namespace {
-std::atomic<int> force_generic_flag{0};
-}
-bool force_generic() { return force_generic_flag.load(std::memory_order_relaxed) != 0; }
-
-namespace {
-std::atomic<unsigned> kernel_class_mask{~0u};
-}
-namespace {
+thread_local int force_generic_flag = 0;
+thread_local unsigned kernel_class_mask = ~0u;
 thread_local int last_path = PLUTO_HIP_PATH_NONE;
-}
+}  // namespace
+bool force_generic() { return force_generic_flag != 0; }
 void note_path(int path) { last_path = path; }
-bool kernel_enabled(KernelClass which) {
-  return (kernel_class_mask.load(std::memory_order_relaxed) & which) != 0;
-}
+bool kernel_enabled(KernelClass which) { return (kernel_class_mask & which) != 0; }
 
 namespace {
 
@@ -80,10 +75,16 @@ using namespace pluto_hip;
 extern "C" {
 
 int pluto_hip_test_force_generic(int enabled) {
-  return force_generic_flag.exchange(enabled != 0 ? 1 : 0);
+  const int before = force_generic_flag;
+  force_generic_flag = enabled != 0 ? 1 : 0;
+  return before;
 }
 
-unsigned pluto_hip_test_kernel_classes(unsigned mask) { return kernel_class_mask.exchange(mask); }
+unsigned pluto_hip_test_kernel_classes(unsigned mask) {
+  const unsigned before = kernel_class_mask;
+  kernel_class_mask = mask;
+  return before;
+}
 
 int pluto_hip_test_last_path(void) { return last_path; }
 

@@ -63,7 +63,7 @@ const char* pluto_hip_error_string(int code) {
   return "unknown error code";
 }
 
-int pluto_hip_abi_version(void) { return 1; }
+int pluto_hip_abi_version(void) { return PLUTO_HIP_ABI_VERSION; }
 const char* pluto_hip_target_arch(void) { return "gfx950"; }
 
 int pluto_hip_executor_create(pluto_hip_executor** out) {

@@ -49,7 +49,7 @@ def test_binding_table_matches_header(library):
     from pluto_amd import capi
     assert sorted(capi.SIGNATURES) == declared_symbols()
     handle = capi.lib()   # loads the library and binds every signature
-    assert handle.pluto_hip_abi_version() == 1
+    assert handle.pluto_hip_abi_version() == 3
     assert handle.pluto_hip_target_arch() == b"gfx950"
     assert handle.pluto_hip_error_name(0) == b"PLUTO_HIP_OK"
     assert handle.pluto_hip_error_name(-1) == b"PLUTO_HIP_EINVAL"

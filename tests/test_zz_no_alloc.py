@@ -86,6 +86,59 @@ def test_two_calls_in_a_row_second_one_smaller(capi):
     run_both(capi, p, make_case(capi, 13, batch, qh, kh, d, capacity, lengths), lengths, 512)
 
 
+def test_reset_then_another_call(capi):
+    """pluto_hip_gqa_decode_static_reset between two calls: the second call starts
+    from cleared arrival counters and still matches the workspace entry point."""
+    handle = capi.lib()
+    batch, qh, kh, d, capacity = 7, 24, 4, 128, 8192
+    p = capi.attention_params(qh, kh, d, 32, capacity=capacity)
+    lengths = np.array([1, 513, 4097, 8192, 700, 1024, 2048])
+    run_both(capi, p, make_case(capi, 21, batch, qh, kh, d, capacity, lengths), lengths, 512)
+    assert handle.pluto_hip_gqa_decode_static_reset(capi.current_stream()) == 0
+    lengths = np.array([8192, 5, 1025, 64, 3000, 512, 6000])
+    run_both(capi, p, make_case(capi, 22, batch, qh, kh, d, capacity, lengths), lengths, 256)
+    # a reset with nothing before it on the stream changes nothing either
+    assert handle.pluto_hip_gqa_decode_static_reset(capi.current_stream()) == 0
+    assert handle.pluto_hip_gqa_decode_static_reset(capi.current_stream()) == 0
+    run_both(capi, p, make_case(capi, 23, batch, qh, kh, d, capacity, lengths), lengths, 512)
+
+
+def test_recorded_into_a_graph(capi):
+    """The stated use of the entry point: {reset, decode on the fixed scratch}
+    recorded into a HIP graph; every replay, with eager calls of the same entry
+    point and synchronizations in between, leaves what the workspace entry
+    point leaves."""
+    handle = capi.lib()
+    batch, qh, kh, d, capacity = 5, 12, 2, 128, 4096
+    p = capi.attention_params(qh, kh, d, 32, capacity=capacity)
+    lengths = [700, 4096, 33, 1500, 2049]
+    positions = [L - 1 for L in lengths]
+    caches, q_gate, k, v, qw, kw = make_case(capi, 31, batch, qh, kh, d, capacity, lengths)
+    want = capi.gqa_decode(p, q_gate, k, v, qw, kw, caches(), positions=positions, advance=False)
+    fixed = caches()
+    out = torch.empty_like(want)
+
+    def step():
+        assert handle.pluto_hip_gqa_decode_static_reset(capi.current_stream()) == 0
+        capi.gqa_decode_static(p, q_gate, k, v, qw, kw, fixed, positions, out)
+
+    step()
+    torch.cuda.synchronize()
+    assert torch.equal(out, want)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for replay in range(4):
+        out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), "replay %d" % replay
+        step()   # eager work on the same scratch between the replays
+        torch.cuda.synchronize()
+        assert torch.equal(out, want)
+
+
 def test_rejects_what_does_not_fit(capi):
     handle = capi.lib()
     batch, qh, kh, d, capacity = 64, 24, 4, 128, 32768
