@@ -70,6 +70,11 @@ def build_device(force=False, verbose=True):
     headers = glob.glob(os.path.join(CSRC, "*.h")) + glob.glob(
         os.path.join(ROOT, "include", "*.h"))
     sources = sorted(glob.glob(os.path.join(CSRC, "*.hip")))
+    # the hand-scheduled instruction streams are generated text
+    generators = sorted(glob.glob(os.path.join(CSRC, "gen_*.py")))
+    for generator in generators:
+        _run([sys.executable, generator])
+    headers += glob.glob(os.path.join(CSRC, "*.inc")) + generators
     if force or not _newer(LIB, sources + headers):
         with concurrent.futures.ThreadPoolExecutor(max_workers=8) as pool:
             objects = list(pool.map(lambda s: _compile(s, DEVICE_FLAGS), sources))

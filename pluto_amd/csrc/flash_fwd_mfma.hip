@@ -29,6 +29,8 @@
 
 #include "mfma_tile.h"
 
+#include <algorithm>
+
 namespace pluto_hip {
 namespace {
 
@@ -839,6 +841,10 @@ int launch_flash_forward(hipStream_t stream, const FlashForwardArgs& a,
   // Long sequences at D = 128 take the eight-wave ping-pong kernel (3-4 %
   // faster at 8192 rows); its 256-row tiles waste waves on short ones.
   if (head_dim == 128 && a.q_rows >= kPingPongFromRows && kernel_enabled(kPingPong)) {
+    // its epilogue addresses a head's rows through 32-bit buffer offsets
+    const long long widest = a.gate ? std::max(a.o_row_stride, a.gate_row_stride) : a.o_row_stride;
+    if (kernel_enabled(kPipelined) && a.q_rows * widest * 2 < (1LL << 31) - 4096)
+      return launch_flash_forward_pipelined(stream, a, sequences);
     const long long pp_tiles = (a.q_rows + 255) / 256;
     const long long pp_units = pp_tiles * sequences * (a.query_heads / a.group);
     const long long pp_blocks = (pp_units + 7) / 8 * 8 * a.group;

@@ -1,0 +1,574 @@
+// Causal flash attention forward for long bf16 sequences on gfx950: the
+// kernel whose main loop is a hand-scheduled instruction stream.
+//
+// Same mathematics, operand layouts and results as flash_forward_kernel
+// (flash_fwd_mfma.hip; semantics of FlashAttentionForwardKernel,
+// src/llm/layers/attention.cc:98-170, and with the gate epilogue of
+// ForwardKernel, src/llm/layers/qwen_attention.cc:68-119).  What differs is who
+// orders the instructions.  A workgroup of eight waves owns 256 query rows,
+// 32 a wave.  The key tiles every one of those rows sees whole (all but the
+// last 256 keys of the causal range) are processed by ONE asm statement,
+// flash_fwd_loop.inc, written by gen_flash_fwd_loop.py: per 32-key block a
+// wave issues the S^T products of the next block, the softmax arithmetic of
+// the current one and the O^T products of the previous one interleaved
+// instruction by instruction, with its own LDS reads and waits, on fixed
+// registers.  The tiles that cross the diagonal (masks, waves with nothing
+// left to do) run the plain loop below, in C++.
+#include "flash_fwd_mfma.h"
+#include "flash_fwd_loop.inc"
+#ifndef TL
+#define TL(slot) do {} while (0)
+#endif
+#include "mfma_tile.h"
+
+#include <algorithm>
+#include <vector>
+
+namespace pluto_hip {
+namespace {
+
+constexpr int BN = 64;
+constexpr int kRows = 256;  // query rows a workgroup processes at a time
+
+// Which query tiles a workgroup processes.  The causal mask makes tiles
+// unequal (tile t costs about t + 1 units plus a fixed part) and a long
+// sequence yields only a few tiles per compute unit, so handing tiles out in
+// launch order leaves compute units idle at the end (measured at 8192 rows, 24
+// heads: 12 % of the kernel).  Instead the launcher packs the tiles into one
+// list per workgroup, equal in cost, and launches one workgroup a compute
+// unit; the lists travel in the kernel arguments.  slots == 0: no lists,
+// workgroup i processes the single tile the XCD-aware numbering gives it.
+constexpr int kScheduleEntries = 1536;
+constexpr uint16_t kNoItem = 0xffff;
+struct Schedule {
+  int slots = 0;  // entries per workgroup; its list ends at kNoItem or after `slots`
+  uint16_t item[kScheduleEntries];  // (sequence * heads + head) * q_tiles + q_tile
+};
+
+template <int D>
+__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
+flash_forward_pipelined_kernel(FlashForwardArgs a_in, int unit_count, Schedule schedule) {
+  struct Args : FlashForwardArgs {
+    int unit_count;
+  } a;
+  static_cast<FlashForwardArgs&>(a) = a_in;
+  a.unit_count = unit_count;
+  constexpr int WAVES = 8, KCH = D / 8, KS = D / 16, DB = D / 32;
+  constexpr int BM = 32 * WAVES;
+  constexpr int kTileBytes = BN * D * 2, kStageBytes = 2 * kTileBytes, kStages = 4;
+  constexpr int kLoads = BN * KCH / (64 * WAVES);
+  constexpr int kHalfTile = 32 * KCH * 16;
+  static_assert(D == 128, "the loop text is instantiated for this head width");
+  static_assert(kLoads == FLASH_LOOP_D128_LOADS && kStageBytes == FLASH_LOOP_D128_STAGE_BYTES);
+  __shared__ __attribute__((aligned(1024))) unsigned char lds[kStages * kStageBytes];
+
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / 64), lane = tid % 64;
+  const int h = lane / 32, n = lane % 32;
+  const int q_tiles = (a.q_rows + BM - 1) / BM;
+  const int list_length = schedule.slots > 0 ? schedule.slots : 1;
+  for (int entry = 0; entry < list_length; ++entry) {
+  int q_tile, head, seq;
+  if (schedule.slots > 0) {
+    const int item = schedule.item[blockIdx.x * schedule.slots + entry];
+    if (item == kNoItem) break;
+    q_tile = item % q_tiles;
+    const int column = item / q_tiles;
+    head = column % a.query_heads;
+    seq = column / a.query_heads;
+  } else {
+    // The query heads of a kv head at one query tile run on one XCD (workgroup
+    // i lands on XCD i mod 8, each with a private L2), heaviest tiles first.
+    const int kv_heads = a.query_heads / a.group;
+    const int kv_units = a.unit_count / q_tiles;
+    const int xcd = blockIdx.x % 8, slot = blockIdx.x / 8;
+    const int u = 8 * (slot / a.group) + xcd;
+    if (u >= a.unit_count) return;  // the whole workgroup
+    q_tile = q_tiles - 1 - u / kv_units;
+    const int kv_unit = u % kv_units;
+    head = (kv_unit % kv_heads) * a.group + slot % a.group;
+    seq = kv_unit / kv_heads;
+  }
+  TL(0);
+  const int kv_head = head / a.group;
+  const uint16_t* q_base = a.q + seq * a.q_seq_stride + head * a.q_head_stride;
+  const uint16_t* k_base = a.k + seq * a.k_seq_stride + kv_head * a.k_head_stride;
+  const uint16_t* v_base = a.v + seq * a.v_seq_stride + kv_head * a.v_head_stride;
+  const float scale2 = a.scale * kLog2e;
+  // the loop statement takes the factor as a scalar operand
+  const uint32_t scale2_bits = __builtin_amdgcn_readfirstlane(__float_as_uint(scale2));
+  bf16x8 ones;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) ones[e] = static_cast<__bf16>(1.0f);
+
+  // lane addresses: the tile layouts of flash_forward_kernel
+  uint32_t k_fill[kLoads], v_fill[kLoads];
+#pragma unroll
+  for (int i = 0; i < kLoads; ++i) {
+    const int p = (wave * kLoads + i) * 64 + lane;
+    const int row = p / KCH, slot = p % KCH;
+    k_fill[i] = static_cast<uint32_t>(row * a.k_row_stride * 2 + (slot ^ (row & 7)) * 16);
+    v_fill[i] = static_cast<uint32_t>(row * a.v_row_stride * 2 + (slot ^ (2 * (row & 3))) * 16);
+  }
+  int k_read[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) k_read[ks] = (n * KCH + ((2 * ks + h) ^ (n & 7))) * 16;
+  int v_read[DB];
+  {
+    const int gq = lane / 16, kk = (lane % 16) / 4, b = lane % 4;
+    const int row = 4 * (gq / 2) + kk;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      const int chunk = 4 * db + 2 * (gq % 2) + b / 2;
+      v_read[db] = (row * KCH + (chunk ^ (2 * kk))) * 16 + (b % 2) * 8;
+    }
+  }
+
+  const int q0 = q_tile * BM;
+  const int wave_q0 = q0 + 32 * wave;
+  const int q_row = wave_q0 + n;
+  bf16x8 qf[KS];
+  {
+    const int row = min(q_row, a.q_rows - 1);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      qf[ks] = as_bf16x8(*reinterpret_cast<const uint4*>(
+          q_base + static_cast<long long>(row) * a.q_row_stride + 16 * ks + 8 * h));
+  }
+  const int row_limit = min(a.start_position + q_row, a.kv_rows - 1);
+  floatx16 o_acc[DB], l_acc;
+  constexpr float kLazy = 8.0f;
+  float m_used = kMasked, m_true = kMasked;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) l_acc[i] = 0.0f;
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) o_acc[db][i] = 0.0f;
+
+  // workgroup-uniform loop bounds
+  const int last_row = min(q0 + BM, a.q_rows) - 1;
+  const int visible_keys = min(a.kv_rows, a.start_position + last_row + 1);
+  const int tiles = (visible_keys + BN - 1) / BN;
+  // tiles every row of the workgroup sees whole: no masks, no wave drops out
+  const int whole_tiles = min(tiles, min(a.start_position + q0 + 1, a.kv_rows) / BN);
+  const int32x4 k_all = make_rsrc(
+      k_base, static_cast<uint32_t>(((a.kv_rows - 1) * a.k_row_stride + D) * 2));
+  const int32x4 v_all = make_rsrc(
+      v_base, static_cast<uint32_t>(((a.kv_rows - 1) * a.v_row_stride + D) * 2));
+  const uint32_t lds_address = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_void*)lds));
+
+  TL(1);
+  TL(6);
+  if (whole_tiles > 0) {
+    // ---- the hand-scheduled loop over the whole tiles ------------------------------
+    const uint32_t k_tile_step = static_cast<uint32_t>(BN * a.k_row_stride * 2);
+    const uint32_t v_tile_step = static_cast<uint32_t>(BN * a.v_row_stride * 2);
+    uint32_t steps = static_cast<uint32_t>(whole_tiles - 1), flag = 0, k_offset = 0, v_offset = 0;
+    const uint32_t drain = static_cast<uint32_t>(((whole_tiles - 1) % kStages) * kStageBytes);
+    const uint32_t lds_wave = lds_address + wave * kLoads * 1024;
+    uint32_t saved_m0;
+    float threshold = m_used + kLazy;
+    // the second load of a pair lands 1024 bytes further on in LDS through the
+    // instruction's offset, which also moves its global address: taken out of
+    // the lane's offset again
+    const uint32_t k_second = k_fill[1] - 1024u, v_second = v_fill[1] - 1024u;
+    const int k_read_high[KS] = {k_read[0] + 65536, k_read[1] + 65536, k_read[2] + 65536,
+                                 k_read[3] + 65536, k_read[4] + 65536, k_read[5] + 65536,
+                                 k_read[6] + 65536, k_read[7] + 65536};
+    const int v_read_high[DB] = {v_read[0] + 65536, v_read[1] + 65536, v_read[2] + 65536,
+                                 v_read[3] + 65536};
+    asm volatile(FLASH_LOOP_D128_ASM
+                 : FLASH_LOOP_D128_O0(o_acc[0]), FLASH_LOOP_D128_O1(o_acc[1]),
+                   FLASH_LOOP_D128_O2(o_acc[2]), FLASH_LOOP_D128_O3(o_acc[3]),
+                   FLASH_LOOP_D128_L(l_acc), FLASH_LOOP_D128_MUSED(m_used),
+                   FLASH_LOOP_D128_MTRUE(m_true), FLASH_LOOP_D128_THR(threshold),
+                   [steps] "+s"(steps), [flag] "+s"(flag), [koff] "+s"(k_offset),
+                   [voff] "+s"(v_offset), [m0save] "=&s"(saved_m0)
+                 : FLASH_LOOP_D128_QF0(qf[0]), FLASH_LOOP_D128_QF1(qf[1]),
+                   FLASH_LOOP_D128_QF2(qf[2]), FLASH_LOOP_D128_QF3(qf[3]),
+                   FLASH_LOOP_D128_QF4(qf[4]), FLASH_LOOP_D128_QF5(qf[5]),
+                   FLASH_LOOP_D128_QF6(qf[6]), FLASH_LOOP_D128_QF7(qf[7]),
+                   FLASH_LOOP_D128_ONES(ones),
+                   FLASH_LOOP_D128_KADDR0_0(k_read[0]), FLASH_LOOP_D128_KADDR0_1(k_read[1]),
+                   FLASH_LOOP_D128_KADDR0_2(k_read[2]), FLASH_LOOP_D128_KADDR0_3(k_read[3]),
+                   FLASH_LOOP_D128_KADDR0_4(k_read[4]), FLASH_LOOP_D128_KADDR0_5(k_read[5]),
+                   FLASH_LOOP_D128_KADDR0_6(k_read[6]), FLASH_LOOP_D128_KADDR0_7(k_read[7]),
+                   FLASH_LOOP_D128_KADDR1_0(k_read_high[0]), FLASH_LOOP_D128_KADDR1_1(k_read_high[1]),
+                   FLASH_LOOP_D128_KADDR1_2(k_read_high[2]), FLASH_LOOP_D128_KADDR1_3(k_read_high[3]),
+                   FLASH_LOOP_D128_KADDR1_4(k_read_high[4]), FLASH_LOOP_D128_KADDR1_5(k_read_high[5]),
+                   FLASH_LOOP_D128_KADDR1_6(k_read_high[6]), FLASH_LOOP_D128_KADDR1_7(k_read_high[7]),
+                   FLASH_LOOP_D128_VADDR0_0(v_read[0]), FLASH_LOOP_D128_VADDR0_1(v_read[1]),
+                   FLASH_LOOP_D128_VADDR0_2(v_read[2]), FLASH_LOOP_D128_VADDR0_3(v_read[3]),
+                   FLASH_LOOP_D128_VADDR1_0(v_read_high[0]), FLASH_LOOP_D128_VADDR1_1(v_read_high[1]),
+                   FLASH_LOOP_D128_VADDR1_2(v_read_high[2]), FLASH_LOOP_D128_VADDR1_3(v_read_high[3]),
+                   FLASH_LOOP_D128_KFILL0(k_fill[0]), FLASH_LOOP_D128_KFILL1(k_second),
+                   FLASH_LOOP_D128_VFILL0(v_fill[0]), FLASH_LOOP_D128_VFILL1(v_second),
+                   [krsrc] "s"(k_all), [vrsrc] "s"(v_all), [scale2] "s"(scale2_bits),
+                   [kstep] "s"(k_tile_step), [vstep] "s"(v_tile_step), [ldsw] "s"(lds_wave),
+                   [drain] "s"(drain)
+                 : FLASH_LOOP_D128_CLOBBERS);
+  }
+
+  TL(7);
+  TL(2);
+  // ---- the tiles that cross the diagonal: two LDS stages, one barrier a tile ------------
+  {
+    auto fill = [&](int tile, int stage) {
+      const long long rows_left = a.kv_rows - 1 - static_cast<long long>(tile) * BN;
+      const int32x4 k_rsrc = make_rsrc(
+          k_base + static_cast<long long>(tile) * BN * a.k_row_stride,
+          static_cast<uint32_t>((rows_left * a.k_row_stride + D) * 2));
+      const int32x4 v_rsrc = make_rsrc(
+          v_base + static_cast<long long>(tile) * BN * a.v_row_stride,
+          static_cast<uint32_t>((rows_left * a.v_row_stride + D) * 2));
+#pragma unroll
+      for (int i = 0; i < kLoads; ++i) {
+        const int at = stage * kStageBytes + (wave * kLoads + i) * 1024;
+        lds_fill<16>(k_rsrc, lds + at, k_fill[i]);
+        lds_fill<16>(v_rsrc, lds + kTileBytes + at, v_fill[i]);
+      }
+    };
+    if (whole_tiles < tiles) fill(whole_tiles, 0);
+    for (int tile = whole_tiles; tile < tiles; ++tile) {
+      const int stage = (tile - whole_tiles) & 1;
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+      if (tile + 1 < tiles) fill(tile + 1, stage ^ 1);
+      const unsigned char* k_tile = lds + stage * kStageBytes;
+      const unsigned char* v_tile = k_tile + kTileBytes;
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) {
+        const int kb0 = tile * BN + 32 * kb;
+        // nothing of this block is visible to any of the wave's rows
+        if (kb0 > a.start_position + wave_q0 + 31) continue;
+        bf16x8 kf[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+          kf[ks] = as_bf16x8(
+              *reinterpret_cast<const uint4*>(k_tile + k_read[ks] + kb * kHalfTile));
+        bf16x8 vf[2][DB];
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+          for (int db = 0; db < DB; ++db) {
+            const int at = v_read[db] + kb * kHalfTile + 16 * s2 * KCH * 16;
+            const uint2 lo = lds_transpose_read(v_tile, at);
+            const uint2 hi = lds_transpose_read(v_tile, at + 8 * KCH * 16);
+            vf[s2][db] = __builtin_bit_cast(bf16x8, make_uint4(lo.x, lo.y, hi.x, hi.y));
+          }
+        floatx16 s;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[i] = 0.0f;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) s = mfma32(kf[ks], qf[ks], s);
+        if (kb0 + 31 > a.start_position + wave_q0 || kb0 + 32 > a.kv_rows) {
+          const int limit = row_limit - kb0 - 4 * h;
+#pragma unroll
+          for (int i = 0; i < 16; ++i) s[i] = (8 * (i / 4) + (i % 4) > limit) ? kMasked : s[i];
+        }
+        float row_max = fmaxf(fmaxf(s[0], s[1]), s[2]);
+#pragma unroll
+        for (int i = 3; i < 15; i += 2) row_max = fmaxf(fmaxf(row_max, s[i]), s[i + 1]);
+        row_max = fmaxf(row_max, s[15]);
+        m_true = fmaxf(m_true, half_swap_max(row_max));
+        const float candidate = m_true * scale2;
+        if (__any(candidate > m_used + kLazy)) {
+          const float m_new = candidate > m_used + kLazy ? candidate : m_used;
+          const float alpha = __builtin_amdgcn_exp2f(m_used - m_new);
+          m_used = m_new;
+          l_acc[0] *= alpha;
+#pragma unroll
+          for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) o_acc[db][i] *= alpha;
+        }
+        bf16x8 pf[2];
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+          uint32_t packed[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            packed[e] = pack_bf16(
+                __builtin_amdgcn_exp2f(__builtin_fmaf(s[8 * s2 + 2 * e], scale2, -m_used)),
+                __builtin_amdgcn_exp2f(__builtin_fmaf(s[8 * s2 + 2 * e + 1], scale2, -m_used)));
+          pf[s2] = __builtin_bit_cast(bf16x8, make_uint4(packed[0], packed[1], packed[2], packed[3]));
+        }
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+          l_acc = mfma32(ones, pf[s2], l_acc);
+#pragma unroll
+          for (int db = 0; db < DB; ++db) o_acc[db] = mfma32(vf[s2][db], pf[s2], o_acc[db]);
+        }
+      }
+    }
+  }
+
+  TL(3);
+  // ---- epilogue ------------------------------------------------------------------
+  // The arithmetic of flash_forward_kernel's epilogue.  Every access goes
+  // through a bounds-checked buffer descriptor instead of a branch: rows past
+  // the end (and, for the row statistics, the upper lane halves) get an
+  // offset beyond the descriptor's range, which the hardware drops.  The
+  // kernel thus never narrows exec, and nothing the register allocator spills
+  // around the loop statement above can be saved under a partial mask.
+  {
+    constexpr uint32_t kDropped = 0x7fffffffu;  // beyond every descriptor below
+    const bool in_range = q_row < a.q_rows;
+    const long long row_bytes = static_cast<long long>(a.q_rows - 1) * a.o_row_stride * 2;
+    uint16_t* o_base = a.out + seq * a.o_seq_stride + head * a.o_head_stride;
+    const __amdgpu_buffer_rsrc_t o_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        o_base, 0, static_cast<int>(row_bytes + D * 2), 0x00020000);
+    const __amdgpu_buffer_rsrc_t core_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        a.core ? a.core + (o_base - a.out) : o_base, 0, static_cast<int>(row_bytes + D * 2),
+        0x00020000);
+    const uint16_t* gate_base =
+        a.gate ? a.gate + seq * a.gate_seq_stride + head * a.gate_head_stride : a.q;
+    const __amdgpu_buffer_rsrc_t gate_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t*>(gate_base), 0,
+        static_cast<int>(static_cast<long long>(a.q_rows - 1) * a.gate_row_stride * 2 + D * 2),
+        0x00020000);
+    const uint32_t o_at =
+        in_range ? static_cast<uint32_t>(static_cast<long long>(q_row) * a.o_row_stride * 2)
+                 : kDropped;
+    const uint32_t gate_at =
+        in_range ? static_cast<uint32_t>(static_cast<long long>(q_row) * a.gate_row_stride * 2)
+                 : kDropped;
+    const float l_used = l_acc[0] > 0.0f ? l_acc[0] : 1.0f;
+    const float inverse = 1.0f / l_used;
+    // A lane owns, for its query, channels 32db + 8j + 4h .. +3: four bf16 =
+    // one 8-byte store.
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int d = 32 * db + 8 * j + 4 * h;
+        float c[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) c[e] = o_acc[db][4 * j + e] * inverse;
+        if (a.core) {
+          const uint32x2 plain = {pack_bf16(c[0], c[1]), pack_bf16(c[2], c[3])};
+          __builtin_amdgcn_raw_buffer_store_b64(plain, core_rsrc, o_at + d * 2, 0, 0);
+        }
+        if (a.gate) {
+          // out = bf16(bf16(core) * bf16(sigmoid(gate))): qwen_attention.cc:103-108
+          const uint32x2 gw = __builtin_amdgcn_raw_buffer_load_b64(gate_rsrc, gate_at + d * 2, 0, 0);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float logit =
+                __uint_as_float((e & 1) ? (gw[e / 2] & 0xffff0000u) : (gw[e / 2] << 16));
+            c[e] = round_to_bf16(c[e]) * round_to_bf16(1.0f / (1.0f + expf(-logit)));
+          }
+        }
+        const uint32x2 packed = {pack_bf16(c[0], c[1]), pack_bf16(c[2], c[3])};
+        __builtin_amdgcn_raw_buffer_store_b64(packed, o_rsrc, o_at + d * 2, 0, 0);
+      }
+    // statistics relative to the true maximum (attention.cc:161-168), from the
+    // lower lane half
+    const float normalizer = l_used * __builtin_amdgcn_exp2f(m_used - m_true * scale2);
+    const float maximum = m_true * a.scale;
+    const uint32_t stat_at = in_range && h == 0 ? static_cast<uint32_t>(q_row) * 4u : kDropped;
+    const long long stat = (static_cast<long long>(seq) * a.query_heads + head) * a.q_rows;
+    if (a.maxima)
+      __builtin_amdgcn_raw_buffer_store_b32(
+          __float_as_uint(maximum),
+          __builtin_amdgcn_make_buffer_rsrc(a.maxima + stat, 0, a.q_rows * 4, 0x00020000), stat_at,
+          0, 0);
+    if (a.normalizers)
+      __builtin_amdgcn_raw_buffer_store_b32(
+          __float_as_uint(normalizer),
+          __builtin_amdgcn_make_buffer_rsrc(a.normalizers + stat, 0, a.q_rows * 4, 0x00020000),
+          stat_at, 0, 0);
+    if (a.lse) {
+      float* lse_base = a.lse + static_cast<long long>(seq) * a.q_rows * a.query_heads + head;
+      const long long lse_bytes = (static_cast<long long>(a.q_rows - 1) * a.query_heads + 1) * 4;
+      const uint32_t lse_at =
+          in_range && h == 0 ? static_cast<uint32_t>(static_cast<long long>(q_row) * a.query_heads * 4)
+                             : kDropped;
+      __builtin_amdgcn_raw_buffer_store_b32(
+          __float_as_uint(maximum + __logf(normalizer)),
+          __builtin_amdgcn_make_buffer_rsrc(lse_base, 0, static_cast<int>(lse_bytes), 0x00020000),
+          lse_at, 0, 0);
+    }
+  }
+  TL(4);
+#ifdef PLUTO_TIMELINE
+  {
+    const tl_u32x2 tl_v = {static_cast<unsigned>(whole_tiles), 0u};
+    __builtin_amdgcn_raw_buffer_store_b64(
+        tl_v, __builtin_amdgcn_make_buffer_rsrc(timeline, 0, 4096 * 8 * 8, 0x00020000),
+        threadIdx.x == 0 ? ((blockIdx.x * 4 + entry) * 8 + 5) * 8 : 0x7fffffff, 0, 0);
+  }
+#endif
+  // the next tile's fills must not overtake this tile's last LDS reads
+  __syncthreads();
+  }
+}
+
+}  // namespace
+
+// ---- host side: packing tiles into per-workgroup lists ------------------------------------
+namespace {
+
+struct ScheduleKey {
+  int q_rows = -1, kv_rows = 0, start_position = 0, query_heads = 0, group = 0, sequences = 0,
+      compute_units = 0;
+  bool operator==(const ScheduleKey& o) const {
+    return q_rows == o.q_rows && kv_rows == o.kv_rows && start_position == o.start_position &&
+           query_heads == o.query_heads && group == o.group && sequences == o.sequences &&
+           compute_units == o.compute_units;
+  }
+};
+
+// Cost of a query tile in key tiles: those it walks plus a fixed part (fills
+// in flight before the first product, the masked tiles, the epilogue) that was
+// measured at about ten key tiles' time.
+constexpr int kFixedCost = 10;
+
+int tile_cost(const ScheduleKey& k, int q_tile) {
+  const long long last_row = std::min<long long>((q_tile + 1LL) * kRows, k.q_rows) - 1;
+  const long long visible = std::min<long long>(k.kv_rows, k.start_position + last_row + 1);
+  return static_cast<int>((visible + BN - 1) / BN) + kFixedCost;
+}
+
+// Longest-first greedy packing, then moves and swaps out of the fullest list
+// while they lower it.  Items are indices into `cost`.
+void pack(const std::vector<int>& cost, int lists, std::vector<std::vector<int>>& out) {
+  std::vector<int> order(cost.size());
+  for (size_t i = 0; i < order.size(); ++i) order[i] = static_cast<int>(i);
+  std::stable_sort(order.begin(), order.end(), [&](int x, int y) { return cost[x] > cost[y]; });
+  out.assign(lists, {});
+  std::vector<long long> load(lists, 0);
+  for (int item : order) {
+    int best = 0;
+    for (int b = 1; b < lists; ++b)
+      if (load[b] < load[best]) best = b;
+    out[best].push_back(item);
+    load[best] += cost[item];
+  }
+  for (int round = 0; round < 64; ++round) {
+    int hi = 0;
+    for (int b = 1; b < lists; ++b)
+      if (load[b] > load[hi]) hi = b;
+    long long best_top = load[hi];
+    int best_lo = -1, best_a = -1, best_b = -1;
+    for (int lo = 0; lo < lists; ++lo) {
+      const long long gap = load[hi] - load[lo];
+      if (lo == hi || gap <= 0) continue;
+      for (size_t ia = 0; ia < out[hi].size(); ++ia) {
+        const int wa = cost[out[hi][ia]];
+        if (wa < gap) {
+          const long long top = std::max(load[hi] - wa, load[lo] + wa);
+          if (top < best_top) best_top = top, best_lo = lo, best_a = static_cast<int>(ia), best_b = -1;
+        }
+        for (size_t ib = 0; ib < out[lo].size(); ++ib) {
+          const int delta = wa - cost[out[lo][ib]];
+          if (delta <= 0 || delta >= gap) continue;
+          const long long top = std::max(load[hi] - delta, load[lo] + delta);
+          if (top < best_top)
+            best_top = top, best_lo = lo, best_a = static_cast<int>(ia), best_b = static_cast<int>(ib);
+        }
+      }
+    }
+    if (best_lo < 0) break;
+    const int moved = out[hi][best_a];
+    out[hi].erase(out[hi].begin() + best_a);
+    load[hi] -= cost[moved];
+    if (best_b >= 0) {
+      const int back = out[best_lo][best_b];
+      out[best_lo].erase(out[best_lo].begin() + best_b);
+      load[best_lo] -= cost[back];
+      out[hi].push_back(back);
+      load[hi] += cost[back];
+    }
+    out[best_lo].push_back(moved);
+    load[best_lo] += cost[moved];
+  }
+}
+
+// Fills `schedule` and returns the number of workgroups, or 0 when the launch
+// should number its tiles by workgroup index instead (more tiles than the table
+// holds, fewer tiles than compute units, an unusual device).
+int build_schedule(const ScheduleKey& k, Schedule& schedule) {
+  schedule.slots = 0;
+  const int q_tiles = (k.q_rows + kRows - 1) / kRows;
+  const int kv_heads = k.query_heads / k.group;
+  const int kv_units = k.sequences * kv_heads;
+  const long long items = 1LL * q_tiles * k.sequences * k.query_heads;
+  if (k.compute_units % 8 != 0 || k.compute_units <= 0 || items <= k.compute_units ||
+      items >= kNoItem)
+    return 0;
+  // Workgroup i runs on XCD i mod 8 and every XCD has its own L2: the heads of
+  // a kv head stay on as few XCDs as the unit count allows.  All partitions
+  // hold the same multiset of tiles, so one packing serves them all.
+  int partitions, xcds_each, units_each;
+  if (kv_units % 8 == 0)
+    partitions = 8, xcds_each = 1, units_each = kv_units / 8;
+  else if (8 % kv_units == 0)
+    partitions = kv_units, xcds_each = 8 / kv_units, units_each = 1;
+  else
+    partitions = 1, xcds_each = 8, units_each = kv_units;
+  const int lists = k.compute_units / 8 * xcds_each;
+  std::vector<int> cost;
+  cost.reserve(static_cast<size_t>(units_each) * k.group * q_tiles);
+  for (int local = 0; local < units_each * k.group; ++local)
+    for (int t = 0; t < q_tiles; ++t) cost.push_back(tile_cost(k, t));
+  std::vector<std::vector<int>> packed;
+  pack(cost, lists, packed);
+  size_t slots = 0;
+  for (const auto& list : packed) slots = std::max(slots, list.size());
+  if (slots == 0 || slots * k.compute_units > static_cast<size_t>(kScheduleEntries)) return 0;
+  for (size_t i = 0; i < slots * k.compute_units; ++i) schedule.item[i] = kNoItem;
+  for (int p = 0; p < partitions; ++p)
+    for (int j = 0; j < lists; ++j) {
+      // list j of partition p -> workgroup on XCD x: the partition's XCDs are
+      // p, p + partitions, ...
+      const int xcd = p + partitions * (j % xcds_each);
+      const int workgroup = (j / xcds_each) * 8 + (partitions == 1 ? j % 8 : xcd);
+      std::vector<int> list = packed[j];
+      std::stable_sort(list.begin(), list.end(), [&](int x, int y) { return cost[x] > cost[y]; });
+      for (size_t e = 0; e < list.size(); ++e) {
+        const int local = list[e] / q_tiles, q_tile = list[e] % q_tiles;
+        // local = (unit within the partition) * group + head within the group
+        const int unit = partitions == 1 ? local / k.group
+                                         : (kv_units % 8 == 0 ? p + 8 * (local / k.group) : p);
+        const int sequence = unit / kv_heads, kv_head = unit % kv_heads;
+        const int head = kv_head * k.group + local % k.group;
+        schedule.item[workgroup * slots + e] =
+            static_cast<uint16_t>((sequence * k.query_heads + head) * q_tiles + q_tile);
+      }
+    }
+  schedule.slots = static_cast<int>(slots);
+  return k.compute_units;
+}
+
+}  // namespace
+
+int launch_flash_forward_pipelined(hipStream_t stream, const FlashForwardArgs& a, int sequences) {
+  const long long q_tiles = (a.q_rows + kRows - 1) / kRows;
+  const long long units = q_tiles * sequences * (a.query_heads / a.group);
+  long long blocks = (units + 7) / 8 * 8 * a.group;
+  if (blocks <= 0 || blocks > 0x7fffffffLL) return PLUTO_HIP_EINVAL;
+  // The packing depends on the shape only; a thread keeps the last one it made.
+  thread_local ScheduleKey known;
+  thread_local Schedule schedule;
+  thread_local int scheduled_blocks = 0;
+  ScheduleKey key;
+  key.q_rows = a.q_rows, key.kv_rows = a.kv_rows, key.start_position = a.start_position;
+  key.query_heads = a.query_heads, key.group = a.group, key.sequences = sequences;
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess ||
+      hipDeviceGetAttribute(&key.compute_units, hipDeviceAttributeMultiprocessorCount, device) !=
+          hipSuccess)
+    key.compute_units = 0;
+  if (!(key == known)) {
+    scheduled_blocks = build_schedule(key, schedule);
+    known = key;
+  }
+  if (scheduled_blocks > 0) blocks = scheduled_blocks;
+  flash_forward_pipelined_kernel<128><<<dim3(static_cast<unsigned>(blocks)), 512, 0, stream>>>(
+      a, static_cast<int>(units), schedule);
+  return launch_status();
+}
+
+}  // namespace pluto_hip
