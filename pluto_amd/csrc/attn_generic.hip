@@ -138,7 +138,7 @@ generic_forward_kernel(GenericForwardArgs a) {
         const float logit = load_element(
             a.gate.base, view_offset(a.gate, seq, row, head) + channel,
             a.gate.dtype);
-        float sigmoid = 1.0f / (1.0f + expf(-logit));
+        float sigmoid = gate_sigmoid(logit);
         if (a.round_to_bf16) {
           value = round_to_bf16(round_to_bf16(value) * round_to_bf16(sigmoid));
         } else {

@@ -48,6 +48,14 @@ __host__ __device__ inline float round_to_bf16(float value) {
   return bf16_bits_to_float(float_to_bf16_bits(value));
 }
 
+// Sigmoid of a gate logit, the one form every kernel of the library uses (the
+// cached step, the sequence kernels and the any-shape kernels must agree bit
+// for bit): one v_exp_f32 and one v_rcp_f32, about two units in the last place
+// of FP32 before the result is rounded to bf16.  Saturates to 0 and 1.
+__device__ inline float gate_sigmoid(float logit) {
+  return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-logit * kLog2e));
+}
+
 // Runtime-typed element access for the generic (any shape) kernels.
 __device__ inline float load_element(const void* base, long long index,
                                      int dtype) {

@@ -365,7 +365,7 @@ flash_forward_kernel(FlashForwardArgs a_in, int unit_count) {
               for (int e = 0; e < 4; ++e) {
                 const float logit = __uint_as_float(
                     (e & 1) ? (gw[e / 2] & 0xffff0000u) : (gw[e / 2] << 16));
-                c[e] = round_to_bf16(c[e]) * round_to_bf16(1.0f / (1.0f + expf(-logit)));
+                c[e] = round_to_bf16(c[e]) * round_to_bf16(gate_sigmoid(logit));
               }
             }
             uint2 packed;
@@ -777,7 +777,7 @@ flash_forward_pingpong_kernel(FlashForwardArgs a_in, int unit_count) {
           for (int e = 0; e < 4; ++e) {
             const float logit =
                 __uint_as_float((e & 1) ? (gw[e / 2] & 0xffff0000u) : (gw[e / 2] << 16));
-            c[e] = round_to_bf16(c[e]) * round_to_bf16(1.0f / (1.0f + expf(-logit)));
+            c[e] = round_to_bf16(c[e]) * round_to_bf16(gate_sigmoid(logit));
           }
         }
         uint2 packed;

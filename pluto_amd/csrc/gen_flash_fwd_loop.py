@@ -77,7 +77,10 @@ class Registers:
         self.T0 = take(1, 1)
         self.T1 = take(1, 1)
         self.ALPHA = take(1, 1)
-        self.DADDR = [take(1, 1) for _ in range(self.DB)]   # drain: V^T read addresses
+        self.DADDR = [take(1, 1) for _ in range(self.DB)]   # V^T read addresses of the last blocks
+        self.LIM = take(1, 1)      # last key offset a lane's query sees in the block at hand
+        self.KMASK = take(1, 1)    # the finite sentinel of masked scores
+        self.ROWLIM = take(1, 1)   # input: last key the lane's query sees, minus 4 h
         self.lowest = top
 
     def tile_bytes(self):
@@ -189,11 +192,17 @@ class Emitter:
                 self.emit("s_add_u32 %[voff], %[voff], %[vstep]")
 
     # ---- the softmax of one block as a list of vector-side items ------------------------
-    def softmax_items(self, parity, rare_label, resume_label):
+    def softmax_items(self, parity, rare_label, resume_label, masked=False):
         r = self.r
         S = r.S[parity]
         PF = r.PF[parity]
         items = []
+        if masked:
+            # register i holds key 8 (i / 4) + i % 4 (+ 4 h, folded into LIM) of the block;
+            # keys beyond the lane's limit get the finite sentinel of the reference kernels
+            for i in range(16):
+                items.append("v_cmp_gt_i32 vcc, %d, v%d" % (8 * (i // 4) + i % 4, r.LIM))
+                items.append("v_cndmask_b32 v%d, v%d, v%d, vcc" % (S + i, S + i, r.KMASK))
         # running maximum: the order of flash_forward_kernel
         items.append("v_max3_f32 v%d, v%d, v%d, v%d" % (r.T0, S, S + 1, S + 2))
         for i in range(3, 15, 2):
@@ -258,7 +267,7 @@ class Emitter:
 
     # ---- one iteration -----------------------------------------------------------------
     def iteration(self, parity, scores=True, accumulate=True, softmax=True, v_from=None,
-                  k_from=None, drain_address=None, out_of_line=None):
+                  k_from=None, drain_address=None, out_of_line=None, masked=False):
         """Block b with b % 2 == parity.  scores: S^T(b+1) into S[1 - parity] from
         the K operands in OP.  accumulate: block b-1 from PF[1 - parity] and the
         V^T operands read here from v_from = (stage, half).  k_from: where the K
@@ -276,7 +285,7 @@ class Emitter:
         rescale_label = None
         if softmax:
             rare, resume = self.label("rare"), self.label("resume")
-            items = self.softmax_items(parity, rare, resume)
+            items = self.softmax_items(parity, rare, resume, masked)
             out_of_line.append(("rare", rare, resume))
         if not slots:
             for text in items:
@@ -297,7 +306,7 @@ class Emitter:
                 self.emit("v_mfma_f32_32x32x16_bf16 %s, %s, %s, %s" %
                           (acc, vt(r.OP[ks], 4), vt(r.QF[ks], 4), "0" if ks == 0 else acc))
                 if accumulate:
-                    self.v_read(ks, v_from[0], v_from[1])
+                    self.v_read(ks, v_from[0], v_from[1], drain_address)
                 elif k_from is not None:
                     self.k_read(ks, k_from[0], k_from[1])
             elif slot[0] == "L":
@@ -326,73 +335,155 @@ class Emitter:
             self.emit("%s:" % back)
             out_of_line.append(("rescale", rescale_label, back))
 
-    def step_barrier(self, fill_stage):
+    def step_barrier(self):
+        """The barrier that starts step t (before odd iteration 2t-1): unit t has
+        landed for every wave, everyone is done with unit t-2, whose stage takes
+        unit t+2.  The stage is computed, so the same text serves every place."""
         r = self.r
-        self.emit("s_waitcnt vmcnt(%d)" % (2 * r.loads))
-        self.emit("s_barrier")
-        self.fill(fill_stage)
+        n = r.loads
+        e = self.emit
+        e("s_waitcnt vmcnt(%d)" % (2 * n))
+        e("s_barrier")
+        e("s_add_u32 %[tcount], %[tcount], 1")
+        e("s_add_u32 %[t0], %[tcount], 2")
+        e("s_and_b32 %[t0], %[t0], 3")
+        e("s_mul_i32 %%[t0], %%[t0], %d" % r.stage_bytes())
+        e("s_add_u32 %[t0], %[t0], %[ldsw]")
+        for i in range(n):
+            e("v_add_u32 v%d, %%[koff], v%d" % (r.FTMP[i], r.KFILL[i]))
+        for i in range(n):
+            e("v_add_u32 v%d, %%[voff], v%d" % (r.FTMP[n + i], r.VFILL[i]))
+        e("s_mov_b32 m0, %[t0]")
+        e("s_nop 0")
+        for i in range(n):
+            e("buffer_load_dwordx4 v%d, %%[krsrc], 0 offen%s lds" %
+              (r.FTMP[i], " offset:%d" % (1024 * i) if i else ""))
+        e("s_add_u32 m0, %%[t0], %d" % r.tile_bytes())
+        e("s_nop 0")
+        for i in range(n):
+            e("buffer_load_dwordx4 v%d, %%[vrsrc], 0 offen%s lds" %
+              (r.FTMP[n + i], " offset:%d" % (1024 * i) if i else ""))
+        e("s_add_u32 %[koff], %[koff], %[kstep]")
+        e("s_add_u32 %[voff], %[voff], %[vstep]")
+
+    def last_block_setup(self, masked):
+        """Before one of a wave's last iterations, which read V^T of block
+        %[vblk] from computed addresses and (masked) work on block vblk + 1."""
+        r = self.r
+        e = self.emit
+        # V block j sits in unit j / 2: stage (j / 2) % 4, half j % 2
+        e("s_lshr_b32 %[t0], %[vblk], 1")
+        e("s_and_b32 %[t0], %[t0], 3")
+        e("s_mul_i32 %%[t0], %%[t0], %d" % r.stage_bytes())
+        e("s_and_b32 %[t1], %[vblk], 1")
+        e("s_mul_i32 %%[t1], %%[t1], %d" % r.half_bytes())
+        e("s_add_u32 %[t0], %[t0], %[t1]")
+        for db in range(r.DB):
+            e("v_add_u32 v%d, %%[t0], v%d" % (r.DADDR[db], r.VADDR[0][db]))
+        if masked:
+            e("s_add_u32 %[t1], %[vblk], 1")
+            e("s_lshl_b32 %[t1], %[t1], 5")
+            e("v_subrev_u32 v%d, %%[t1], v%d" % (r.LIM, r.ROWLIM))
 
     # ---- the whole statement ------------------------------------------------------------
     def build(self):
         r = self.r
         out_of_line = []
         e = self.emit
+        n = r.loads
+        one, drain_odd, pre_odd, pre_even, idle = ("Lone_%=", "Ldrain_odd_%=", "Lpre_odd_%=",
+                                                   "Lpre_even_%=", "Lidle_%=")
         e("s_mov_b32 %[m0save], m0")
         e("s_waitcnt vmcnt(0)")
-        # ---- prologue: K(0) into the K half of stage 3, units 0..2 ----------------------
+        e("v_mov_b32 v%d, 0xff7fffff" % r.KMASK)
+        # ---- prologue: K(0) into the K half of stage 3, units 0..2; K(0) and unit 0 awaited ----
         self.fill(3, v_part=False)
         for u in range(3):
             self.fill(u)
-        e("s_waitcnt vmcnt(%d)" % (6 * r.loads))
+        e("s_waitcnt vmcnt(%d)" % (4 * n))
         e("s_barrier")
         for ks in range(r.KS):
             self.k_read(ks, 3, 0)
         # S^T(0), then the K operands of block 1 into the registers it leaves
         self.iteration(1, scores=True, accumulate=False, softmax=False, k_from=(3, 1),
                        out_of_line=out_of_line)
-        e("s_waitcnt vmcnt(%d)" % (4 * r.loads))
-        e("s_barrier")
         e("s_nop 15")   # S^T(0) has left the matrix pipe before the vector side reads it
+        e("v_mov_b32 v%d, v%d" % (r.LIM, r.ROWLIM))
+        e("s_cmp_eq_u32 %[nblk], 1")
+        e("s_cbranch_scc1 %s" % one)
         # iteration 0: softmax(0), S^T(1); K operands of block 2 = K(1), first half (unit 0)
         self.iteration(0, scores=True, accumulate=False, softmax=True, k_from=(0, 0),
-                       out_of_line=out_of_line)
-        # a block whose reference point moved before anything was accumulated: O and l are
-        # zero, only the flag has to go
+                       out_of_line=out_of_line, masked=True)
+        # a reference point that moved before anything was accumulated: O and l are zero
         e("s_mov_b32 %[flag], 0")
-        # ---- steady state: steps t = 1 .. whole_tiles - 1, four to a round -----------------
-        done = "Ldone_%="
+        e("s_cmp_eq_u32 %[nblk], 2")
+        e("s_cbranch_scc1 %s" % drain_odd)
+        # ---- steady state: iterations b = 1 .. nblk - 3, eight to a round (four units) --------
         loop = "Lloop_%="
-        e("s_cmp_eq_u32 %[steps], 0")
-        e("s_cbranch_scc1 %s" % done)
         e("%s:" % loop)
         at_loop_top = list(self.lds_queue)
-        for j in range(4):
-            prev, cur = j % 4, (j + 1) % 4
-            # odd iteration 2t-1: unit t-1 holds V(t-1) and K(t)
-            self.step_barrier((j + 3) % 4)
-            self.iteration(1, v_from=(prev, 0), k_from=(prev, 1), out_of_line=out_of_line)
-            # even iteration 2t: V(t-1) second half; K(t+1) first half (unit t)
-            self.iteration(0, v_from=(prev, 1), k_from=(cur, 0), out_of_line=out_of_line)
-            e("s_sub_u32 %[steps], %[steps], 1")
-            e("s_cmp_eq_u32 %[steps], 0")
-            e("s_cbranch_scc1 %s" % done)
-            # every way into the next step and into the drain leaves the same reads in flight
+        for position in range(8):
+            b = position + 1           # b mod 8
+            t = (b + 1) // 2           # its step, mod 4 below
+            e("s_cmp_eq_u32 %[iters], 0")
+            e("s_cbranch_scc1 %s" % (pre_odd if b % 2 else pre_even))
+            if b % 2:
+                # odd iteration 2t-1: unit t-1 holds V(t-1) and K(t)
+                self.step_barrier()
+                self.iteration(1, v_from=((t - 1) % 4, 0), k_from=((t - 1) % 4, 1),
+                               out_of_line=out_of_line)
+            else:
+                # even iteration 2t: V(t-1) second half; K(t+1) first half (unit t)
+                self.iteration(0, v_from=((t - 1) % 4, 1), k_from=(t % 4, 0),
+                               out_of_line=out_of_line)
+            e("s_sub_u32 %[iters], %[iters], 1")
+            e("s_add_u32 %[vblk], %[vblk], 1")
+            # every way on leaves the same reads in flight
             assert self.lds_queue == at_loop_top
         e("s_branch %s" % loop)
-        e("%s:" % done)
-        # ---- drain: softmax(2W-1) with the products of block 2W-2, then block 2W-1 ---------
-        # unit W-1 must have landed (a one-tile call never passed a step barrier)
-        e("s_waitcnt vmcnt(0)")
-        e("s_barrier")
-        e("s_nop 15")
-        for db in range(r.DB):
-            e("v_add_u32 v%d, %%[drain], v%d" % (r.DADDR[db], r.VADDR[0][db]))
-        self.iteration(1, scores=False, accumulate=True, softmax=True, v_from=(0, 0),
-                       drain_address=r.DADDR, out_of_line=out_of_line)
+        # ---- a wave's last two blocks (masks) and the products still owed -----------------------
+        for first_odd in (True, False):
+            e("%s:" % (pre_odd if first_odd else pre_even))
+            self.lds_queue = list(at_loop_top)
+            if first_odd:
+                self.step_barrier()
+            self.last_block_setup(masked=True)
+            self.iteration(1 if first_odd else 0, scores=True, accumulate=True, softmax=True,
+                           v_from=(0, 0), drain_address=r.DADDR, out_of_line=out_of_line,
+                           masked=True)
+            e("s_add_u32 %[vblk], %[vblk], 1")
+            if not first_odd:
+                e("%s:" % drain_odd)
+                self.step_barrier()
+            self.last_block_setup(masked=True)
+            self.iteration(0 if first_odd else 1, scores=False, accumulate=True, softmax=True,
+                           v_from=(0, 0), drain_address=r.DADDR, out_of_line=out_of_line,
+                           masked=True)
+            e("s_add_u32 %[vblk], %[vblk], 1")
+            self.last_block_setup(masked=False)
+            e("s_nop 7")
+            self.iteration(1 if first_odd else 0, scores=False, accumulate=True, softmax=False,
+                           v_from=(0, 0), drain_address=r.DADDR, out_of_line=out_of_line)
+            e("s_branch %s" % idle)
+        # ---- a wave with a single block ---------------------------------------------------------
+        e("%s:" % one)
+        self.iteration(0, scores=False, accumulate=False, softmax=True, out_of_line=out_of_line,
+                       masked=True)
+        self.last_block_setup(masked=False)
         e("s_nop 7")
-        self.iteration(0, scores=False, accumulate=True, softmax=False, v_from=(0, 1),
+        self.iteration(1, scores=False, accumulate=True, softmax=False, v_from=(0, 0),
                        drain_address=r.DADDR, out_of_line=out_of_line)
-        e("s_waitcnt lgkmcnt(0)")
+        # ---- the steps the slowest wave still has to take: barriers and fills only ------------
+        e("%s:" % idle)
+        again, finished = "Lidle_again_%=", "Lfinished_%="
+        e("%s:" % again)
+        e("s_cmp_eq_u32 %[idle], 0")
+        e("s_cbranch_scc1 %s" % finished)
+        self.step_barrier()
+        e("s_sub_u32 %[idle], %[idle], 1")
+        e("s_branch %s" % again)
+        e("%s:" % finished)
+        e("s_waitcnt vmcnt(0) lgkmcnt(0)")
         e("s_nop 15")
         e("s_nop 15")
         e("s_barrier")
@@ -450,6 +541,7 @@ def render(D):
     define("MUSED", '"+{v%d}"' % r.MUSED)
     define("MTRUE", '"+{v%d}"' % r.MTRUE)
     define("THR", '"+{v%d}"' % r.THR)
+    define("ROWLIM", '"{v%d}"' % r.ROWLIM)
     pinned = set()
     for base in r.O + [r.L]:
         pinned.update(range(base, base + 16))
@@ -457,7 +549,7 @@ def render(D):
         pinned.update(range(base, base + 4))
     for group in r.KADDR + r.VADDR:
         pinned.update(group)
-    pinned.update(r.KFILL + r.VFILL + [r.MUSED, r.MTRUE, r.THR])
+    pinned.update(r.KFILL + r.VFILL + [r.MUSED, r.MTRUE, r.THR, r.ROWLIM])
     clobbers = [v for v in range(r.lowest, 256) if v not in pinned]
     define("CLOBBERS", ", ".join('"v%d"' % v for v in clobbers) + ', "vcc", "scc", "memory"')
     define("LOWEST_VGPR", str(r.lowest))

@@ -588,7 +588,7 @@ decode_fused_kernel(DecodeArgs a, DecodeBatch batch) {
     const float core = o[u] / head_state[1 * GROUP + hh];
     const long long at = static_cast<long long>(seq) * a.query_heads + g * GROUP + hh;
     const float logit = load_element(a.q_gate, (at * 2 + 1) * D + c, a.io_dtype);
-    const float sigmoid = 1.0f / (1.0f + expf(-logit));
+    const float sigmoid = gate_sigmoid(logit);
     store_element(a.out, at * D + c, a.io_dtype,
                   round_to_bf16(round_to_bf16(core) * round_to_bf16(sigmoid)));
   }
