@@ -55,7 +55,7 @@ MEASURED_TRAFFIC_BYTES = {
     ("mha_train_bf16", "flash_forward_kernel<64>"): 126.4e6,
     ("mha_train_bf16", "flash_dq_kernel<64>"): 198.1e6 + 91.3e6,
     ("mha_train_bf16", "flash_dkv_kernel<64>"): 154.2e6 + 100.7e6,
-    ("gqa_prefill", "flash_forward_pingpong_kernel<128>"): 168.8e6 + 52.8e6,
+    ("gqa_prefill", "flash_forward_pipelined_kernel<128>"): 168.8e6 + 52.8e6,
     ("gqa_decode", "decode_fused_kernel<128,6>"): 1044.3e6 + 13.0e6,
     ("gdn_scan", "gdn_chunk_prepare + gdn_chunk_scan"): 1052.6e6,
 }
@@ -181,7 +181,7 @@ def gqa_prefill(torch, capi):
 
     work = 4.0 * qh * d * causal_pairs(T)
     return dict(step=step,
-                kernels=[("flash_forward_pingpong_kernel<128>", step, capi.MAIN_KERNEL | capi.PING_PONG, work),
+                kernels=[("flash_forward_pipelined_kernel<128>", step, capi.MAIN_KERNEL | capi.EIGHT_WAVE, work),
                          ("rope table + prepare", step, capi.AUXILIARY_KERNELS, None)],
                 work=work,
                 metric="gqa_prefill_tflops", unit="TFLOP/s", dtype="bf16", bound="mfma",

@@ -546,8 +546,9 @@ int pluto_hip_test_force_generic(int enabled);
  * attention forward, key-owned attention backward, split-K decode, delta-net
  * scan; 2 = the query-owned attention backward kernel; 4 = auxiliary kernels:
  * preparation, tables, combines; 16 = not a kernel: with this bit cleared the
- * attention forward at head width 128 keeps to its four-wave kernel whatever
- * the sequence length, which lets a test compare its two kernels).  A benchmark
+ * attention forward at head widths 64 and 128 keeps to its four-wave kernel
+ * whatever the sequence length, which lets a test compare it with the
+ * eight-wave kernel that long sequences take).  A benchmark
  * runs the whole call once, then times one class with events around the call.  Returns the previous mask;
  * the default, ~0u, runs everything.  Thread-local like the switch above, and
  * like it written by nothing on the product path. */

@@ -176,7 +176,7 @@ class force_generic:
 
 
 MAIN_KERNEL, QUERY_KERNEL, AUXILIARY_KERNELS = 1, 2, 4
-PING_PONG = 16  # permission bit, not a kernel: see pluto_hip_test_kernel_classes
+EIGHT_WAVE = 16  # permission bit, not a kernel: see pluto_hip_test_kernel_classes
 (PATH_NONE, PATH_GENERIC, PATH_MATRIX_F32, PATH_FLASH, PATH_SPLIT_K, PATH_CHUNKED,
  PATH_RECURRENCE) = range(7)
 

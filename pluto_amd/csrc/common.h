@@ -107,8 +107,7 @@ enum KernelClass : unsigned {
   kMainKernel = 1u,       // the kernel that bounds the call (flash, split-K, scan ...)
   kQueryKernel = 2u,      // the query-owned half of the attention backward
   kAuxiliaryKernel = 4u,  // preparation, tables, combines
-  kPingPong = 16u,        // not a kernel: the D = 128 forward may use its eight-wave variants
-  kPipelined = 32u,       // not a kernel: of those, the one with the hand-scheduled loop
+  kEightWave = 16u,        // not a kernel: the forward may use its eight-wave kernel (hand-scheduled loop)
 };
 bool kernel_enabled(KernelClass which);  // mha_capi.hip
 // Records the kernel family a compute call chose (pluto_hip_test_last_path).

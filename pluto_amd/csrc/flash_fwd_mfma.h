@@ -34,9 +34,9 @@ struct FlashForwardArgs {
 bool flash_forward_supported(const FlashForwardArgs& args, int head_dim);
 int launch_flash_forward(hipStream_t stream, const FlashForwardArgs& args,
                          int head_dim, int sequences);
-// flash_fwd_pipelined.hip: head width 128, 256-row query tiles, hand-scheduled
+// flash_fwd_pipelined.hip: head widths 64 and 128, 256-row query tiles, hand-scheduled
 // main loop; what launch_flash_forward picks for long sequences.
 int launch_flash_forward_pipelined(hipStream_t stream, const FlashForwardArgs& args,
-                                   int sequences);
+                                   int head_dim, int sequences);
 
 }  // namespace pluto_hip

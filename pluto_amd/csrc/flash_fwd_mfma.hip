@@ -35,7 +35,9 @@ namespace pluto_hip {
 namespace {
 
 constexpr int BN = 64;  // keys per LDS tile
-constexpr int kPingPongFromRows = 1024;
+// measured on both head widths: level with the four-wave kernel at 2048 rows,
+// 10-15 % ahead from 4096, behind it at 1024 (few, short tiles per workgroup)
+constexpr int kPipelinedFromRows = 2048;
 
 // Queues the loads of one K tile and one V tile (keys k0..k0+63) into an LDS
 // stage.  Lane l of load i of a wave writes 16 bytes at chunk
@@ -393,411 +395,6 @@ flash_forward_kernel(FlashForwardArgs a_in, int unit_count) {
   }
 }
 
-// ---------------------------------------------------------------------------
-// Ping-pong variant (D = 128, one query tile of 256 rows a workgroup, unpaired
-// schedule).
-//
-// What bounds flash_forward_kernel is instruction issue: a wave issues at most
-// one instruction every four cycles, whatever its kind, and stalls on its own
-// dependencies, while the matrix pipe needs a new instruction only every 32.
-// Per 32-key block a wave has a matrix phase M(b) = { S^T of block b,
-// O^T += V^T P^T of block b-1 } and a vector phase V(b) = { softmax of block b }.
-// The K operands of M(b+1) are read from LDS in the middle of V(b), the V^T
-// operands of M(b+1) at its own start (they are needed only after the S^T
-// chain).  Here a workgroup has eight waves,
-// two a SIMD; every phase ends with a workgroup barrier and the wave of a SIMD
-// that arrives second runs one phase behind the first, so that on every SIMD
-// one wave is in its matrix phase while the other is in its vector phase, and
-// neither phase contains anything the other unit has to wait for.  Every wave
-// passes the same number of barriers whatever it sees of the causal mask: the
-// loop bounds are the workgroup's, only the work inside a phase is conditional.
-//
-// K/V tiles (64 keys = two blocks) rotate through three LDS stages.  Tile t is
-// read from V(2t-1) (K operands of its first block) to M(2t+2) (V^T operands
-// of its second); tile t+3 takes its place and is requested in M(2t+3) by
-// either kind of wave, after the barrier that ends the late waves' M(2t+2);
-// its first read is in V(2t+5), and the barrier before that phase is passed
-// only by waves whose own loads of the tile have landed.
-template <int D>
-__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
-flash_forward_pingpong_kernel(FlashForwardArgs a_in, int unit_count) {
-  struct Args : FlashForwardArgs {
-    int unit_count;
-  } a;
-  static_cast<FlashForwardArgs&>(a) = a_in;
-  a.unit_count = unit_count;
-  constexpr int WAVES = 8, KCH = D / 8, KS = D / 16, DB = D / 32;
-  constexpr int BM = 32 * WAVES;
-  constexpr int kTileBytes = BN * D * 2, kStageBytes = 2 * kTileBytes, kStages = 3;
-  constexpr int kLoads = BN * KCH / (64 * WAVES);  // 16-byte loads per lane, tensor and tile
-  constexpr int kFillLoads = 2 * kLoads;           // vector-memory operations of one fill
-  constexpr int kHalfTile = 32 * KCH * 16;         // bytes of a 32-key block within a tile
-  static_assert(kLoads >= 1 && BN == 64, "two 32-key blocks a tile, a load for every lane");
-  __shared__ __attribute__((aligned(1024))) unsigned char lds[kStages * kStageBytes];
-  __shared__ int arrivals[4];
-
-  const int tid = threadIdx.x;
-  const int wave = __builtin_amdgcn_readfirstlane(tid / 64), lane = tid % 64;
-  const int h = lane / 32, n = lane % 32;
-  const int q_tiles = (a.q_rows + BM - 1) / BM;
-  int q_tile, head, seq;
-  {
-    // as in flash_forward_kernel's unpaired schedule: the query heads of a kv
-    // head at one query tile run on one XCD, heaviest tiles first
-    const int kv_heads = a.query_heads / a.group;
-    const int kv_units = a.unit_count / q_tiles;
-    const int xcd = blockIdx.x % 8, slot = blockIdx.x / 8;
-    const int u = 8 * (slot / a.group) + xcd;
-    if (u >= a.unit_count) return;  // the whole workgroup
-    q_tile = q_tiles - 1 - u / kv_units;
-    const int kv_unit = u % kv_units;
-    head = (kv_unit % kv_heads) * a.group + slot % a.group;
-    seq = kv_unit / kv_heads;
-  }
-  // Which of the two waves of a SIMD runs one phase behind: the one that gets
-  // here second (the hardware places two of these waves on each SIMD, by no
-  // rule in the wave's index).  HW_ID bits 5:4 are the SIMD.
-  if (tid < 4) arrivals[tid] = 0;
-  __syncthreads();
-  int late;
-  {
-    const int simd = static_cast<int>(__builtin_amdgcn_s_getreg((1 << 11) | (4 << 6) | 4));
-    int order = 0;
-    if (lane == 0) order = atomicAdd(&arrivals[simd], 1);
-    late = __builtin_amdgcn_readfirstlane(order) & 1;
-  }
-  const int kv_head = head / a.group;
-  const uint16_t* q_base = a.q + seq * a.q_seq_stride + head * a.q_head_stride;
-  const uint16_t* k_base = a.k + seq * a.k_seq_stride + kv_head * a.k_head_stride;
-  const uint16_t* v_base = a.v + seq * a.v_seq_stride + kv_head * a.v_head_stride;
-  uint16_t* o_base = a.out + seq * a.o_seq_stride + head * a.o_head_stride;
-  const uint16_t* gate_base =
-      a.gate ? a.gate + seq * a.gate_seq_stride + head * a.gate_head_stride : nullptr;
-  const float scale2 = a.scale * kLog2e;
-  bf16x8 ones;
-#pragma unroll
-  for (int e = 0; e < 8; ++e) ones[e] = static_cast<__bf16>(1.0f);
-
-  // lane addresses: the layouts of flash_forward_kernel
-  uint32_t k_fill[kLoads], v_fill[kLoads];
-#pragma unroll
-  for (int i = 0; i < kLoads; ++i) {
-    const int p = (wave * kLoads + i) * 64 + lane;
-    const int row = p / KCH, slot = p % KCH;
-    k_fill[i] = static_cast<uint32_t>(row * a.k_row_stride * 2 + (slot ^ (row & 7)) * 16);
-    v_fill[i] = static_cast<uint32_t>(row * a.v_row_stride * 2 + (slot ^ (2 * (row & 3))) * 16);
-  }
-  int k_read[KS];
-#pragma unroll
-  for (int ks = 0; ks < KS; ++ks) k_read[ks] = (n * KCH + ((2 * ks + h) ^ (n & 7))) * 16;
-  int v_read[DB];
-  {
-    const int gq = lane / 16, kk = (lane % 16) / 4, b = lane % 4;
-    const int row = 4 * (gq / 2) + kk;
-#pragma unroll
-    for (int db = 0; db < DB; ++db) {
-      const int chunk = 4 * db + 2 * (gq % 2) + b / 2;
-      v_read[db] = (row * KCH + (chunk ^ (2 * kk))) * 16 + (b % 2) * 8;
-    }
-  }
-
-  const int q0 = q_tile * BM;
-  const int wave_q0 = q0 + 32 * wave;
-  const int q_row = wave_q0 + n;
-  bf16x8 qf[KS];
-  {
-    const int row = min(q_row, a.q_rows - 1);
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
-      qf[ks] = as_bf16x8(*reinterpret_cast<const uint4*>(
-          q_base + static_cast<long long>(row) * a.q_row_stride + 16 * ks + 8 * h));
-  }
-  const int row_limit = min(a.start_position + q_row, a.kv_rows - 1);
-  floatx16 o_acc[DB], l_acc;
-  constexpr float kLazy = 8.0f;
-  float m_used = kMasked, m_true = kMasked;
-#pragma unroll
-  for (int i = 0; i < 16; ++i) l_acc[i] = 0.0f;
-#pragma unroll
-  for (int db = 0; db < DB; ++db)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) o_acc[db][i] = 0.0f;
-
-  // workgroup-uniform loop bounds
-  const int last_row = min(q0 + BM, a.q_rows) - 1;
-  const int visible_keys = min(a.kv_rows, a.start_position + last_row + 1);
-  const int tiles = (visible_keys + BN - 1) / BN;
-  const int blocks = 2 * tiles;
-  // tiles every row of the workgroup sees whole: no masks, no wave drops out
-  const int whole_tiles = min(tiles, min(a.start_position + q0 + 1, a.kv_rows) / BN);
-  // block b (keys 32 b ..) matters to this wave if any of its rows sees it
-  const int wave_last_key = a.start_position + wave_q0 + 31;
-  auto matters = [&](int b) { return b < blocks && 32 * b <= wave_last_key; };
-  // One descriptor per tensor for all rows of this (sequence, kv head): rows at
-  // or beyond kv_rows read as zero; a tile's byte offset goes into the lanes'
-  // offsets (flash_forward_supported keeps all of it below 2^31).
-  const int32x4 k_all = make_rsrc(
-      k_base, static_cast<uint32_t>(((a.kv_rows - 1) * a.k_row_stride + D) * 2));
-  const int32x4 v_all = make_rsrc(
-      v_base, static_cast<uint32_t>(((a.kv_rows - 1) * a.v_row_stride + D) * 2));
-  const uint32_t k_tile_step = static_cast<uint32_t>(BN * a.k_row_stride * 2);
-  const uint32_t v_tile_step = static_cast<uint32_t>(BN * a.v_row_stride * 2);
-  // s_waitcnt lgkmcnt(0), the other counters left alone; as a builtin, so that
-  // the compiler's own bookkeeping knows the LDS reads of a phase are complete
-  // when the next one starts
-  constexpr int kWaitLds = 0xC07F;
-  const uint32_t lds_address = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_void*)lds));
-  static_assert(kLoads == 2, "the fill below pairs a lane's two loads of a tensor under one M0");
-  // the second load of a pair lands 1024 bytes further on in LDS through the
-  // instruction's offset, which also moves its global address: taken out of
-  // the lane's offset again
-  const uint32_t k_second = k_fill[1] - 1024u, v_second = v_fill[1] - 1024u;
-  auto fill = [&](int tile, int stage_offset) {
-    const uint32_t k_at = static_cast<uint32_t>(tile) * k_tile_step;
-    const uint32_t v_at = static_cast<uint32_t>(tile) * v_tile_step;
-    const uint32_t k_lds = lds_address + stage_offset + wave * kLoads * 1024;
-    const uint32_t v_lds = k_lds + kTileBytes;
-    uint32_t saved_m0;
-    asm volatile(
-        "s_mov_b32 %0, m0\n\t"
-        "s_mov_b32 m0, %1\n\ts_nop 0\n\t"
-        "buffer_load_dwordx4 %3, %7, 0 offen lds\n\t"
-        "buffer_load_dwordx4 %4, %7, 0 offen offset:1024 lds\n\t"
-        "s_mov_b32 m0, %2\n\ts_nop 0\n\t"
-        "buffer_load_dwordx4 %5, %8, 0 offen lds\n\t"
-        "buffer_load_dwordx4 %6, %8, 0 offen offset:1024 lds\n\t"
-        "s_mov_b32 m0, %0"
-        : "=&s"(saved_m0)
-        : "s"(k_lds), "s"(v_lds), "v"(k_fill[0] + k_at), "v"(k_second + k_at), "v"(v_fill[0] + v_at),
-          "v"(v_second + v_at), "s"(k_all), "s"(v_all)
-        : "memory");
-  };
-  // this wave's loads of tile `tile` have landed; the fill of tile + 1, if there
-  // is one, was requested later and may still travel (loads complete in order)
-  auto landed = [&](int tile) {
-    if (tile + 1 < tiles)
-      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kFillLoads) : "memory");
-    else
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  };
-  // nothing moves across a phase boundary, neither in the compiler's schedule
-  // nor (for memory) in its earlier passes
-  auto phase_barrier = [&]() {
-    __builtin_amdgcn_sched_barrier(0);
-    asm volatile("s_barrier" ::: "memory");
-    __builtin_amdgcn_sched_barrier(0);
-  };
-
-  bf16x8 kf[KS], vf[2][DB], pf[2];
-  floatx16 s;
-  floatx16 zero;
-#pragma unroll
-  for (int i = 0; i < 16; ++i) zero[i] = 0.0f;
-  auto read_k = [&](int stage_offset, int half) {  // A operands of S^T
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
-      kf[ks] = as_bf16x8(*reinterpret_cast<const uint4*>(lds + stage_offset + k_read[ks] + half * kHalfTile));
-  };
-  auto read_v = [&](int stage_offset, int half) {  // A operands of O^T
-    const unsigned char* tile = lds + stage_offset + kTileBytes + half * kHalfTile;
-#pragma unroll
-    for (int s2 = 0; s2 < 2; ++s2)
-#pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        const int at = v_read[db] + 16 * s2 * KCH * 16;
-        const uint2 lo = lds_transpose_read(tile, at);
-        const uint2 hi = lds_transpose_read(tile, at + 8 * KCH * 16);
-        vf[s2][db] = __builtin_bit_cast(bf16x8, make_uint4(lo.x, lo.y, hi.x, hi.y));
-      }
-  };
-  auto scores = [&]() {  // S^T of the block whose K operands are in kf
-    s = mfma32(kf[0], qf[0], zero);
-#pragma unroll
-    for (int ks = 1; ks < KS; ++ks) s = mfma32(kf[ks], qf[ks], s);
-  };
-  auto accumulate = [&]() {  // O^T += V^T P^T, l += 1^T P^T
-#pragma unroll
-    for (int s2 = 0; s2 < 2; ++s2) {
-      l_acc = mfma32(ones, pf[s2], l_acc);
-#pragma unroll
-      for (int db = 0; db < DB; ++db) o_acc[db] = mfma32(vf[s2][db], pf[s2], o_acc[db]);
-    }
-  };
-  auto statistics = [&](int b, bool may_mask) {  // masks s, follows the row maximum
-    const int kb0 = 32 * b;
-    if (may_mask && (kb0 + 31 > a.start_position + wave_q0 || kb0 + 32 > a.kv_rows)) {
-      const int limit = row_limit - kb0 - 4 * h;
-#pragma unroll
-      for (int i = 0; i < 16; ++i) s[i] = (8 * (i / 4) + (i % 4) > limit) ? kMasked : s[i];
-    }
-    float row_max = fmaxf(fmaxf(s[0], s[1]), s[2]);
-#pragma unroll
-    for (int i = 3; i < 15; i += 2) row_max = fmaxf(fmaxf(row_max, s[i]), s[i + 1]);
-    row_max = fmaxf(row_max, s[15]);
-    m_true = fmaxf(m_true, half_swap_max(row_max));
-    const float candidate = m_true * scale2;
-    if (__any(candidate > m_used + kLazy)) {
-      const float m_new = candidate > m_used + kLazy ? candidate : m_used;
-      const float alpha = __builtin_amdgcn_exp2f(m_used - m_new);
-      m_used = m_new;
-      l_acc[0] *= alpha;
-#pragma unroll
-      for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) o_acc[db][i] *= alpha;
-    }
-  };
-  auto probabilities = [&]() {  // s -> pf
-#pragma unroll
-    for (int s2 = 0; s2 < 2; ++s2) {
-      uint32_t packed[4];
-#pragma unroll
-      for (int e = 0; e < 4; ++e)
-        packed[e] = pack_bf16(
-            __builtin_amdgcn_exp2f(__builtin_fmaf(s[8 * s2 + 2 * e], scale2, -m_used)),
-            __builtin_amdgcn_exp2f(__builtin_fmaf(s[8 * s2 + 2 * e + 1], scale2, -m_used)));
-      // the probabilities exist at the end of the vector phase, not where the
-      // matrix phase happens to use them
-      asm volatile("" : "+v"(packed[0]), "+v"(packed[1]), "+v"(packed[2]), "+v"(packed[3]));
-      pf[s2] = __builtin_bit_cast(bf16x8, make_uint4(packed[0], packed[1], packed[2], packed[3]));
-    }
-  };
-
-  if (tiles > 0) {
-    // ---- prologue: three tiles requested, the first awaited; M(0) -----------
-    fill(0, 0);
-    if (tiles > 1) fill(1, kStageBytes);
-    if (tiles > 2) fill(2, 2 * kStageBytes);
-    if (tiles > 2)
-      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kFillLoads) : "memory");
-    else if (tiles > 1)
-      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kFillLoads) : "memory");
-    else
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    phase_barrier();
-    if (late) phase_barrier();
-    // ---- M(0)
-    read_k(0, 0);  // block 0 matters to every wave
-    __builtin_amdgcn_s_setprio(2);
-    scores();
-    __builtin_amdgcn_s_setprio(0);
-    phase_barrier();
-
-    // stage offsets of tiles t, t + 1, t + 2
-    int cur = 0, nxt = kStageBytes, third = 2 * kStageBytes;
-    // One tile: V(2t), M(2t+1), V(2t+1), M(2t+2).  `conditional`: blocks may be
-    // masked or invisible to this wave (the diagonal tiles).  Tile t+1 is first
-    // read in V(2t+1); the barrier before it ends the early waves' M(2t+1) and
-    // the late waves' V(2t), which is where each kind waits for its own loads
-    // of that tile.  Tile t+2 is requested in M(2t+1), into the stage tile t-1
-    // left with the late waves' M(2t).
-    auto one_tile = [&](int t, bool conditional) {
-      const bool m0 = !conditional || matters(2 * t);
-      const bool m1 = !conditional || matters(2 * t + 1);
-      const bool m2 = conditional ? matters(2 * t + 2) : true;
-      // ---- V(2t): the K operands of the next matrix phase are requested in
-      // mid-phase, once the other waves' V^T reads, all issued as their matrix
-      // phase starts, have left the LDS queue
-      if (m0) statistics(2 * t, conditional);
-      __builtin_amdgcn_sched_barrier(0);
-      if (m1) read_k(cur, 1);
-      __builtin_amdgcn_sched_barrier(0);
-      if (m0) probabilities();
-      __builtin_amdgcn_s_waitcnt(kWaitLds);
-      if (late && t + 1 < tiles) {
-        // the late waves' newest request is tile t + 1 itself, except in the
-        // first iteration, where the prologue also asked for tile 2
-        if (t == 0 && tiles > 2)
-          asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kFillLoads) : "memory");
-        else
-          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      }
-      phase_barrier();
-      // ---- M(2t+1)
-      if (m0) read_v(cur, 0);
-      __builtin_amdgcn_s_setprio(2);
-      if (m1) scores();
-      if (t >= 1 && t + 2 < tiles) fill(t + 2, third);
-      if (m0) accumulate();
-      __builtin_amdgcn_s_setprio(0);
-      if (!late && t + 1 < tiles) landed(t + 1);
-      phase_barrier();
-      // ---- V(2t+1)
-      if (m1) statistics(2 * t + 1, conditional);
-      __builtin_amdgcn_sched_barrier(0);
-      if (m2) read_k(nxt, 0);
-      __builtin_amdgcn_sched_barrier(0);
-      if (m1) probabilities();
-      __builtin_amdgcn_s_waitcnt(kWaitLds);
-      phase_barrier();
-      // ---- M(2t+2)
-      if (m1) read_v(cur, 1);
-      __builtin_amdgcn_s_setprio(2);
-      if (m2) scores();
-      if (m1) accumulate();
-      __builtin_amdgcn_s_setprio(0);
-      phase_barrier();
-      const int freed = cur;
-      cur = nxt;
-      nxt = third;
-      third = freed;
-    };
-    int t = 0;
-    for (; t < whole_tiles && t + 1 < tiles; ++t) one_tile(t, false);
-    for (; t < tiles; ++t) one_tile(t, true);
-    if (!late) phase_barrier();
-  }
-
-  // ---- epilogue: as in flash_forward_kernel ------------------------------------
-  const float l_used = l_acc[0] > 0.0f ? l_acc[0] : 1.0f;
-  const float inverse = 1.0f / l_used;
-  if (q_row < a.q_rows) {
-    uint16_t* o_row = o_base + static_cast<long long>(q_row) * a.o_row_stride;
-    uint16_t* core_row = a.core ? a.core + (o_row - a.out) : nullptr;
-    const uint16_t* gate_row =
-        gate_base ? gate_base + static_cast<long long>(q_row) * a.gate_row_stride : nullptr;
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int d = 32 * db + 8 * j + 4 * h;
-        float c[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) c[e] = o_acc[db][4 * j + e] * inverse;
-        if (core_row) {
-          uint2 plain;
-          plain.x = pack_bf16(c[0], c[1]);
-          plain.y = pack_bf16(c[2], c[3]);
-          *reinterpret_cast<uint2*>(core_row + d) = plain;
-        }
-        if (gate_row) {
-          const uint2 gate_bits = *reinterpret_cast<const uint2*>(gate_row + d);
-          const uint32_t gw[2] = {gate_bits.x, gate_bits.y};
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const float logit =
-                __uint_as_float((e & 1) ? (gw[e / 2] & 0xffff0000u) : (gw[e / 2] << 16));
-            c[e] = round_to_bf16(c[e]) * round_to_bf16(gate_sigmoid(logit));
-          }
-        }
-        uint2 packed;
-        packed.x = pack_bf16(c[0], c[1]);
-        packed.y = pack_bf16(c[2], c[3]);
-        *reinterpret_cast<uint2*>(o_row + d) = packed;
-      }
-    if (h == 0) {
-      const float normalizer = l_used * __builtin_amdgcn_exp2f(m_used - m_true * scale2);
-      const float maximum = m_true * a.scale;
-      const long long stat = (static_cast<long long>(seq) * a.query_heads + head) * a.q_rows + q_row;
-      if (a.maxima) a.maxima[stat] = maximum;
-      if (a.normalizers) a.normalizers[stat] = normalizer;
-      if (a.lse)
-        a.lse[(static_cast<long long>(seq) * a.q_rows + q_row) * a.query_heads + head] =
-            maximum + __logf(normalizer);
-    }
-  }
-}
-
 long long grid_blocks(const FlashForwardArgs& a, int block_rows, int sequences, bool paired) {
   const long long q_tiles = (a.q_rows + block_rows - 1) / block_rows;
   return (paired ? (q_tiles + 1) / 2 : q_tiles) * a.query_heads * sequences;
@@ -838,20 +435,15 @@ int launch_flash_forward(hipStream_t stream, const FlashForwardArgs& a,
   const dim3 grid(static_cast<unsigned>(blocks));
   const int unit_count = static_cast<int>(units);
   if (!kernel_enabled(kMainKernel)) return 0;
-  // Long sequences at D = 128 take the eight-wave ping-pong kernel (3-4 %
-  // faster at 8192 rows); its 256-row tiles waste waves on short ones.
-  if (head_dim == 128 && a.q_rows >= kPingPongFromRows && kernel_enabled(kPingPong)) {
-    // its epilogue addresses a head's rows through 32-bit buffer offsets
+  // Long sequences at head widths 64 and 128 take the eight-wave kernel with
+  // the hand-scheduled loop (flash_fwd_pipelined.hip): 256-row tiles, which
+  // short sequences do not fill.  Its epilogue addresses a head's rows through
+  // 32-bit buffer offsets.
+  if ((head_dim == 128 || head_dim == 64) && a.q_rows >= kPipelinedFromRows &&
+      kernel_enabled(kEightWave)) {
     const long long widest = a.gate ? std::max(a.o_row_stride, a.gate_row_stride) : a.o_row_stride;
-    if (kernel_enabled(kPipelined) && a.q_rows * widest * 2 < (1LL << 31) - 4096)
-      return launch_flash_forward_pipelined(stream, a, sequences);
-    const long long pp_tiles = (a.q_rows + 255) / 256;
-    const long long pp_units = pp_tiles * sequences * (a.query_heads / a.group);
-    const long long pp_blocks = (pp_units + 7) / 8 * 8 * a.group;
-    if (pp_blocks > 0x7fffffffLL) return PLUTO_HIP_EINVAL;
-    flash_forward_pingpong_kernel<128><<<dim3(static_cast<unsigned>(pp_blocks)), 512, 0, stream>>>(
-        a, static_cast<int>(pp_units));
-    return launch_status();
+    if (a.q_rows * widest * 2 < (1LL << 31) - 4096)
+      return launch_flash_forward_pipelined(stream, a, head_dim, sequences);
   }
   if (head_dim == 256)
     flash_forward_kernel<256, 1, 4><<<grid, 256, 0, stream>>>(a, unit_count);

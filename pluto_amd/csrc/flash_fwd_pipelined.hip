@@ -28,7 +28,6 @@ namespace pluto_hip {
 namespace {
 
 constexpr int BN = 64;
-constexpr int kRows = 256;  // query rows a workgroup processes at a time
 
 // Which query tiles a workgroup processes.  The causal mask makes tiles
 // unequal (tile t costs about t + 1 units plus a fixed part) and a long
@@ -45,20 +44,29 @@ struct Schedule {
   uint16_t item[kScheduleEntries];  // (sequence * heads + head) * q_tiles + q_tile
 };
 
+// Head width 128: eight waves, 256 query rows and 128 KiB of key/value stages
+// a workgroup, one workgroup a compute unit.  Head width 64: four waves, 128
+// rows, 64 KiB, two workgroups a compute unit, so that one computes while the
+// other waits for its first tiles or writes its output (at 1024 rows a tile's
+// loop is short against those).
 template <int D>
-__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
+constexpr int kWaves = D == 128 ? FLASH_LOOP_D128_WAVES : FLASH_LOOP_D64_WAVES;
+
+template <int D>
+__global__ void __launch_bounds__(64 * kWaves<D>) __attribute__((amdgpu_waves_per_eu(2, 2)))
 flash_forward_pipelined_kernel(FlashForwardArgs a_in, int unit_count, Schedule schedule) {
   struct Args : FlashForwardArgs {
     int unit_count;
   } a;
   static_cast<FlashForwardArgs&>(a) = a_in;
   a.unit_count = unit_count;
-  constexpr int WAVES = 8, KCH = D / 8, KS = D / 16, DB = D / 32;
+  constexpr int WAVES = kWaves<D>, KCH = D / 8, KS = D / 16, DB = D / 32;
   constexpr int BM = 32 * WAVES;
   constexpr int kTileBytes = BN * D * 2, kStageBytes = 2 * kTileBytes, kStages = 4;
   constexpr int kLoads = BN * KCH / (64 * WAVES);
-    static_assert(D == 128, "the loop text is instantiated for this head width");
-  static_assert(kLoads == FLASH_LOOP_D128_LOADS && kStageBytes == FLASH_LOOP_D128_STAGE_BYTES);
+  static_assert(D == 128 || D == 64, "the loop text is instantiated for these head widths");
+  static_assert(D == 128 ? (kLoads == FLASH_LOOP_D128_LOADS && kStageBytes == FLASH_LOOP_D128_STAGE_BYTES)
+                         : (kLoads == FLASH_LOOP_D64_LOADS && kStageBytes == FLASH_LOOP_D64_STAGE_BYTES));
   __shared__ __attribute__((aligned(1024))) unsigned char lds[kStages * kStageBytes];
 
   const int tid = threadIdx.x;
@@ -174,48 +182,74 @@ flash_forward_pipelined_kernel(FlashForwardArgs a_in, int unit_count, Schedule s
     uint32_t saved_m0, scalar_temp0, scalar_temp1;
     float threshold = m_used + kLazy;
     const int row_limit_lane = row_limit - 4 * h;
-    // the second load of a pair lands 1024 bytes further on in LDS through the
-    // instruction's offset, which also moves its global address: taken out of
-    // the lane's offset again
-    const uint32_t k_second = k_fill[1] - 1024u, v_second = v_fill[1] - 1024u;
-    const int k_read_high[KS] = {k_read[0] + 65536, k_read[1] + 65536, k_read[2] + 65536,
-                                 k_read[3] + 65536, k_read[4] + 65536, k_read[5] + 65536,
-                                 k_read[6] + 65536, k_read[7] + 65536};
-    const int v_read_high[DB] = {v_read[0] + 65536, v_read[1] + 65536, v_read[2] + 65536,
-                                 v_read[3] + 65536};
-    asm volatile(FLASH_LOOP_D128_ASM
-                 : FLASH_LOOP_D128_O0(o_acc[0]), FLASH_LOOP_D128_O1(o_acc[1]),
-                   FLASH_LOOP_D128_O2(o_acc[2]), FLASH_LOOP_D128_O3(o_acc[3]),
-                   FLASH_LOOP_D128_L(l_acc), FLASH_LOOP_D128_MUSED(m_used),
-                   FLASH_LOOP_D128_MTRUE(m_true), FLASH_LOOP_D128_THR(threshold),
-                   [iters] "+s"(iterations), [flag] "+s"(flag), [koff] "+s"(k_offset),
-                   [voff] "+s"(v_offset), [tcount] "+s"(steps_done), [vblk] "+s"(v_block),
-                   [idle] "+s"(idle_steps), [m0save] "=&s"(saved_m0), [t0] "=&s"(scalar_temp0),
-                   [t1] "=&s"(scalar_temp1)
-                 : FLASH_LOOP_D128_QF0(qf[0]), FLASH_LOOP_D128_QF1(qf[1]),
-                   FLASH_LOOP_D128_QF2(qf[2]), FLASH_LOOP_D128_QF3(qf[3]),
-                   FLASH_LOOP_D128_QF4(qf[4]), FLASH_LOOP_D128_QF5(qf[5]),
-                   FLASH_LOOP_D128_QF6(qf[6]), FLASH_LOOP_D128_QF7(qf[7]),
-                   FLASH_LOOP_D128_ONES(ones),
-                   FLASH_LOOP_D128_KADDR0_0(k_read[0]), FLASH_LOOP_D128_KADDR0_1(k_read[1]),
-                   FLASH_LOOP_D128_KADDR0_2(k_read[2]), FLASH_LOOP_D128_KADDR0_3(k_read[3]),
-                   FLASH_LOOP_D128_KADDR0_4(k_read[4]), FLASH_LOOP_D128_KADDR0_5(k_read[5]),
-                   FLASH_LOOP_D128_KADDR0_6(k_read[6]), FLASH_LOOP_D128_KADDR0_7(k_read[7]),
-                   FLASH_LOOP_D128_KADDR1_0(k_read_high[0]), FLASH_LOOP_D128_KADDR1_1(k_read_high[1]),
-                   FLASH_LOOP_D128_KADDR1_2(k_read_high[2]), FLASH_LOOP_D128_KADDR1_3(k_read_high[3]),
-                   FLASH_LOOP_D128_KADDR1_4(k_read_high[4]), FLASH_LOOP_D128_KADDR1_5(k_read_high[5]),
-                   FLASH_LOOP_D128_KADDR1_6(k_read_high[6]), FLASH_LOOP_D128_KADDR1_7(k_read_high[7]),
-                   FLASH_LOOP_D128_VADDR0_0(v_read[0]), FLASH_LOOP_D128_VADDR0_1(v_read[1]),
-                   FLASH_LOOP_D128_VADDR0_2(v_read[2]), FLASH_LOOP_D128_VADDR0_3(v_read[3]),
-                   FLASH_LOOP_D128_VADDR1_0(v_read_high[0]), FLASH_LOOP_D128_VADDR1_1(v_read_high[1]),
-                   FLASH_LOOP_D128_VADDR1_2(v_read_high[2]), FLASH_LOOP_D128_VADDR1_3(v_read_high[3]),
-                   FLASH_LOOP_D128_KFILL0(k_fill[0]), FLASH_LOOP_D128_KFILL1(k_second),
-                   FLASH_LOOP_D128_VFILL0(v_fill[0]), FLASH_LOOP_D128_VFILL1(v_second),
-                   FLASH_LOOP_D128_ROWLIM(row_limit_lane),
-                   [krsrc] "s"(k_all), [vrsrc] "s"(v_all), [scale2] "s"(scale2_bits),
-                   [kstep] "s"(k_tile_step), [vstep] "s"(v_tile_step), [ldsw] "s"(lds_wave),
-                   [nblk] "s"(wave_blocks)
-                 : FLASH_LOOP_D128_CLOBBERS);
+    if constexpr (D == 128) {
+      // the second load of a pair lands 1024 bytes further on in LDS through the
+      // instruction's offset, which also moves its global address: taken out of
+      // the lane's offset again
+      const uint32_t k_second = k_fill[1] - 1024u, v_second = v_fill[1] - 1024u;
+      const int k_read_high[KS] = {k_read[0] + 65536, k_read[1] + 65536, k_read[2] + 65536,
+                                   k_read[3] + 65536, k_read[4] + 65536, k_read[5] + 65536,
+                                   k_read[6] + 65536, k_read[7] + 65536};
+      const int v_read_high[DB] = {v_read[0] + 65536, v_read[1] + 65536, v_read[2] + 65536,
+                                   v_read[3] + 65536};
+      asm volatile(FLASH_LOOP_D128_ASM
+                   : FLASH_LOOP_D128_O0(o_acc[0]), FLASH_LOOP_D128_O1(o_acc[1]),
+                     FLASH_LOOP_D128_O2(o_acc[2]), FLASH_LOOP_D128_O3(o_acc[3]),
+                     FLASH_LOOP_D128_L(l_acc), FLASH_LOOP_D128_MUSED(m_used),
+                     FLASH_LOOP_D128_MTRUE(m_true), FLASH_LOOP_D128_THR(threshold),
+                     [iters] "+s"(iterations), [flag] "+s"(flag), [koff] "+s"(k_offset),
+                     [voff] "+s"(v_offset), [tcount] "+s"(steps_done), [vblk] "+s"(v_block),
+                     [idle] "+s"(idle_steps), [m0save] "=&s"(saved_m0), [t0] "=&s"(scalar_temp0),
+                     [t1] "=&s"(scalar_temp1)
+                   : FLASH_LOOP_D128_QF0(qf[0]), FLASH_LOOP_D128_QF1(qf[1]),
+                     FLASH_LOOP_D128_QF2(qf[2]), FLASH_LOOP_D128_QF3(qf[3]),
+                     FLASH_LOOP_D128_QF4(qf[4]), FLASH_LOOP_D128_QF5(qf[5]),
+                     FLASH_LOOP_D128_QF6(qf[6]), FLASH_LOOP_D128_QF7(qf[7]),
+                     FLASH_LOOP_D128_ONES(ones),
+                     FLASH_LOOP_D128_KADDR0_0(k_read[0]), FLASH_LOOP_D128_KADDR0_1(k_read[1]),
+                     FLASH_LOOP_D128_KADDR0_2(k_read[2]), FLASH_LOOP_D128_KADDR0_3(k_read[3]),
+                     FLASH_LOOP_D128_KADDR0_4(k_read[4]), FLASH_LOOP_D128_KADDR0_5(k_read[5]),
+                     FLASH_LOOP_D128_KADDR0_6(k_read[6]), FLASH_LOOP_D128_KADDR0_7(k_read[7]),
+                     FLASH_LOOP_D128_KADDR1_0(k_read_high[0]), FLASH_LOOP_D128_KADDR1_1(k_read_high[1]),
+                     FLASH_LOOP_D128_KADDR1_2(k_read_high[2]), FLASH_LOOP_D128_KADDR1_3(k_read_high[3]),
+                     FLASH_LOOP_D128_KADDR1_4(k_read_high[4]), FLASH_LOOP_D128_KADDR1_5(k_read_high[5]),
+                     FLASH_LOOP_D128_KADDR1_6(k_read_high[6]), FLASH_LOOP_D128_KADDR1_7(k_read_high[7]),
+                     FLASH_LOOP_D128_VADDR0_0(v_read[0]), FLASH_LOOP_D128_VADDR0_1(v_read[1]),
+                     FLASH_LOOP_D128_VADDR0_2(v_read[2]), FLASH_LOOP_D128_VADDR0_3(v_read[3]),
+                     FLASH_LOOP_D128_VADDR1_0(v_read_high[0]), FLASH_LOOP_D128_VADDR1_1(v_read_high[1]),
+                     FLASH_LOOP_D128_VADDR1_2(v_read_high[2]), FLASH_LOOP_D128_VADDR1_3(v_read_high[3]),
+                     FLASH_LOOP_D128_KFILL0(k_fill[0]), FLASH_LOOP_D128_KFILL1(k_second),
+                     FLASH_LOOP_D128_VFILL0(v_fill[0]), FLASH_LOOP_D128_VFILL1(v_second),
+                     FLASH_LOOP_D128_ROWLIM(row_limit_lane),
+                     [krsrc] "s"(k_all), [vrsrc] "s"(v_all), [scale2] "s"(scale2_bits),
+                     [kstep] "s"(k_tile_step), [vstep] "s"(v_tile_step), [ldsw] "s"(lds_wave),
+                     [nblk] "s"(wave_blocks)
+                   : FLASH_LOOP_D128_CLOBBERS);
+    } else {
+      // all four stages within reach of one base register per operand
+      const uint32_t k_second = k_fill[1] - 1024u, v_second = v_fill[1] - 1024u;
+      asm volatile(FLASH_LOOP_D64_ASM
+                   : FLASH_LOOP_D64_O0(o_acc[0]), FLASH_LOOP_D64_O1(o_acc[1]),
+                     FLASH_LOOP_D64_L(l_acc), FLASH_LOOP_D64_MUSED(m_used),
+                     FLASH_LOOP_D64_MTRUE(m_true), FLASH_LOOP_D64_THR(threshold),
+                     [iters] "+s"(iterations), [flag] "+s"(flag), [koff] "+s"(k_offset),
+                     [voff] "+s"(v_offset), [tcount] "+s"(steps_done), [vblk] "+s"(v_block),
+                     [idle] "+s"(idle_steps), [m0save] "=&s"(saved_m0), [t0] "=&s"(scalar_temp0),
+                     [t1] "=&s"(scalar_temp1)
+                   : FLASH_LOOP_D64_QF0(qf[0]), FLASH_LOOP_D64_QF1(qf[1]),
+                     FLASH_LOOP_D64_QF2(qf[2]), FLASH_LOOP_D64_QF3(qf[3]),
+                     FLASH_LOOP_D64_ONES(ones),
+                     FLASH_LOOP_D64_KADDR0_0(k_read[0]), FLASH_LOOP_D64_KADDR0_1(k_read[1]),
+                     FLASH_LOOP_D64_KADDR0_2(k_read[2]), FLASH_LOOP_D64_KADDR0_3(k_read[3]),
+                     FLASH_LOOP_D64_VADDR0_0(v_read[0]), FLASH_LOOP_D64_VADDR0_1(v_read[1]),
+                     FLASH_LOOP_D64_KFILL0(k_fill[0]), FLASH_LOOP_D64_KFILL1(k_second),
+                     FLASH_LOOP_D64_VFILL0(v_fill[0]), FLASH_LOOP_D64_VFILL1(v_second),
+                     FLASH_LOOP_D64_ROWLIM(row_limit_lane),
+                     [krsrc] "s"(k_all), [vrsrc] "s"(v_all), [scale2] "s"(scale2_bits),
+                     [kstep] "s"(k_tile_step), [vstep] "s"(v_tile_step), [ldsw] "s"(lds_wave),
+                     [nblk] "s"(wave_blocks)
+                   : FLASH_LOOP_D64_CLOBBERS);
+    }
   }
   TL(2);
   TL(3);
@@ -266,14 +300,15 @@ flash_forward_pipelined_kernel(FlashForwardArgs a_in, int unit_count, Schedule s
     // the banks.
     unsigned char* rows_out = lds + 2 * kStageBytes + wave * (32 * D * 2);
     TL(6);
-    const int part = lane_here / 16, chunk = lane_here % 16;
+    constexpr int kRowChunks = D / 8, kRowsAtOnce = 64 / kRowChunks;  // 16-byte pieces a row
+    const int part = lane_here / kRowChunks, chunk = lane_here % kRowChunks;
     // every gate load is requested before the first store: a load returns
     // behind the stores issued before it, and those take their time
-    uint32x4 gate_words[8];
+    uint32x4 gate_words[32 / kRowsAtOnce];
     if (a.gate) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int row = wave_q0 + 4 * i + part;
+      for (int i = 0; i < 32 / kRowsAtOnce; ++i) {
+        const int row = wave_q0 + kRowsAtOnce * i + part;
         const uint32_t gate_at =
             row < a.q_rows
                 ? static_cast<uint32_t>(static_cast<long long>(row) * a.gate_row_stride * 2) + chunk * 16
@@ -288,15 +323,15 @@ flash_forward_pipelined_kernel(FlashForwardArgs a_in, int unit_count, Schedule s
         const int chunk = 4 * db + j;
         const uint2 plain = {pack_bf16(o_acc[db][4 * j + 0] * inverse, o_acc[db][4 * j + 1] * inverse),
                              pack_bf16(o_acc[db][4 * j + 2] * inverse, o_acc[db][4 * j + 3] * inverse)};
-        *reinterpret_cast<uint2*>(rows_out + n * (D * 2) + ((chunk ^ (n & 15)) * 16) + 8 * h) = plain;
+        *reinterpret_cast<uint2*>(rows_out + n * (D * 2) + ((chunk ^ (n & (kRowChunks - 1))) * 16) + 8 * h) = plain;
       }
     __builtin_amdgcn_s_waitcnt(0xC07F);
     TL(7);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int r = 4 * i + part;
+    for (int i = 0; i < 32 / kRowsAtOnce; ++i) {
+      const int r = kRowsAtOnce * i + part;
       const uint4 core_bits =
-          *reinterpret_cast<const uint4*>(rows_out + r * (D * 2) + ((chunk ^ (r & 15)) * 16));
+          *reinterpret_cast<const uint4*>(rows_out + r * (D * 2) + ((chunk ^ (r & (kRowChunks - 1))) * 16));
       const int row = wave_q0 + r;
       const bool row_in_range = row < a.q_rows;
       const uint32_t at = row_in_range
@@ -369,11 +404,12 @@ namespace {
 
 struct ScheduleKey {
   int q_rows = -1, kv_rows = 0, start_position = 0, query_heads = 0, group = 0, sequences = 0,
-      compute_units = 0;
+      workgroups = 0,  // resident at once: compute units x workgroups a compute unit
+      tile_rows = 0;   // query rows of a tile
   bool operator==(const ScheduleKey& o) const {
     return q_rows == o.q_rows && kv_rows == o.kv_rows && start_position == o.start_position &&
            query_heads == o.query_heads && group == o.group && sequences == o.sequences &&
-           compute_units == o.compute_units;
+           workgroups == o.workgroups && tile_rows == o.tile_rows;
   }
 };
 
@@ -386,7 +422,7 @@ struct ScheduleKey {
 constexpr int kFixedCost = PLUTO_FIXED_COST;
 
 int tile_cost(const ScheduleKey& k, int q_tile) {
-  const long long last_row = std::min<long long>((q_tile + 1LL) * kRows, k.q_rows) - 1;
+  const long long last_row = std::min<long long>((q_tile + 1LL) * k.tile_rows, k.q_rows) - 1;
   const long long visible = std::min<long long>(k.kv_rows, k.start_position + last_row + 1);
   return static_cast<int>((visible + BN - 1) / BN) + kFixedCost;
 }
@@ -453,11 +489,11 @@ void pack(const std::vector<int>& cost, int lists, std::vector<std::vector<int>>
 // holds, fewer tiles than compute units, an unusual device).
 int build_schedule(const ScheduleKey& k, Schedule& schedule) {
   schedule.slots = 0;
-  const int q_tiles = (k.q_rows + kRows - 1) / kRows;
+  const int q_tiles = (k.q_rows + k.tile_rows - 1) / k.tile_rows;
   const int kv_heads = k.query_heads / k.group;
   const int kv_units = k.sequences * kv_heads;
   const long long items = 1LL * q_tiles * k.sequences * k.query_heads;
-  if (k.compute_units % 8 != 0 || k.compute_units <= 0 || items <= k.compute_units ||
+  if (k.workgroups % 8 != 0 || k.workgroups <= 0 || items <= k.workgroups ||
       items >= kNoItem)
     return 0;
   // Workgroup i runs on XCD i mod 8 and every XCD has its own L2: the heads of
@@ -470,7 +506,7 @@ int build_schedule(const ScheduleKey& k, Schedule& schedule) {
     partitions = kv_units, xcds_each = 8 / kv_units, units_each = 1;
   else
     partitions = 1, xcds_each = 8, units_each = kv_units;
-  const int lists = k.compute_units / 8 * xcds_each;
+  const int lists = k.workgroups / 8 * xcds_each;
   std::vector<int> cost;
   cost.reserve(static_cast<size_t>(units_each) * k.group * q_tiles);
   for (int local = 0; local < units_each * k.group; ++local)
@@ -479,8 +515,8 @@ int build_schedule(const ScheduleKey& k, Schedule& schedule) {
   pack(cost, lists, packed);
   size_t slots = 0;
   for (const auto& list : packed) slots = std::max(slots, list.size());
-  if (slots == 0 || slots * k.compute_units > static_cast<size_t>(kScheduleEntries)) return 0;
-  for (size_t i = 0; i < slots * k.compute_units; ++i) schedule.item[i] = kNoItem;
+  if (slots == 0 || slots * k.workgroups > static_cast<size_t>(kScheduleEntries)) return 0;
+  for (size_t i = 0; i < slots * k.workgroups; ++i) schedule.item[i] = kNoItem;
   for (int p = 0; p < partitions; ++p)
     for (int j = 0; j < lists; ++j) {
       // list j of partition p -> workgroup on XCD x: the partition's XCDs are
@@ -501,13 +537,17 @@ int build_schedule(const ScheduleKey& k, Schedule& schedule) {
       }
     }
   schedule.slots = static_cast<int>(slots);
-  return k.compute_units;
+  return k.workgroups;
 }
 
 }  // namespace
 
-int launch_flash_forward_pipelined(hipStream_t stream, const FlashForwardArgs& a, int sequences) {
-  const long long q_tiles = (a.q_rows + kRows - 1) / kRows;
+int launch_flash_forward_pipelined(hipStream_t stream, const FlashForwardArgs& a, int head_dim,
+                                   int sequences) {
+  if (head_dim != 64 && head_dim != 128) return PLUTO_HIP_EUNSUPPORTED;
+  const int tile_rows = 32 * (head_dim == 128 ? kWaves<128> : kWaves<64>);
+  const int per_compute_unit = head_dim == 128 ? 1 : 2;  // resident workgroups
+  const long long q_tiles = (a.q_rows + tile_rows - 1) / tile_rows;
   const long long units = q_tiles * sequences * (a.query_heads / a.group);
   long long blocks = (units + 7) / 8 * 8 * a.group;
   if (blocks <= 0 || blocks > 0x7fffffffLL) return PLUTO_HIP_EINVAL;
@@ -518,18 +558,26 @@ int launch_flash_forward_pipelined(hipStream_t stream, const FlashForwardArgs& a
   ScheduleKey key;
   key.q_rows = a.q_rows, key.kv_rows = a.kv_rows, key.start_position = a.start_position;
   key.query_heads = a.query_heads, key.group = a.group, key.sequences = sequences;
-  int device = 0;
+  key.tile_rows = tile_rows;
+  int device = 0, compute_units = 0;
   if (hipGetDevice(&device) != hipSuccess ||
-      hipDeviceGetAttribute(&key.compute_units, hipDeviceAttributeMultiprocessorCount, device) !=
+      hipDeviceGetAttribute(&compute_units, hipDeviceAttributeMultiprocessorCount, device) !=
           hipSuccess)
-    key.compute_units = 0;
+    compute_units = 0;
+  key.workgroups = compute_units * per_compute_unit;
   if (!(key == known)) {
     scheduled_blocks = build_schedule(key, schedule);
     known = key;
   }
   if (scheduled_blocks > 0) blocks = scheduled_blocks;
-  flash_forward_pipelined_kernel<128><<<dim3(static_cast<unsigned>(blocks)), 512, 0, stream>>>(
-      a, static_cast<int>(units), schedule);
+  if (head_dim == 128)
+    flash_forward_pipelined_kernel<128>
+        <<<dim3(static_cast<unsigned>(blocks)), 64 * kWaves<128>, 0, stream>>>(
+            a, static_cast<int>(units), schedule);
+  else
+    flash_forward_pipelined_kernel<64>
+        <<<dim3(static_cast<unsigned>(blocks)), 64 * kWaves<64>, 0, stream>>>(
+            a, static_cast<int>(units), schedule);
   return launch_status();
 }
 

@@ -39,8 +39,9 @@ import sys
 class Registers:
     """Vector register map, allocated from v255 downwards."""
 
-    def __init__(self, D):
+    def __init__(self, D, waves):
         self.D = D
+        self.waves = waves
         self.KS = D // 16          # contraction steps of S^T = operand tuples
         self.DB = D // 32          # 32-channel blocks of O^T
         top = 256
@@ -67,7 +68,7 @@ class Registers:
         if self.two_bases:
             self.KADDR.append([take(1, 1) for _ in range(self.KS)])
             self.VADDR.append([take(1, 1) for _ in range(self.DB)])
-        self.loads = 64 * (D // 8) // 512           # 16-byte loads a lane, tensor and tile
+        self.loads = 64 * (D // 8) // (64 * waves)  # 16-byte loads a lane, tensor and tile
         self.KFILL = [take(1, 1) for _ in range(self.loads)]
         self.VFILL = [take(1, 1) for _ in range(self.loads)]
         self.FTMP = [take(1, 1) for _ in range(2 * self.loads)]
@@ -101,8 +102,8 @@ def vt(base, n):
 
 
 class Emitter:
-    def __init__(self, D):
-        self.r = Registers(D)
+    def __init__(self, D, waves):
+        self.r = Registers(D, waves)
         self.lines = []
         self.label_count = 0
         self.lds_queue = []     # destination tuples of LDS reads in flight, oldest first
@@ -506,14 +507,14 @@ def c_string(lines, indent="  "):
                      for line in lines)
 
 
-def render(D):
-    g = Emitter(D)
+def render(D, waves):
+    g = Emitter(D, waves)
     g.build()
     r = g.r
     name = "FLASH_LOOP_D%d" % D
     out = []
-    out.append("// head width %d: %d instructions and labels, vector registers v%d..v255" %
-               (D, len(g.lines), r.lowest))
+    out.append("// head width %d, %d waves a workgroup: %d instructions and labels, vector registers "
+               "v%d..v255" % (D, waves, len(g.lines), r.lowest))
     out.append("#define %s_ASM \\" % name)
     body = c_string(g.lines).split("\n")
     out.append(" \\\n".join(body))
@@ -538,6 +539,7 @@ def render(D):
         define("KFILL%d" % i, '"{v%d}"' % r.KFILL[i])
         define("VFILL%d" % i, '"{v%d}"' % r.VFILL[i])
     define("LOADS", str(r.loads))
+    define("WAVES", str(waves))
     define("MUSED", '"+{v%d}"' % r.MUSED)
     define("MTRUE", '"+{v%d}"' % r.MTRUE)
     define("THR", '"+{v%d}"' % r.THR)
@@ -562,8 +564,8 @@ def main():
     target = sys.argv[1] if len(sys.argv) > 1 else os.path.join(here, "flash_fwd_loop.inc")
     text = ("// Generated by gen_flash_fwd_loop.py; do not edit.  The instruction stream of the\n"
             "// main loop of flash_forward_pipelined_kernel, see the generator for the schedule.\n\n")
-    for D in (128, 64):
-        text += render(D) + "\n"
+    for D, waves in ((128, 8), (64, 4)):
+        text += render(D, waves) + "\n"
     with open(target, "w") as f:
         f.write(text)
 

@@ -291,13 +291,15 @@ def test_config3_prefill_8192(capi, oracle):
     assert_close_bf16(got, out2.float().cpu().numpy(), "config 3 vs fp32-arithmetic kernel")
 
 
-@pytest.mark.parametrize("lengths", [(1024,), (1301,), (1100, 1237)])
+@pytest.mark.parametrize("lengths", [(2048,), (2301,), (2100, 2237)])
 def test_long_prefill_kernels_agree_bit_for_bit(capi, oracle, lengths):
-    # From 1024 rows on the forward at head width 128 runs its eight-wave kernel
-    # (two waves a SIMD one phase apart, 256-row tiles, three LDS stages).  It
-    # walks the keys in the same order with the same arithmetic as the four-wave
-    # kernel, so outputs, statistics and cache must be identical: whole tiles,
-    # a ragged last tile, and a second piece that continues a filled cache.
+    # From 2048 rows on the forward at head width 128 runs its eight-wave kernel
+    # (256-row tiles packed into per-workgroup lists, a hand-scheduled main
+    # loop in which every wave walks its own number of key blocks, four LDS
+    # stages).  It walks the keys in the same order with the same arithmetic as
+    # the four-wave kernel, so outputs, statistics and cache must be identical:
+    # whole tiles, a ragged last tile, and a second piece that continues a
+    # filled cache (a start position that is no multiple of the block size).
     qh, kh, d = 6, 2, 128
     total = sum(lengths)
     kw = dict(query_heads=qh, key_value_heads=kh, head_dim=d, rotary_dim=32, capacity=total)
@@ -307,7 +309,7 @@ def test_long_prefill_kernels_agree_bit_for_bit(capi, oracle, lengths):
     qw, kw_ = dev(values(d, 0.2, 0.3)), dev(values(d, 0.8, 0.4))
     bf = torch.bfloat16
     results = []
-    for mask in (0xffffffff, 0xffffffff & ~capi.PING_PONG):
+    for mask in (0xffffffff, 0xffffffff & ~capi.EIGHT_WAVE):
         cache = capi.KvCache(total, kh, d)
         outs = []
         with capi.only_kernels(mask):

@@ -148,28 +148,30 @@ def test_mfma_heads_of_128(capi, oracle):
     check(capi, oracle, 300, 2, 256, 2, True, seed=12)
 
 
-def test_long_sequences_of_128_wide_heads_take_the_eight_wave_kernel(capi, oracle):
-    # From 1024 rows on the forward at head width 128 runs an eight-wave kernel
-    # (256-row tiles; here with the packed [rows, 3E] layout, several sequences
-    # and heads, and a length that is not a multiple of its tile).  It must
-    # leave exactly what the four-wave kernel leaves, which the oracle pins.
-    T, H, E, B = 1100, 3, 384, 2
+@pytest.mark.parametrize("T, H, E, B", [(2100, 3, 384, 2), (2048, 5, 320, 3), (2301, 2, 128, 9),
+                                        (2048, 12, 768, 6), (4096, 4, 512, 3)])
+def test_long_sequences_take_the_eight_wave_kernel(capi, oracle, T, H, E, B):
+    # From 2048 rows on the forward at head widths 64 and 128 runs an eight-wave
+    # kernel (256-row tiles; here with the packed [rows, 3E] layout, several
+    # sequences and heads, lengths that are not a multiple of its tile, more
+    # and fewer tiles than compute units).  It must leave exactly what the
+    # four-wave kernel leaves, which the oracle pins.
     rng = np.random.default_rng(31)
     host = rng.standard_normal((B * T, 3 * E)).astype(np.float32)
     x = torch.from_numpy(host).cuda().to(torch.bfloat16)
     new = capi.mha_forward(x, T, H)
-    with capi.only_kernels(0xffffffff & ~capi.PING_PONG):
+    with capi.only_kernels(0xffffffff & ~capi.EIGHT_WAVE):
         old = capi.mha_forward(x, T, H)
     torch.cuda.synchronize()
     for a, b in zip(new, old):
         assert torch.equal(a, b)
     # one (sequence, head) against the oracle
     bits = to_bf16_bits(oracle, host)
-    out_bits, maxima, normalizers = oracle.mha_fwd(bits, T, H, oracle.BF16, (1, 2), (2, 3))
+    out_bits, maxima, normalizers = oracle.mha_fwd(bits, T, H, oracle.BF16, (1, 2), (1, 2))
     want = from_bf16_bits(oracle, out_bits)
     D = E // H
     got = new[0].float().cpu().numpy()
-    assert_close_bf16(got[T:, 2 * D:3 * D], want[T:, 2 * D:3 * D], "sequence 1, head 2")
+    assert_close_bf16(got[T:2 * T, D:2 * D], want[T:2 * T, D:2 * D], "sequence 1, head 1")
 
 
 def test_closed_form_two_tokens(capi):
