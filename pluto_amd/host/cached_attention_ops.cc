@@ -199,4 +199,17 @@ Status DeltaNetState::Reset() {
                         "reset Qwen recurrent state");
 }
 
+Status DeltaNetState::Reset(int sequence) {
+  if (sequence < 0 || sequence >= batch_)
+    return InvalidArgumentError(StrCat("no sequence ", sequence, " in a state of ", batch_));
+  for (hip::Buffer* state : {&convolution_state_, &recurrent_state_}) {
+    const size_t each = state->size_bytes() / batch_;
+    RETURN_IF_ERROR(hip::HipStatus(
+        pluto_hip_memset_async(executor_.stream(),
+                               static_cast<char*>(state->data()) + each * sequence, 0, each),
+        "reset one sequence of the Qwen delta-net state"));
+  }
+  return OkStatus();
+}
+
 }  // namespace pluto::llm::cached_attention_ops

@@ -104,6 +104,9 @@ class DeltaNetState final {
                       const float* conv_weight, const float* a_log, const float* dt_bias,
                       const float* norm_weight, void* output);
   Status Reset();
+  // One sequence of the batch back to its initial (zero) state; the others keep
+  // theirs.  Both states are laid out sequence by sequence.
+  Status Reset(int sequence);
 
  private:
   DeltaNetState(hip::Executor& executor, DeltaNetParameters parameters, int batch,

@@ -124,6 +124,8 @@ class BatchedDeltaNetBranch final : public Layer {
 
   int batch() const { return state_->batch(); }
   Status Reset() { return state_->Reset(); }
+  // One sequence back to its initial state, the others untouched.
+  Status Reset(int sequence) { return state_->Reset(sequence); }
 
  private:
   BatchedDeltaNetBranch(hip::Executor& executor,

@@ -38,7 +38,8 @@ def test_every_reference_class_has_cases(runner):
     suites = {name.split(".")[0] for name in listed}
     assert {"AttentionLayerTest", "AttentionOpsTest", "QwenAttentionTest", "SequenceDeltaNetTest",
             "KeyValueCacheTest", "BufferTest", "ExecutorTest", "PageLockedHostArrayTest",
-            "ActivationTypeCpu", "StatusCpu", "LayerHooksTest", "DeltaNetLayerTest"} <= suites
+            "ActivationTypeCpu", "StatusCpu", "LayerHooksTest", "DeltaNetLayerTest",
+            "DecoderBranchTest", "DecoderStepTest"} <= suites
 
 
 @pytest.mark.gpu
