@@ -280,7 +280,7 @@ void RunAgainstTheOracle(MatrixStorage storage, double magnitude, const char* wh
       double square = 0;
       for (float value : want) square += double(value) * value;
       const double rms = std::sqrt(square / want.size());
-      EXPECT_GT(rms, 1e-2);  // rows of order one, not a comparison of zeros
+      EXPECT_GT(rms, 1e-3);  // not a comparison of zeros
       for (int c = 0; c < width; ++c) {
         const double error = std::fabs(double(got[static_cast<size_t>(s) * width + c]) - want[c]);
         // the bf16 bound of the configurations: 2e-2 of |x| + rms
@@ -299,8 +299,8 @@ void RunAgainstTheOracle(MatrixStorage storage, double magnitude, const char* wh
 }
 
 TEST(DecoderStepTest, TwoLayerDecoderFollowsTheOracleChain) {
-  RunAgainstTheOracle(MatrixStorage::kBFloat16, 1.7, "bf16 projections");
-  RunAgainstTheOracle(MatrixStorage::kFp8E4M3, 1.7, "FP8 projections");
+  RunAgainstTheOracle(MatrixStorage::kBFloat16, 6.0, "bf16 projections");
+  RunAgainstTheOracle(MatrixStorage::kFp8E4M3, 6.0, "FP8 projections");
 }
 
 TEST(DecoderStepTest, IdentityFixtureLeavesZeroRows) {
