@@ -148,12 +148,22 @@ def test_config5_chunked_scan(capi, oracle):
     assert capi.last_path() == capi.PATH_CHUNKED
     torch.cuda.synchronize()
     got, got_state = out.float().cpu().numpy(), state.cpu().numpy()
-    # CPU recurrence on whole (sequence, head) chains (they are independent)
-    for b, h in ((0, 3), (1, 12)):
+    # CPU recurrence on every one of the 32 (sequence, head) chains (they are
+    # independent; the oracle's C code runs outside the interpreter lock)
+    import concurrent.futures
+
+    def chain(index):
+        b, h = divmod(index, H)
         core, want_state = oracle.gdn_scan(po, q[b], k[b], v[b], g[b], beta[b], False, scale,
                                            state0[b], (h, h + 1))
-        assert_close_bf16(got[b, :, h], core[:, h], "config 5 seq %d head %d out" % (b, h))
-        assert_close_bf16(got_state[b, h], want_state[h], "config 5 seq %d head %d state" % (b, h))
+        return core[:, h], want_state[h]
+
+    with concurrent.futures.ThreadPoolExecutor(max_workers=16) as pool:
+        chains = list(pool.map(chain, range(B * H)))
+    want = np.stack([c[0] for c in chains]).reshape(B, H, T, vd).transpose(0, 2, 1, 3)
+    want_state = np.stack([c[1] for c in chains]).reshape(B, H, kd, vd)
+    assert_close_bf16(got, want, "config 5 out, all 32 chains")
+    assert_close_bf16(got_state, want_state, "config 5 state, all 32 chains")
     # every chain: against the token-by-token kernel
     state2 = dev(state0.astype(np.float32))
     out2 = capi.gdn_recurrence(p, dq, dk, dv, dg, db, state2, q_scale=scale)

@@ -177,9 +177,10 @@ def test_benchmarked_shape_against_fp32_kernels(capi):
         assert capi.last_path() == capi.PATH_GENERIC
     for name in fast:
         # (fifty million elements: the tail of the per-element error reaches further
-        # than in the small cases; the max-norm bound still holds for every element)
+        # than in the small cases: the farthest observed sits at 19.1 times the
+        # per-element bound; the max-norm bound still holds for every element)
         assert_close_bf16_gradient(fast[name].cpu().numpy(), slow[name].cpu().numpy(),
-                                   "%s T%d vs fp32-arithmetic kernels" % (name, T), far=50.0)
+                                   "%s T%d vs fp32-arithmetic kernels" % (name, T), far=20.0)
 
 
 def test_saved_state_is_refused_where_none_is_kept(capi):

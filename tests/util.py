@@ -69,9 +69,11 @@ def assert_close_bf16(actual, expected, what, rel=2e-2, outliers=1e-4, far=2.0):
     scale = np.abs(expected) + rms
     beyond = int((diff > rel * scale).sum())
     far_beyond = int((diff > far * rel * scale).sum())
+    ratio = float((diff / (rel * scale)).max()) if diff.size else 0.0
     print("%s: max-abs error %.3e (%.2e of max|expected| %.3e), relative L2 error %.2e, "
-          "%d of %d elements beyond %.0e * (|expected| + rms %.3e)" % (
-              what, worst, worst / (peak or 1.0), peak, l2, beyond, diff.size, rel, rms))
+          "%d of %d elements beyond %.0e * (|expected| + rms %.3e), the farthest at %.2f times "
+          "that bound" % (what, worst, worst / (peak or 1.0), peak, l2, beyond, diff.size, rel, rms,
+                          ratio))
     assert beyond <= outliers * diff.size and far_beyond == 0, (
         "%s: %d of %d elements beyond %.1e * (|expected| + rms %.3e), %d beyond %g times that" % (
             what, beyond, diff.size, rel, rms, far_beyond, far))
@@ -89,10 +91,13 @@ def beyond_reference_tolerance(actual, expected, absolute, relative):
     return float(np.mean(np.abs(actual - expected) > absolute + relative * np.abs(expected)))
 
 
-def assert_close_bf16_gradient(actual, expected, what, outliers=2e-3, far=12.0):
+def assert_close_bf16_gradient(actual, expected, what, outliers=2e-3, far=10.0):
     """assert_close_bf16 for gradients of the bf16 attention kernels: dS and P
     are rounded to bf16 before the products that sum them over hundreds of
     rows, so a few elements per thousand miss the per-element bound (measured:
     up to 0.15 % on random inputs; more when the scores are peaked and most
-    gradients are tiny).  Max-norm and L2 bounds are the same 2e-2."""
+    gradients are tiny).  `far` is the worst miss observed, rounded up: over
+    all 192 units of the training configuration the farthest element of dQ sits
+    at 9.03 times the per-element bound (dK 4.4, dV 4.4; every call prints its
+    own figure).  Max-norm and L2 bounds are the same 2e-2."""
     assert_close_bf16(actual, expected, what, outliers=outliers, far=far)
