@@ -11,11 +11,13 @@ D=64.  The default run (--workload all) appends the other four configurations
 of the path under "workloads", each with its own `roofline` and
 `cpu_baseline`; --workload NAME runs one workload alone.
 
-Each workload first runs untimed for --settle-seconds (0.3 s) of continuous
-work, then the W warm-up steps, then the K timed steps: the part reaches the
-clocks it sustains only after some 30 ms of work, and a training or serving
-loop lives in that state (the first 20 steps after an idle period run 10-15 %
-slower in the matrix-core kernels).  `config.settle_s` records the setting.
+Each workload runs its W warm-up steps and times K steps straight after them
+(`first_steps_ms`: the clocks of a part that was idle a moment ago), then runs
+untimed for --settle-seconds (0.3 s) of continuous work and times K steps
+again: `ms_per_step` and `value`.  The part reaches the clocks it sustains only
+after some 30 ms of work, and a training or serving loop lives in that state
+(the first 20 steps after an idle period run 10-15 % slower in the matrix-core
+kernels).  `config.settle_s` records the setting; both figures are in the line.
 
 `ms_per_step` (and `value`) come from HIP events recorded on the launch
 stream just inside the two synchronizations that bracket the K steps;
@@ -23,11 +25,16 @@ stream just inside the two synchronizations that bracket the K steps;
 contains the host's wake-up after the last kernel.
 
 Exactly one JSON line is printed.  `roofline` describes the kernel of the
-step that takes longest: its average duration is measured live with HIP
-events on the launch stream around calls that queue only that kernel (the
-library's measurement hook switches the other kernels of the call off after
-a complete step has filled every buffer), `achieved` is the kernel's
-algorithmic work divided by that duration.  `cpu_baseline` is the scalar CPU
+step that takes longest.  Kernel durations come from one source: K further
+steps in which every kernel group of the step is queued by a call of its own
+(the library's measurement hook switches the other kernels of that call off;
+a complete step has filled every buffer before), in the step's order, with a
+HIP event on the launch stream between the groups.  The groups thus run in the
+thermal state of the step, their durations add up to that split step's
+(`split_step_ms`, a few microseconds of event gaps above `ms_per_step`), and
+none can exceed it.  `achieved` is the kernel's algorithmic work divided by
+its duration; where the step moves more bytes than the algorithm needs
+(`roofline.moved_bytes`, from the counters), `frac_moved` prices those.  `cpu_baseline` is the scalar CPU
 oracle timed on this host on a bounded sample of the same workload, on one
 thread as the reference runs it (`value`, `cores` 1) and on `threads.cores`
 threads over independent units (a reported baseline only).
@@ -52,12 +59,13 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E (published)
 # the factors a 1 GiB device copy gives: `--workload copy`).  The summaries are
 # kept as profiles/*_hbm_traffic.md.  None = not measured.
 MEASURED_TRAFFIC_BYTES = {
-    ("mha_train_bf16", "flash_forward_kernel<64>"): 126.4e6,
-    ("mha_train_bf16", "flash_dq_kernel<64>"): 198.1e6 + 91.3e6,
-    ("mha_train_bf16", "flash_dkv_kernel<64>"): 154.2e6 + 100.7e6,
-    ("gqa_prefill", "flash_forward_pipelined_kernel<128>"): 168.8e6 + 52.8e6,
-    ("gqa_decode", "decode_fused_kernel<128,6>"): 1044.3e6 + 13.0e6,
-    ("gdn_scan", "gdn_chunk_prepare + gdn_chunk_scan"): 1052.6e6,
+    # (workload, kernel group): (bytes, commit the counters were read at)
+    ("mha_train_bf16", "flash_forward_kernel<64>"): (126.4e6, "d8f10f7"),
+    ("mha_train_bf16", "flash_dq_kernel<64>"): (198.1e6 + 91.3e6, "d8f10f7"),
+    ("mha_train_bf16", "flash_dkv_kernel<64>"): (154.2e6 + 100.7e6, "d8f10f7"),
+    ("gqa_prefill", "flash_forward_pipelined_kernel<128>"): None,
+    ("gqa_decode", "decode_fused_kernel<128,6>"): (1044.3e6 + 13.0e6, "d8f10f7"),
+    ("gdn_scan", "gdn_chunk_scan"): None,
 }
 
 NAMES = ["mha_train_bf16", "mha_fwd_fp32", "gqa_prefill", "gqa_decode", "gdn_scan"]
@@ -181,8 +189,8 @@ def gqa_prefill(torch, capi):
 
     work = 4.0 * qh * d * causal_pairs(T)
     return dict(step=step,
-                kernels=[("flash_forward_pipelined_kernel<128>", step, capi.MAIN_KERNEL | capi.EIGHT_WAVE, work),
-                         ("rope table + prepare", step, capi.AUXILIARY_KERNELS, None)],
+                kernels=[("rope table + prepare", step, capi.AUXILIARY_KERNELS, None),
+                         ("flash_forward_pipelined_kernel<128>", step, capi.MAIN_KERNEL | capi.EIGHT_WAVE, work)],
                 work=work,
                 metric="gqa_prefill_tflops", unit="TFLOP/s", dtype="bf16", bound="mfma",
                 peak=PEAK_BF16_TFLOPS,
@@ -296,8 +304,8 @@ def gqa_decode(torch, capi):
 
     work = 2.0 * kh * d * 2 * float(lengths.sum())   # K and V bytes of the valid prefix
     return dict(step=step, graph_outputs=lambda: [out],
-                kernels=[("decode_fused_kernel<128,6>", step, capi.MAIN_KERNEL, work),
-                         ("counter clear", step, capi.AUXILIARY_KERNELS, None)],
+                kernels=[("counter clear", step, capi.AUXILIARY_KERNELS, None),
+                         ("decode_fused_kernel<128,6>", step, capi.MAIN_KERNEL, work)],
                 work=work,
                 metric="gqa_decode_hbm_gbs", unit="GB/s", dtype="bf16", bound="hbm",
                 peak=PEAK_HBM_GBS,
@@ -330,9 +338,15 @@ def gdn_scan(torch, capi):
         state.zero_()
         scan()
 
+    # The sequential kernel bounds the step; it reads K, Q, V, the prepared
+    # per-chunk operands and the state, and writes the outputs and the state.
+    # Priced against the whole step's algorithmic bytes it gives the fraction
+    # of the roofline the step would reach if the preparation were free.
     work = B * T * H * (2 * dk + 2 * dv) * 2.0 + 2.0 * B * T * H * 4 + B * H * dk * dv * 4.0
     return dict(step=step,
-                kernels=[("gdn_chunk_prepare + gdn_chunk_scan", scan, None, work)],
+                kernels=[("state clear", state.zero_, None, None),
+                         ("gdn_chunk_prepare", scan, capi.AUXILIARY_KERNELS, None),
+                         ("gdn_chunk_scan", scan, capi.MAIN_KERNEL, work)],
                 work=work,
                 metric="gated_delta_scan_hbm_gbs", unit="GB/s", dtype="bf16", bound="hbm",
                 peak=PEAK_HBM_GBS,
@@ -755,16 +769,22 @@ def capture_step(torch, w):
 
 def measure(torch, capi, w, steps, warmup, launch="eager", settle_seconds=0.0):
     stream = torch.cuda.current_stream()
-    # The part needs some 30 ms of continuous work to reach the clocks it then
-    # sustains (the matrix-core kernels run 10-15 % slower until then), far more
-    # than a handful of warm-up steps of 0.2 ms: the step first runs untimed
-    # for `settle_seconds`, then come the warm-up steps asked for.
-    settle_until = time.perf_counter() + settle_seconds
-    while time.perf_counter() < settle_until:
-        for _ in range(50):
-            w["step"]()
+
+    def timed(run, count):
+        """`count` calls between two events on the launch stream, themselves just
+        inside two synchronizations: the host's wake-up after the last kernel
+        (tens of microseconds, 5 % of 20 steps of 0.2 ms) is not charged to the
+        steps; the host's own clock over the same bracket is returned too."""
+        first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
-    w["config"]["settle_s"] = settle_seconds
+        t0 = time.perf_counter()
+        first.record(stream)
+        for _ in range(count):
+            run()
+        last.record(stream)
+        torch.cuda.synchronize()
+        return first.elapsed_time(last) / count, (time.perf_counter() - t0) * 1e3 / count
+
     for _ in range(warmup):
         w["step"]()
     torch.cuda.synchronize()
@@ -772,39 +792,44 @@ def measure(torch, capi, w, steps, warmup, launch="eager", settle_seconds=0.0):
     run_step = graph.replay if graph is not None else w["step"]
     w["config"]["launch"] = ("hip graph replay, one per step" if graph is not None
                              else "eager, one launch per kernel")
-    run_step()
-    torch.cuda.synchronize()
-    # The K steps lie between two synchronizations; their duration is read from
-    # HIP events recorded on the launch stream just inside that bracket, so
-    # that the host's wake-up after the last kernel (tens of microseconds, 5 %
-    # of 20 steps of 0.2 ms) is not charged to the steps.  The host's own clock
-    # over the same bracket is kept as `host_ms_per_step`.
-    first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    first.record(stream)
-    for _ in range(steps):
-        run_step()
-    last.record(stream)
-    torch.cuda.synchronize()
-    host_ms_per_step = (time.perf_counter() - t0) * 1e3 / steps
-    ms_per_step = first.elapsed_time(last) / steps
-    # Every buffer now holds what a complete step leaves, so any one kernel of
-    # the step can run alone on valid inputs.
-    kernels = {}
-    for name, fn, mask, work in w["kernels"]:
-        pairs = []
-        with capi.only_kernels(0xffffffff if mask is None else mask):
-            fn()
-            torch.cuda.synchronize()
-            for _ in range(steps):
-                start = torch.cuda.Event(enable_timing=True)
-                end = torch.cuda.Event(enable_timing=True)
-                start.record(stream)
+    # the K steps right after the W warm-up steps: a part that was idle a moment ago
+    first_steps_ms, _ = timed(run_step, steps)
+    # The part needs some 30 ms of continuous work to reach the clocks it then
+    # sustains (the matrix-core kernels run 10-15 % slower until then), far more
+    # than a handful of warm-up steps of 0.2 ms: the step runs untimed for
+    # `settle_seconds`, then the K steps are timed again.
+    settle_until = time.perf_counter() + settle_seconds
+    while time.perf_counter() < settle_until:
+        for _ in range(50):
+            run_step()
+        torch.cuda.synchronize()
+    w["config"]["settle_s"] = settle_seconds
+    ms_per_step, host_ms_per_step = timed(run_step, steps)
+    # Every buffer now holds what a complete step leaves, so any one kernel group
+    # of the step can run alone on valid inputs.  K split steps: the groups in
+    # the step's order, each queued by its own call, an event between them.
+    groups = w["kernels"]
+    marks = [[torch.cuda.Event(enable_timing=True) for _ in range(len(groups) + 1)]
+             for _ in range(steps)]
+
+    def split_step(events):
+        events[0].record(stream)
+        for (name, fn, mask, work), event in zip(groups, events[1:]):
+            with capi.only_kernels(0xffffffff if mask is None else mask):
                 fn()
-                end.record(stream)
-                pairs.append((start, end))
-            torch.cuda.synchronize()
-        kernels[name] = (sum(s.elapsed_time(e) for s, e in pairs) / len(pairs), work)
+            event.record(stream)
+
+    for _ in range(max(3, warmup)):
+        split_step(marks[0])
+    torch.cuda.synchronize()
+    for events in marks:
+        split_step(events)
+    torch.cuda.synchronize()
+    kernels = {}
+    for index, (name, fn, mask, work) in enumerate(groups):
+        mean = sum(e[index].elapsed_time(e[index + 1]) for e in marks) / steps
+        kernels[name] = (mean, work)
+    split_step_ms = marks[0][0].elapsed_time(marks[-1][-1]) / steps
     w["step"]()   # leave complete results behind
     torch.cuda.synchronize()
     counted = {k: v for k, v in kernels.items() if v[1] is not None}
@@ -813,16 +838,34 @@ def measure(torch, capi, w, steps, warmup, launch="eager", settle_seconds=0.0):
     divisor = 1e12 if w["bound"] == "mfma" else 1e9
     value = w["work"] / (ms_per_step * 1e-3) / divisor
     achieved = dom_work / (dom_ms * 1e-3) / divisor
-    return dict(ms_per_step=ms_per_step, host_ms_per_step=host_ms_per_step, value=value,
+    return dict(ms_per_step=ms_per_step, host_ms_per_step=host_ms_per_step,
+                first_steps_ms=first_steps_ms, split_step_ms=split_step_ms, value=value,
                 kernels=kernels, dominant=dominant, achieved=achieved, kernel_ms=dom_ms)
 
 
 def roofline(name, w, m):
-    return {"bound": w["bound"], "kernel": m["dominant"], "achieved": round(m["achieved"], 3),
-            "peak": w["peak"], "unit": "TFLOP/s" if w["bound"] == "mfma" else "GB/s",
-            "frac": round(m["achieved"] / w["peak"], 4),
-            "traffic": MEASURED_TRAFFIC_BYTES.get((name, m["dominant"])),
-            "kernel_ms": round(m["kernel_ms"], 4)}
+    unit = "TFLOP/s" if w["bound"] == "mfma" else "GB/s"
+    line = {"bound": w["bound"], "kernel": m["dominant"], "achieved": round(m["achieved"], 3),
+            "peak": w["peak"], "unit": unit, "frac": round(m["achieved"] / w["peak"], 4),
+            "traffic": None, "kernel_ms": round(m["kernel_ms"], 4)}
+    measured = MEASURED_TRAFFIC_BYTES.get((name, m["dominant"]))
+    if measured is not None:
+        moved, commit = measured
+        line["traffic"] = moved
+        line["traffic_commit"] = commit
+        if w["bound"] == "hbm":
+            # `achieved` and `frac` price the algorithmic bytes; these the bytes moved
+            line["algorithmic_bytes"] = w["work"]
+            line["moved_bytes"] = moved
+            line["frac_moved"] = round(moved / (m["kernel_ms"] * 1e-3) / 1e9 / w["peak"], 4)
+    return line
+
+
+def summary(w, m):
+    return {"ms_per_step": round(m["ms_per_step"], 4),
+            "host_ms_per_step": round(m["host_ms_per_step"], 4),
+            "first_steps_ms": round(m["first_steps_ms"], 4),
+            "split_step_ms": round(m["split_step_ms"], 4)}
 
 
 def main():
@@ -841,8 +884,7 @@ def main():
     m = measure(torch, capi, w, args.steps, args.warmup, args.launch, args.settle_seconds)
     result = {
         "metric": w["metric"], "value": round(m["value"], 3), "unit": w["unit"], "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(m["ms_per_step"], 4),
-        "host_ms_per_step": round(m["host_ms_per_step"], 4),
+        "steps": args.steps, "warmup": args.warmup, **summary(w, m),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": w["dtype"], "data": "synthetic", "config": w["config"],
         "roofline": roofline(head, w, m),
@@ -860,8 +902,7 @@ def main():
             w = WORKLOADS[name](torch, capi)
             mm = measure(torch, capi, w, args.steps, args.warmup, args.launch, args.settle_seconds)
             others[name] = {"metric": w["metric"], "value": round(mm["value"], 3), "unit": w["unit"],
-                            "ms_per_step": round(mm["ms_per_step"], 4),
-                            "host_ms_per_step": round(mm["host_ms_per_step"], 4), "dtype": w["dtype"],
+                            **summary(w, mm), "dtype": w["dtype"],
                             "config": w["config"], "roofline": roofline(name, w, mm),
                             "kernels_ms": {k: round(v[0], 4) for k, v in mm["kernels"].items()}}
             if not args.no_cpu_baseline and w["cpu"] is not None:
