@@ -548,7 +548,11 @@ int pluto_hip_test_force_generic(int enabled);
  * preparation, tables, combines; 16 = not a kernel: with this bit cleared the
  * attention forward at head widths 64 and 128 keeps to its four-wave kernel
  * whatever the sequence length, which lets a test compare it with the
- * eight-wave kernel that long sequences take).  A benchmark
+ * eight-wave kernel that long sequences take, and the key-owned attention
+ * backward at head width 64 keeps to its compiler-scheduled kernel; 32 = not a
+ * kernel either: with this bit cleared (and 16 set) that backward takes its
+ * hand-scheduled kernel at every sequence length instead of from 4096 rows,
+ * which lets a test compare the two bit for bit on small shapes).  A benchmark
  * runs the whole call once, then times one class with events around the call.  Returns the previous mask;
  * the default, ~0u, runs everything.  Thread-local like the switch above, and
  * like it written by nothing on the product path. */

@@ -177,6 +177,7 @@ class force_generic:
 
 MAIN_KERNEL, QUERY_KERNEL, AUXILIARY_KERNELS = 1, 2, 4
 EIGHT_WAVE = 16  # permission bit, not a kernel: see pluto_hip_test_kernel_classes
+FROM_LENGTH = 32  # cleared: hand-scheduled kernels at every length (same header comment)
 (PATH_NONE, PATH_GENERIC, PATH_MATRIX_F32, PATH_FLASH, PATH_SPLIT_K, PATH_CHUNKED,
  PATH_RECURRENCE) = range(7)
 

@@ -107,7 +107,8 @@ enum KernelClass : unsigned {
   kMainKernel = 1u,       // the kernel that bounds the call (flash, split-K, scan ...)
   kQueryKernel = 2u,      // the query-owned half of the attention backward
   kAuxiliaryKernel = 4u,  // preparation, tables, combines
-  kEightWave = 16u,        // not a kernel: the forward may use its eight-wave kernel (hand-scheduled loop)
+  kEightWave = 16u,       // not a kernel: the hand-scheduled kernels may be taken (pipelined forward, wide dK/dV)
+  kFromLength = 32u,      // not a kernel: ... but only from the sequence lengths where they win
 };
 bool kernel_enabled(KernelClass which);  // mha_capi.hip
 // Records the kernel family a compute call chose (pluto_hip_test_last_path).

@@ -35,6 +35,7 @@ constexpr int kThreads = 256;
 // faster unpaired (1554 -> 1177 us for dK/dV and 754 -> 644 us for dQ at
 // T = 8192, 24 heads of 128; 99 -> 94 us for dK/dV at T = 1024, 12 heads of
 // 64, 16 sequences; the 64-wide dQ kernel is 8 % slower unpaired).
+constexpr int kWideFromRows = 4096;
 constexpr bool kDqPaired64 = true;
 constexpr bool kOtherPaired = false;
 
@@ -511,6 +512,11 @@ int launch_flash_backward(hipStream_t stream, const GenericBackwardArgs& a,
   status = launch_status();
   if (status != 0) return status;
   if (!kernel_enabled(kMainKernel)) return 0;
+  // The hand-scheduled kernel (one wave a SIMD, 64 keys a wave) gives the same
+  // bits; it is level with the kernel below at 2048 rows and 6 % ahead at 4096.
+  if (dim == 64 && kernel_enabled(kEightWave) &&
+      (a.context_length >= kWideFromRows || !kernel_enabled(kFromLength)))
+    return launch_flash_dkv_wide(stream, a, lse2, d_out_bf16);
   if (dim == 64)
     flash_dkv_kernel<64, kOtherPaired><<<kOtherPaired ? paired : unpaired, kThreads, 0, stream>>>(
         a, lse2, d_out_bf16);

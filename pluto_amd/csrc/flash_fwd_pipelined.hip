@@ -197,9 +197,9 @@ flash_forward_pipelined_kernel(FlashForwardArgs a_in, int unit_count, Schedule s
                      FLASH_LOOP_D128_O2(o_acc[2]), FLASH_LOOP_D128_O3(o_acc[3]),
                      FLASH_LOOP_D128_L(l_acc), FLASH_LOOP_D128_MUSED(m_used),
                      FLASH_LOOP_D128_MTRUE(m_true), FLASH_LOOP_D128_THR(threshold),
-                     [iters] "+s"(iterations), [flag] "+s"(flag), [koff] "+s"(k_offset),
-                     [voff] "+s"(v_offset), [tcount] "+s"(steps_done), [vblk] "+s"(v_block),
-                     [idle] "+s"(idle_steps), [m0save] "=&s"(saved_m0), [t0] "=&s"(scalar_temp0),
+                     [iters] "+&s"(iterations), [flag] "+&s"(flag), [koff] "+&s"(k_offset),
+                     [voff] "+&s"(v_offset), [tcount] "+&s"(steps_done), [vblk] "+&s"(v_block),
+                     [idle] "+&s"(idle_steps), [m0save] "=&s"(saved_m0), [t0] "=&s"(scalar_temp0),
                      [t1] "=&s"(scalar_temp1)
                    : FLASH_LOOP_D128_QF0(qf[0]), FLASH_LOOP_D128_QF1(qf[1]),
                      FLASH_LOOP_D128_QF2(qf[2]), FLASH_LOOP_D128_QF3(qf[3]),
@@ -232,9 +232,9 @@ flash_forward_pipelined_kernel(FlashForwardArgs a_in, int unit_count, Schedule s
                    : FLASH_LOOP_D64_O0(o_acc[0]), FLASH_LOOP_D64_O1(o_acc[1]),
                      FLASH_LOOP_D64_L(l_acc), FLASH_LOOP_D64_MUSED(m_used),
                      FLASH_LOOP_D64_MTRUE(m_true), FLASH_LOOP_D64_THR(threshold),
-                     [iters] "+s"(iterations), [flag] "+s"(flag), [koff] "+s"(k_offset),
-                     [voff] "+s"(v_offset), [tcount] "+s"(steps_done), [vblk] "+s"(v_block),
-                     [idle] "+s"(idle_steps), [m0save] "=&s"(saved_m0), [t0] "=&s"(scalar_temp0),
+                     [iters] "+&s"(iterations), [flag] "+&s"(flag), [koff] "+&s"(k_offset),
+                     [voff] "+&s"(v_offset), [tcount] "+&s"(steps_done), [vblk] "+&s"(v_block),
+                     [idle] "+&s"(idle_steps), [m0save] "=&s"(saved_m0), [t0] "=&s"(scalar_temp0),
                      [t1] "=&s"(scalar_temp1)
                    : FLASH_LOOP_D64_QF0(qf[0]), FLASH_LOOP_D64_QF1(qf[1]),
                      FLASH_LOOP_D64_QF2(qf[2]), FLASH_LOOP_D64_QF3(qf[3]),

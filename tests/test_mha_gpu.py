@@ -226,6 +226,34 @@ def test_bitwise_repeatable(capi, bf16):
             np.testing.assert_array_equal(a, b)
 
 
+@pytest.mark.parametrize("T,H,B", [(32, 1, 1), (64, 1, 2), (65, 2, 2), (129, 1, 1), (257, 3, 2),
+                                   (1000, 2, 3), (1024, 4, 2), (4096, 2, 1), (4100, 1, 1)])
+def test_hand_scheduled_key_owned_backward_gives_the_same_bits(capi, oracle, T, H, B):
+    """The key-owned backward kernel with the hand-scheduled loop (heads of 64,
+    taken from 4096 rows) against the compiler-scheduled one it replaces there:
+    same products, same reduction order over query blocks, hence the same bits,
+    at every length (the switch below lifts the length threshold) including
+    those that end inside a block of 32 or a tile of 128.  One case of moderate
+    size also goes against the oracle."""
+    E = 64 * H
+    rng = np.random.default_rng(T + H)
+    x = torch.from_numpy(rng.standard_normal((B * T, 3 * E)).astype(np.float32)).cuda().to(torch.bfloat16)
+    d_out = torch.from_numpy(rng.standard_normal((B * T, E)).astype(np.float32)).cuda()
+    out, maxima, normalizers = capi.mha_forward(x, T, H)
+    with capi.only_kernels(0xffffffff & ~capi.FROM_LENGTH):
+        wide = capi.mha_backward(x, out, d_out, maxima, normalizers, T, H)
+    with capi.only_kernels(0xffffffff & ~capi.EIGHT_WAVE):
+        plain = capi.mha_backward(x, out, d_out, maxima, normalizers, T, H)
+    torch.cuda.synchronize()
+    assert torch.isfinite(wide).all()
+    assert torch.equal(wide, plain)
+    if T == 257:
+        want = oracle.mha_bwd(to_bf16_bits(oracle, x.float().cpu().numpy()),
+                              to_bf16_bits(oracle, out.float().cpu().numpy()),
+                              d_out.cpu().numpy(), T, H, oracle.BF16, None, None)
+        assert_close_bf16_gradient(wide.cpu().numpy(), want, "wide dK/dV T%d" % T)
+
+
 @pytest.mark.parametrize("bf16", [False, True])
 def test_probabilities_pass(capi, bf16):
     # attention_test.cc:41-146: rows sum to one, zeros above the diagonal, P.V = out
