@@ -38,6 +38,7 @@ constexpr int BN = 64;  // keys per LDS tile
 // measured on both head widths: level with the four-wave kernel at 2048 rows,
 // 10-15 % ahead from 4096, behind it at 1024 (few, short tiles per workgroup)
 constexpr int kPipelinedFromRows = 2048;
+constexpr int kPipelined256FromRows = 1024;
 
 // Queues the loads of one K tile and one V tile (keys k0..k0+63) into an LDS
 // stage.  Lane l of load i of a wave writes 16 bytes at chunk
@@ -435,12 +436,14 @@ int launch_flash_forward(hipStream_t stream, const FlashForwardArgs& a,
   const dim3 grid(static_cast<unsigned>(blocks));
   const int unit_count = static_cast<int>(units);
   if (!kernel_enabled(kMainKernel)) return 0;
-  // Long sequences at head widths 64 and 128 take the eight-wave kernel with
-  // the hand-scheduled loop (flash_fwd_pipelined.hip): 256-row tiles, which
-  // short sequences do not fill.  Its epilogue addresses a head's rows through
+  // Long sequences take the kernel with the hand-scheduled loop
+  // (flash_fwd_pipelined.hip): tiles of 256 rows (128 at head widths 64 and
+  // 256), which short sequences do not fill.  Its epilogue addresses a head's rows through
   // 32-bit buffer offsets.
-  if ((head_dim == 128 || head_dim == 64) && a.q_rows >= kPipelinedFromRows &&
-      kernel_enabled(kEightWave)) {
+  // (a test lifts the threshold at head width 256 to compare the two kernels on small shapes)
+  const int from_rows = head_dim != 256 ? kPipelinedFromRows
+                        : kernel_enabled(kFromLength) ? kPipelined256FromRows : 1;
+  if (a.q_rows >= from_rows && kernel_enabled(kEightWave)) {
     const long long widest = a.gate ? std::max(a.o_row_stride, a.gate_row_stride) : a.o_row_stride;
     if (a.q_rows * widest * 2 < (1LL << 31) - 4096)
       return launch_flash_forward_pipelined(stream, a, head_dim, sequences);

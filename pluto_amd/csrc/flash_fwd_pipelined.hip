@@ -16,6 +16,7 @@
 // left to do) run the plain loop below, in C++.
 #include "flash_fwd_mfma.h"
 #include "flash_fwd_loop.inc"
+#include "flash_fwd_loop256.inc"
 #ifndef TL
 #define TL(slot) do {} while (0)
 #endif
@@ -49,11 +50,16 @@ struct Schedule {
 // rows, 64 KiB, two workgroups a compute unit, so that one computes while the
 // other waits for its first tiles or writes its output (at 1024 rows a tile's
 // loop is short against those).
+// Head width 256: four waves, 128 rows, one wave a SIMD (448 registers: O^T and
+// Q^T in AGPRs), 128 KiB of stages that hold single blocks of 32 keys, one
+// workgroup a compute unit.
 template <int D>
-constexpr int kWaves = D == 128 ? FLASH_LOOP_D128_WAVES : FLASH_LOOP_D64_WAVES;
+constexpr int kWaves = D == 256 ? FLASH_LOOP_D256_WAVES
+                                : (D == 128 ? FLASH_LOOP_D128_WAVES : FLASH_LOOP_D64_WAVES);
 
 template <int D>
-__global__ void __launch_bounds__(64 * kWaves<D>) __attribute__((amdgpu_waves_per_eu(2, 2)))
+__global__ void __launch_bounds__(64 * kWaves<D>)
+__attribute__((amdgpu_waves_per_eu(D == 256 ? 1 : 2, D == 256 ? 1 : 2)))
 flash_forward_pipelined_kernel(FlashForwardArgs a_in, int unit_count, Schedule schedule) {
   struct Args : FlashForwardArgs {
     int unit_count;
@@ -62,11 +68,14 @@ flash_forward_pipelined_kernel(FlashForwardArgs a_in, int unit_count, Schedule s
   a.unit_count = unit_count;
   constexpr int WAVES = kWaves<D>, KCH = D / 8, KS = D / 16, DB = D / 32;
   constexpr int BM = 32 * WAVES;
-  constexpr int kTileBytes = BN * D * 2, kStageBytes = 2 * kTileBytes, kStages = 4;
-  constexpr int kLoads = BN * KCH / (64 * WAVES);
-  static_assert(D == 128 || D == 64, "the loop text is instantiated for these head widths");
-  static_assert(D == 128 ? (kLoads == FLASH_LOOP_D128_LOADS && kStageBytes == FLASH_LOOP_D128_STAGE_BYTES)
-                         : (kLoads == FLASH_LOOP_D64_LOADS && kStageBytes == FLASH_LOOP_D64_STAGE_BYTES));
+  // keys of a K or V tile in an LDS stage: a tile of 64 at the narrower widths, one block at 256
+  constexpr int kTileKeys = D == 256 ? 32 : BN;
+  constexpr int kTileBytes = kTileKeys * D * 2, kStageBytes = 2 * kTileBytes, kStages = 4;
+  constexpr int kLoads = kTileKeys * KCH / (64 * WAVES);
+  static_assert(D == 256 || D == 128 || D == 64, "the loop text is instantiated for these head widths");
+  static_assert(D == 256 ? (kLoads == FLASH_LOOP_D256_LOADS && kStageBytes == FLASH_LOOP_D256_STAGE_BYTES)
+                : D == 128 ? (kLoads == FLASH_LOOP_D128_LOADS && kStageBytes == FLASH_LOOP_D128_STAGE_BYTES)
+                           : (kLoads == FLASH_LOOP_D64_LOADS && kStageBytes == FLASH_LOOP_D64_STAGE_BYTES));
   __shared__ __attribute__((aligned(1024))) unsigned char lds[kStages * kStageBytes];
 
   const int tid = threadIdx.x;
@@ -148,10 +157,12 @@ flash_forward_pipelined_kernel(FlashForwardArgs a_in, int unit_count, Schedule s
   float m_used = kMasked, m_true = kMasked;
 #pragma unroll
   for (int i = 0; i < 16; ++i) l_acc[i] = 0.0f;
+  if constexpr (D != 256) {  // at 256 the loop statement keeps O^T in AGPRs and hands it out at its end
 #pragma unroll
-  for (int db = 0; db < DB; ++db)
+    for (int db = 0; db < DB; ++db)
 #pragma unroll
-    for (int i = 0; i < 16; ++i) o_acc[db][i] = 0.0f;
+      for (int i = 0; i < 16; ++i) o_acc[db][i] = 0.0f;
+  }
 
   // Blocks of 32 keys this wave walks: up to the last key its last row sees.  A
   // wave's last two blocks may be cut by the causal mask or by the end of the
@@ -168,8 +179,8 @@ flash_forward_pipelined_kernel(FlashForwardArgs a_in, int unit_count, Schedule s
       __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(blocks_of(wave_q0)));
   // Every wave passes the same number of step barriers, the last wave's: a step
   // (two blocks) starts with one.
-  const uint32_t total_steps =
-      __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(blocks_of(q0 + BM - 32)) / 2);
+  const uint32_t total_steps = __builtin_amdgcn_readfirstlane(
+      static_cast<uint32_t>(blocks_of(q0 + BM - 32)) / (D == 256 ? 1 : 2));
   TL(1);
   {
     // ---- the hand-scheduled loop ----------------------------------------------------
@@ -182,7 +193,50 @@ flash_forward_pipelined_kernel(FlashForwardArgs a_in, int unit_count, Schedule s
     uint32_t saved_m0, scalar_temp0, scalar_temp1;
     float threshold = m_used + kLazy;
     const int row_limit_lane = row_limit - 4 * h;
-    if constexpr (D == 128) {
+    if constexpr (D == 256) {
+      // one step a block: the waves with fewer blocks idle for the difference
+      uint32_t idle_256 = __builtin_amdgcn_readfirstlane(total_steps - wave_blocks), block_count = 0;
+      const uint32_t lds_base = __builtin_amdgcn_readfirstlane(lds_address);
+      const uint32_t k_block_step = static_cast<uint32_t>(32 * a.k_row_stride * 2);
+      const uint32_t v_block_step = static_cast<uint32_t>(32 * a.v_row_stride * 2);
+      // load i of a lane lands 1024 i bytes further on in LDS through the
+      // instruction's offset, which also moves its global address: taken out of
+      // the lane's offset again
+      const uint32_t k1 = k_fill[1] - 1024u, k2 = k_fill[2] - 2048u, k3 = k_fill[3] - 3072u;
+      const uint32_t v1 = v_fill[1] - 1024u, v2 = v_fill[2] - 2048u, v3 = v_fill[3] - 3072u;
+      asm volatile(FLASH_LOOP_D256_ASM
+                   : FLASH_LOOP_D256_O0(o_acc[0]), FLASH_LOOP_D256_O1(o_acc[1]),
+                     FLASH_LOOP_D256_O2(o_acc[2]), FLASH_LOOP_D256_O3(o_acc[3]),
+                     FLASH_LOOP_D256_O4(o_acc[4]), FLASH_LOOP_D256_O5(o_acc[5]),
+                     FLASH_LOOP_D256_O6(o_acc[6]), FLASH_LOOP_D256_O7(o_acc[7]),
+                     FLASH_LOOP_D256_L(l_acc), FLASH_LOOP_D256_MUSED(m_used),
+                     FLASH_LOOP_D256_MTRUE(m_true), FLASH_LOOP_D256_THR(threshold),
+                     FLASH_LOOP_D256_QF0(qf[0]), FLASH_LOOP_D256_QF1(qf[1]),
+                     FLASH_LOOP_D256_QF2(qf[2]), FLASH_LOOP_D256_QF3(qf[3]),
+                     FLASH_LOOP_D256_QF4(qf[4]), FLASH_LOOP_D256_QF5(qf[5]),
+                     FLASH_LOOP_D256_QF6(qf[6]), FLASH_LOOP_D256_QF7(qf[7]),
+                     FLASH_LOOP_D256_QF8(qf[8]), FLASH_LOOP_D256_QF9(qf[9]),
+                     FLASH_LOOP_D256_QF10(qf[10]), FLASH_LOOP_D256_QF11(qf[11]),
+                     FLASH_LOOP_D256_QF12(qf[12]), FLASH_LOOP_D256_QF13(qf[13]),
+                     FLASH_LOOP_D256_QF14(qf[14]), FLASH_LOOP_D256_QF15(qf[15]),
+                     [iters] "+&s"(iterations), [flag] "+&s"(flag), [koff] "+&s"(k_offset),
+                     [voff] "+&s"(v_offset), [tcount] "+&s"(steps_done), [bcount] "+&s"(block_count),
+                     [idle] "+&s"(idle_256), [m0save] "=&s"(saved_m0), [t0] "=&s"(scalar_temp0),
+                     [t1] "=&s"(scalar_temp1)
+                   : FLASH_LOOP_D256_ONES(ones),
+                     FLASH_LOOP_D256_KADDR0(k_read[0]), FLASH_LOOP_D256_KADDR1(k_read[1]),
+                     FLASH_LOOP_D256_KADDR2(k_read[2]), FLASH_LOOP_D256_KADDR3(k_read[3]),
+                     FLASH_LOOP_D256_VADDR0(v_read[0]), FLASH_LOOP_D256_VADDR1(v_read[1]),
+                     FLASH_LOOP_D256_KFILL0(k_fill[0]), FLASH_LOOP_D256_KFILL1(k1),
+                     FLASH_LOOP_D256_KFILL2(k2), FLASH_LOOP_D256_KFILL3(k3),
+                     FLASH_LOOP_D256_VFILL0(v_fill[0]), FLASH_LOOP_D256_VFILL1(v1),
+                     FLASH_LOOP_D256_VFILL2(v2), FLASH_LOOP_D256_VFILL3(v3),
+                     FLASH_LOOP_D256_ROWLIM(row_limit_lane),
+                     [krsrc] "s"(k_all), [vrsrc] "s"(v_all), [scale2] "s"(scale2_bits),
+                     [kstep] "s"(k_block_step), [vstep] "s"(v_block_step), [ldsw] "s"(lds_wave),
+                     [ldsbase] "s"(lds_base), [nblk] "s"(wave_blocks)
+                   : FLASH_LOOP_D256_CLOBBERS);
+    } else if constexpr (D == 128) {
       // the second load of a pair lands 1024 bytes further on in LDS through the
       // instruction's offset, which also moves its global address: taken out of
       // the lane's offset again
@@ -544,9 +598,10 @@ int build_schedule(const ScheduleKey& k, Schedule& schedule) {
 
 int launch_flash_forward_pipelined(hipStream_t stream, const FlashForwardArgs& a, int head_dim,
                                    int sequences) {
-  if (head_dim != 64 && head_dim != 128) return PLUTO_HIP_EUNSUPPORTED;
-  const int tile_rows = 32 * (head_dim == 128 ? kWaves<128> : kWaves<64>);
-  const int per_compute_unit = head_dim == 128 ? 1 : 2;  // resident workgroups
+  if (head_dim != 64 && head_dim != 128 && head_dim != 256) return PLUTO_HIP_EUNSUPPORTED;
+  const int tile_rows =
+      32 * (head_dim == 256 ? kWaves<256> : head_dim == 128 ? kWaves<128> : kWaves<64>);
+  const int per_compute_unit = head_dim == 64 ? 2 : 1;  // resident workgroups
   const long long q_tiles = (a.q_rows + tile_rows - 1) / tile_rows;
   const long long units = q_tiles * sequences * (a.query_heads / a.group);
   long long blocks = (units + 7) / 8 * 8 * a.group;
@@ -570,7 +625,11 @@ int launch_flash_forward_pipelined(hipStream_t stream, const FlashForwardArgs& a
     known = key;
   }
   if (scheduled_blocks > 0) blocks = scheduled_blocks;
-  if (head_dim == 128)
+  if (head_dim == 256)
+    flash_forward_pipelined_kernel<256>
+        <<<dim3(static_cast<unsigned>(blocks)), 64 * kWaves<256>, 0, stream>>>(
+            a, static_cast<int>(units), schedule);
+  else if (head_dim == 128)
     flash_forward_pipelined_kernel<128>
         <<<dim3(static_cast<unsigned>(blocks)), 64 * kWaves<128>, 0, stream>>>(
             a, static_cast<int>(units), schedule);

@@ -291,8 +291,10 @@ def test_config3_prefill_8192(capi, oracle):
     assert_close_bf16(got, out2.float().cpu().numpy(), "config 3 vs fp32-arithmetic kernel")
 
 
-@pytest.mark.parametrize("lengths", [(2048,), (2301,), (2100, 2237)])
-def test_long_prefill_kernels_agree_bit_for_bit(capi, oracle, lengths):
+@pytest.mark.parametrize("lengths,d", [((2048,), 128), ((2301,), 128), ((2100, 2237), 128),
+                                       ((1024,), 256), ((1301,), 256), ((1100, 1237), 256),
+                                       ((33,), 256), ((130, 70), 256)])
+def test_long_prefill_kernels_agree_bit_for_bit(capi, oracle, lengths, d):
     # From 2048 rows on the forward at head width 128 runs its eight-wave kernel
     # (256-row tiles packed into per-workgroup lists, a hand-scheduled main
     # loop in which every wave walks its own number of key blocks, four LDS
@@ -300,7 +302,11 @@ def test_long_prefill_kernels_agree_bit_for_bit(capi, oracle, lengths):
     # the four-wave kernel, so outputs, statistics and cache must be identical:
     # whole tiles, a ragged last tile, and a second piece that continues a
     # filled cache (a start position that is no multiple of the block size).
-    qh, kh, d = 6, 2, 128
+    # At head width 256 (the model's own, cached_attention_ops.h:13-22) the same
+    # loop runs with one wave a SIMD, the output accumulators in AGPRs and
+    # single blocks of 32 keys in the LDS stages, from 1024 rows; the short
+    # cases lift that threshold (waves with one, two and three blocks).
+    qh, kh = 6, 2
     total = sum(lengths)
     kw = dict(query_heads=qh, key_value_heads=kh, head_dim=d, rotary_dim=32, capacity=total)
     p, po = both_params(capi, oracle, **kw)
@@ -309,7 +315,8 @@ def test_long_prefill_kernels_agree_bit_for_bit(capi, oracle, lengths):
     qw, kw_ = dev(values(d, 0.2, 0.3)), dev(values(d, 0.8, 0.4))
     bf = torch.bfloat16
     results = []
-    for mask in (0xffffffff, 0xffffffff & ~capi.EIGHT_WAVE):
+    for mask in (0xffffffff & ~capi.FROM_LENGTH if total < 1024 else 0xffffffff,
+                 0xffffffff & ~capi.EIGHT_WAVE):
         cache = capi.KvCache(total, kh, d)
         outs = []
         with capi.only_kernels(mask):
