@@ -71,8 +71,9 @@ MEASURED_TRAFFIC_BYTES = {
 NAMES = ["mha_train_bf16", "mha_fwd_fp32", "gqa_prefill", "gqa_decode", "gdn_scan"]
 # "copy" is a plain device copy of known size: the calibration case for the
 # FETCH_SIZE / WRITE_SIZE counters that `roofline.traffic` is derived from.
-# "gqa_prefill_bwd" and "gdn_layer_bwd" time the two sequence backward passes.
-EXTRA = ["copy", "gqa_prefill_bwd", "gdn_layer_bwd", "gdn_decode", "dense_qkv", "dense_imported",
+# "gqa_prefill_d256" is the prefill shape at head width 256; "gqa_prefill_bwd"
+# and "gdn_layer_bwd" time the two sequence backward passes.
+EXTRA = ["copy", "gqa_prefill_d256", "gqa_prefill_bwd", "gdn_layer_bwd", "gdn_decode", "dense_qkv", "dense_imported",
          "decode_block"]
 
 
@@ -168,10 +169,10 @@ def mha_fwd_fp32(torch, capi):
                 cpu=("mha", dict(B=B, T=T, H=H, D=D, bf16=False, backward=False)))
 
 
-def gqa_prefill(torch, capi):
+def gqa_prefill(torch, capi, d=128):
     import numpy as np
-    T, qh, kh, d = 8192, 24, 4, 128
-    p = capi.attention_params(qh, kh, d, 32, capacity=T)
+    T, qh, kh = 8192, 24, 4
+    p = capi.attention_params(qh, kh, d, 32 if d == 128 else 64, capacity=T)
     gen = torch.Generator(device="cuda").manual_seed(2)
     bf = torch.bfloat16
     qg = (0.5 * torch.randn((T, qh, 2, d), generator=gen, device="cuda")).to(bf)
@@ -190,13 +191,22 @@ def gqa_prefill(torch, capi):
     work = 4.0 * qh * d * causal_pairs(T)
     return dict(step=step,
                 kernels=[("rope table + prepare", step, capi.AUXILIARY_KERNELS, None),
-                         ("flash_forward_pipelined_kernel<128>", step, capi.MAIN_KERNEL | capi.EIGHT_WAVE, work)],
+                         ("flash_forward_pipelined_kernel<%d>" % d, step,
+                          capi.MAIN_KERNEL | capi.EIGHT_WAVE | capi.FROM_LENGTH, work)],
                 work=work,
                 metric="gqa_prefill_tflops", unit="TFLOP/s", dtype="bf16", bound="mfma",
                 peak=PEAK_BF16_TFLOPS,
                 config={"workload": "qwen_gqa_prefill", "batch": 1, "seq_len": T, "query_heads": qh,
-                        "kv_heads": kh, "head_dim": d, "kv_cache": "bf16 [1,4,8192,128], written by the call"},
-                cpu=("gqa_prefill", dict(T=T, qh=qh, kh=kh, d=d)))
+                        "kv_heads": kh, "head_dim": d,
+                        "kv_cache": "bf16 [1,4,8192,%d], written by the call" % d},
+                cpu=("gqa_prefill", dict(T=T, qh=qh, kh=kh, d=d)) if d == 128 else None)
+
+
+def gqa_prefill_d256(torch, capi):
+    """The prefill shape at the head width the model's parameters default to
+    (256, rotary width 64): a row after the headline ones, not part of
+    --workload all."""
+    return gqa_prefill(torch, capi, d=256)
 
 
 def gqa_prefill_bwd(torch, capi):
@@ -595,7 +605,8 @@ def copy(torch, capi):
 
 
 WORKLOADS = {"copy": copy, "gdn_decode": gdn_decode, "decode_block": decode_block, "dense_qkv": dense_qkv, "dense_imported": dense_imported, "mha_train_bf16": mha_train_bf16, "mha_fwd_fp32": mha_fwd_fp32,
-             "gqa_prefill": gqa_prefill, "gqa_prefill_bwd": gqa_prefill_bwd, "gdn_layer_bwd": gdn_layer_bwd,
+             "gqa_prefill": gqa_prefill, "gqa_prefill_d256": gqa_prefill_d256,
+             "gqa_prefill_bwd": gqa_prefill_bwd, "gdn_layer_bwd": gdn_layer_bwd,
              "gqa_decode": gqa_decode,
              "gdn_scan": gdn_scan}
 

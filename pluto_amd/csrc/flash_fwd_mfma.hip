@@ -38,7 +38,7 @@ constexpr int BN = 64;  // keys per LDS tile
 // measured on both head widths: level with the four-wave kernel at 2048 rows,
 // 10-15 % ahead from 4096, behind it at 1024 (few, short tiles per workgroup)
 constexpr int kPipelinedFromRows = 2048;
-constexpr int kPipelined256FromRows = 1024;
+constexpr int kPipelined256FromRows = 256;
 
 // Queues the loads of one K tile and one V tile (keys k0..k0+63) into an LDS
 // stage.  Lane l of load i of a wave writes 16 bytes at chunk

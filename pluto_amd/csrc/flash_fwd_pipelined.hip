@@ -196,6 +196,7 @@ flash_forward_pipelined_kernel(FlashForwardArgs a_in, int unit_count, Schedule s
     if constexpr (D == 256) {
       // one step a block: the waves with fewer blocks idle for the difference
       uint32_t idle_256 = __builtin_amdgcn_readfirstlane(total_steps - wave_blocks), block_count = 0;
+      uint32_t scalar_temp2;
       const uint32_t lds_base = __builtin_amdgcn_readfirstlane(lds_address);
       const uint32_t k_block_step = static_cast<uint32_t>(32 * a.k_row_stride * 2);
       const uint32_t v_block_step = static_cast<uint32_t>(32 * a.v_row_stride * 2);
@@ -222,7 +223,7 @@ flash_forward_pipelined_kernel(FlashForwardArgs a_in, int unit_count, Schedule s
                      [iters] "+&s"(iterations), [flag] "+&s"(flag), [koff] "+&s"(k_offset),
                      [voff] "+&s"(v_offset), [tcount] "+&s"(steps_done), [bcount] "+&s"(block_count),
                      [idle] "+&s"(idle_256), [m0save] "=&s"(saved_m0), [t0] "=&s"(scalar_temp0),
-                     [t1] "=&s"(scalar_temp1)
+                     [t1] "=&s"(scalar_temp1), [t2] "=&s"(scalar_temp2)
                    : FLASH_LOOP_D256_ONES(ones),
                      FLASH_LOOP_D256_KADDR0(k_read[0]), FLASH_LOOP_D256_KADDR1(k_read[1]),
                      FLASH_LOOP_D256_KADDR2(k_read[2]), FLASH_LOOP_D256_KADDR3(k_read[3]),

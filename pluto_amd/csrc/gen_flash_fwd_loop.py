@@ -268,7 +268,7 @@ class Emitter:
 
     # ---- one iteration -----------------------------------------------------------------
     def iteration(self, parity, scores=True, accumulate=True, softmax=True, v_from=None,
-                  k_from=None, drain_address=None, out_of_line=None, masked=False):
+                  k_from=None, drain_address=None, out_of_line=None, masked=False, requests=()):
         """Block b with b % 2 == parity.  scores: S^T(b+1) into S[1 - parity] from
         the K operands in OP.  accumulate: block b-1 from PF[1 - parity] and the
         V^T operands read here from v_from = (stage, half).  k_from: where the K
@@ -299,7 +299,9 @@ class Emitter:
                 self.v_read(j, v_from[0] if v_from else 0, v_from[1] if v_from else 0,
                             drain_address)
         at = 0
-        for slot in slots:
+        requests = list(requests)
+        stride = max(1, (len(slots) - 1) // max(len(requests), 1))
+        for number, slot in enumerate(slots, 1):
             if slot[0] == "S":
                 ks = slot[1]
                 self.wait_for(("op", ks))
@@ -327,6 +329,12 @@ class Emitter:
             for text in items[at:at + per_slot]:
                 self.emit(text)
             at += per_slot
+            if requests and number % stride == 0:
+                self.emit(requests.pop(0))
+        for text in requests:
+            self.emit(text)
+            if text.startswith("s_add_u32 m0"):
+                self.emit("s_nop 0")
         for text in items[at:]:
             self.emit(text)
         if softmax and accumulate:
@@ -336,10 +344,15 @@ class Emitter:
             self.emit("%s:" % back)
             out_of_line.append(("rescale", rescale_label, back))
 
-    def step_barrier(self):
+    def step_barrier(self, spread=False):
         """The barrier that starts step t (before odd iteration 2t-1): unit t has
         landed for every wave, everyone is done with unit t-2, whose stage takes
-        unit t+2.  The stage is computed, so the same text serves every place."""
+        unit t+2.  The stage is computed, so the same text serves every place.
+        With `spread` the requests are returned instead of emitted, for the
+        iteration that follows to deal out between its matrix instructions: the
+        waves of a workgroup leave the barrier together, and requests issued
+        there queue behind each other at the compute unit's one address path
+        while nothing else is issued."""
         r = self.r
         n = r.loads
         e = self.emit
@@ -355,17 +368,23 @@ class Emitter:
         for i in range(n):
             e("v_add_u32 v%d, %%[voff], v%d" % (r.FTMP[n + i], r.VFILL[i]))
         e("s_mov_b32 m0, %[t0]")
-        e("s_nop 0")
-        for i in range(n):
-            e("buffer_load_dwordx4 v%d, %%[krsrc], 0 offen%s lds" %
-              (r.FTMP[i], " offset:%d" % (1024 * i) if i else ""))
-        e("s_add_u32 m0, %%[t0], %d" % r.tile_bytes())
-        e("s_nop 0")
-        for i in range(n):
-            e("buffer_load_dwordx4 v%d, %%[vrsrc], 0 offen%s lds" %
-              (r.FTMP[n + i], " offset:%d" % (1024 * i) if i else ""))
         e("s_add_u32 %[koff], %[koff], %[kstep]")
         e("s_add_u32 %[voff], %[voff], %[vstep]")
+        requests = []
+        for i in range(n):
+            requests.append("buffer_load_dwordx4 v%d, %%[krsrc], 0 offen%s lds" %
+                            (r.FTMP[i], " offset:%d" % (1024 * i) if i else ""))
+        requests.append("s_add_u32 m0, m0, %d" % r.tile_bytes())
+        for i in range(n):
+            requests.append("buffer_load_dwordx4 v%d, %%[vrsrc], 0 offen%s lds" %
+                            (r.FTMP[n + i], " offset:%d" % (1024 * i) if i else ""))
+        if spread:
+            return requests
+        for text in requests:
+            e(text)
+            if text.startswith("s_add_u32 m0"):
+                e("s_nop 0")
+        return []
 
     def last_block_setup(self, masked):
         """Before one of a wave's last iterations, which read V^T of block
@@ -430,9 +449,9 @@ class Emitter:
             e("s_cbranch_scc1 %s" % (pre_odd if b % 2 else pre_even))
             if b % 2:
                 # odd iteration 2t-1: unit t-1 holds V(t-1) and K(t)
-                self.step_barrier()
+                requests = self.step_barrier(spread=True)
                 self.iteration(1, v_from=((t - 1) % 4, 0), k_from=((t - 1) % 4, 1),
-                               out_of_line=out_of_line)
+                               out_of_line=out_of_line, requests=requests)
             else:
                 # even iteration 2t: V(t-1) second half; K(t+1) first half (unit t)
                 self.iteration(0, v_from=((t - 1) % 4, 1), k_from=(t % 4, 0),

@@ -148,50 +148,64 @@ class Emitter:
                       (vt(r.OP[j] + 2, 2), base, offset + 8 * ROW_BYTES), ("op", j))
 
     # ---- global -> LDS ----------------------------------------------------------------------------
-    def request(self, stage=None, k_part=True, v_part=True):
+    def request(self, stage=None, k_part=True, v_part=True, spread=False):
         """K rows at byte offset %[koff], V rows at %[voff] into a stage (a number,
-        or the byte offset in %[t0]).  The running offsets are added into the
-        lanes' (a descriptor's range check sees the vector offset only); their
-        updates sit between a write of M0 and the request that reads it."""
+        or the byte offset in %[t2]).  The running offsets are added into the
+        lanes' (a descriptor's range check sees the vector offset only).  Returns
+        the requests themselves when `spread` (the caller deals them out between
+        its matrix instructions: four waves that issue eight requests each right
+        after a barrier queue behind each other at the compute unit's one
+        address path for 500 cycles), else emits them.  A write of M0 and the
+        request that reads it are never adjacent."""
         r = self.r
         e = self.emit
         if k_part:
             for i in range(LOADS):
                 e("v_add_u32 v%d, %%[koff], v%d" % (r.FTMP[i], r.KFILL[i]))
+            e("s_add_u32 %[koff], %[koff], %[kstep]")
         if v_part:
             for i in range(LOADS):
                 e("v_add_u32 v%d, %%[voff], v%d" % (r.FTMP[LOADS + i], r.VFILL[i]))
+            e("s_add_u32 %[voff], %[voff], %[vstep]")
+        out = []
         if k_part:
             if stage is None:
-                e("s_add_u32 m0, %[ldsw], %[t0]")
+                out.append("s_add_u32 m0, %[ldsw], %[t2]")
             else:
-                e("s_add_u32 m0, %%[ldsw], %d" % (stage * STAGE_BYTES))
-            e("s_add_u32 %[koff], %[koff], %[kstep]")
+                out.append("s_add_u32 m0, %%[ldsw], %d" % (stage * STAGE_BYTES))
             for i in range(LOADS):
-                e("buffer_load_dwordx4 v%d, %%[krsrc], 0 offen%s lds" %
-                  (r.FTMP[i], " offset:%d" % (1024 * i) if i else ""))
+                out.append("buffer_load_dwordx4 v%d, %%[krsrc], 0 offen%s lds" %
+                           (r.FTMP[i], " offset:%d" % (1024 * i) if i else ""))
         if v_part:
             if stage is None:
-                e("s_add_u32 m0, %%[t0], %d" % BLOCK_BYTES)
-                e("s_add_u32 m0, m0, %[ldsw]")
+                if k_part:
+                    out.append("s_add_u32 m0, m0, %d" % BLOCK_BYTES)
+                else:
+                    out.append("s_add_u32 m0, %%[t2], %d\n\ts_add_u32 m0, m0, %%[ldsw]" % BLOCK_BYTES)
             else:
-                e("s_add_u32 m0, %%[ldsw], %d" % (stage * STAGE_BYTES + BLOCK_BYTES))
-            e("s_add_u32 %[voff], %[voff], %[vstep]")
+                out.append("s_add_u32 m0, %%[ldsw], %d" % (stage * STAGE_BYTES + BLOCK_BYTES))
             for i in range(LOADS):
-                e("buffer_load_dwordx4 v%d, %%[vrsrc], 0 offen%s lds" %
-                  (r.FTMP[LOADS + i], " offset:%d" % (1024 * i) if i else ""))
+                out.append("buffer_load_dwordx4 v%d, %%[vrsrc], 0 offen%s lds" %
+                           (r.FTMP[LOADS + i], " offset:%d" % (1024 * i) if i else ""))
+        if spread:
+            return out
+        for text in out:
+            e(text)
+            if text.startswith("s_add_u32 m0"):
+                e("s_nop 0")
+        return []
 
-    def step_barrier(self, outstanding=2 * 2 * LOADS):
+    def step_barrier(self, outstanding=2 * 2 * LOADS, spread=False):
         """Starts step s = tcount: unit s-1 has landed for every wave, everyone is
         done with unit s-2, whose stage takes unit s+2."""
         e = self.emit
         e("s_waitcnt vmcnt(%d)" % outstanding)
         e("s_barrier")
-        e("s_add_u32 %[t0], %[tcount], 2")
-        e("s_and_b32 %%[t0], %%[t0], %d" % (STAGES - 1))
-        e("s_mul_i32 %%[t0], %%[t0], %d" % STAGE_BYTES)
-        self.request()
+        e("s_add_u32 %[t2], %[tcount], 2")
+        e("s_and_b32 %%[t2], %%[t2], %d" % (STAGES - 1))
+        e("s_mul_i32 %%[t2], %%[t2], %d" % STAGE_BYTES)
         e("s_add_u32 %[tcount], %[tcount], 1")
+        return self.request(spread=spread)
 
     def stage_addresses(self, k_part=True, v_part=True):
         """Read addresses of unit tcount - 2 (the step just started is tcount - 1)."""
@@ -281,7 +295,8 @@ class Emitter:
         e("s_branch %s" % resume_label)
 
     # ---- one iteration ---------------------------------------------------------------------------------------
-    def iteration(self, parity, scores, accumulate, softmax, masked, read_k, out_of_line):
+    def iteration(self, parity, scores, accumulate, softmax, masked, read_k, out_of_line,
+                  requests=()):
         """Block b with b % 2 == parity.  scores: S^T(b+1) into S[1 - parity] from the
         K operands in OP.  accumulate: block b-1 from PF[1 - parity] and the V^T
         operands read here.  read_k: fetch the K operands of block b+2.  Both
@@ -299,16 +314,23 @@ class Emitter:
             rare, resume = self.label("rare"), self.label("resume")
             items = self.softmax_items(parity, rare, resume, masked)
             out_of_line.append(("rare", rare, resume))
+        requests = list(requests)
         if not slots:
+            for text in requests:
+                self.emit(text)
+                if text.startswith("s_add_u32 m0"):
+                    self.emit("s_nop 0")
             for text in items:
                 self.emit(text)
             return
         per_slot = (len(items) + len(slots) - 1) // len(slots)
+        # one request every `stride` matrix instructions, from the second on
+        stride = max(1, (len(slots) - 1) // max(len(requests), 1))
         if not scores and accumulate:
             for j in range(KS):
                 self.v_read(j)
         at_item = 0
-        for slot in slots:
+        for number, slot in enumerate(slots, 1):
             if slot[0] == "S":
                 ks = slot[1]
                 self.wait_for(("op", ks))
@@ -336,6 +358,12 @@ class Emitter:
             for text in items[at_item:at_item + per_slot]:
                 self.emit(text)
             at_item += per_slot
+            if requests and number % stride == 0:
+                self.emit(requests.pop(0))
+        for text in requests:
+            self.emit(text)
+            if text.startswith("s_add_u32 m0"):
+                self.emit("s_nop 0")
         for text in items[at_item:]:
             self.emit(text)
         if softmax and accumulate:
@@ -394,10 +422,10 @@ class Emitter:
         e("s_cmp_eq_u32 %[nblk], 1")
         e("s_cbranch_scc1 %s" % one)
         # iteration 0: softmax(0), S^T(1); K operands of block 2
-        self.step_barrier()
+        requests = self.step_barrier(spread=True)
         self.stage_addresses(v_part=False)
         self.set_limit()
-        self.iteration(0, True, False, True, True, True, out_of_line)
+        self.iteration(0, True, False, True, True, True, out_of_line, requests=requests)
         e("s_mov_b32 %[flag], 0")   # a reference point that moved before anything was accumulated
         e("s_mov_b32 %[bcount], 1")
         e("s_cmp_eq_u32 %[nblk], 2")
@@ -408,9 +436,9 @@ class Emitter:
         for parity in (1, 0):
             e("s_cmp_eq_u32 %[iters], 0")
             e("s_cbranch_scc1 %s" % tail[parity])
-            self.step_barrier()
+            requests = self.step_barrier(spread=True)
             self.stage_addresses()
-            self.iteration(parity, True, True, True, False, True, out_of_line)
+            self.iteration(parity, True, True, True, False, True, out_of_line, requests=requests)
             e("s_sub_u32 %[iters], %[iters], 1")
             e("s_add_u32 %[bcount], %[bcount], 1")
             assert self.lds_queue == at_loop_top, (self.lds_queue, at_loop_top)
@@ -420,23 +448,23 @@ class Emitter:
             e("%s:" % tail[p])
             self.lds_queue = list(at_loop_top)
             # block nblk - 2: S^T of the last block, no further K operands
-            self.step_barrier()
+            requests = self.step_barrier(spread=True)
             self.stage_addresses()
             self.set_limit()
-            self.iteration(p, True, True, True, True, False, out_of_line)
+            self.iteration(p, True, True, True, True, False, out_of_line, requests=requests)
             e("s_add_u32 %[bcount], %[bcount], 1")
             assert self.lds_queue == []
             e("%s:" % last[1 - p])
             # block nblk - 1 (parity 1 - p): softmax and the products of block nblk - 2
-            self.step_barrier()
+            requests = self.step_barrier(spread=True)
             self.stage_addresses(k_part=False)
             self.set_limit()
-            self.iteration(1 - p, False, True, True, True, False, out_of_line)
+            self.iteration(1 - p, False, True, True, True, False, out_of_line, requests=requests)
             # the products of block nblk - 1
-            self.step_barrier()
+            requests = self.step_barrier(spread=True)
             self.stage_addresses(k_part=False)
             e("s_nop 7")
-            self.iteration(p, False, True, False, False, False, out_of_line)
+            self.iteration(p, False, True, False, False, False, out_of_line, requests=requests)
             assert self.lds_queue == []
             e("s_branch %s" % idle)
         # a wave with two blocks: block 1 is its last (the K operands requested for a
@@ -451,10 +479,10 @@ class Emitter:
         self.step_barrier()
         self.set_limit()
         self.iteration(0, False, False, True, True, False, out_of_line)
-        self.step_barrier()
+        requests = self.step_barrier(spread=True)
         self.stage_addresses(k_part=False)
         e("s_nop 7")
-        self.iteration(1, False, True, False, False, False, out_of_line)
+        self.iteration(1, False, True, False, False, False, out_of_line, requests=requests)
         # the steps the slowest wave still has to take: barriers and requests only
         e("%s:" % idle)
         again, finished = "Lidle_again_%=", "Lfinished_%="

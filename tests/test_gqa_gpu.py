@@ -304,7 +304,7 @@ def test_long_prefill_kernels_agree_bit_for_bit(capi, oracle, lengths, d):
     # filled cache (a start position that is no multiple of the block size).
     # At head width 256 (the model's own, cached_attention_ops.h:13-22) the same
     # loop runs with one wave a SIMD, the output accumulators in AGPRs and
-    # single blocks of 32 keys in the LDS stages, from 1024 rows; the short
+    # single blocks of 32 keys in the LDS stages, from 256 rows; the short
     # cases lift that threshold (waves with one, two and three blocks).
     qh, kh = 6, 2
     total = sum(lengths)
@@ -315,7 +315,7 @@ def test_long_prefill_kernels_agree_bit_for_bit(capi, oracle, lengths, d):
     qw, kw_ = dev(values(d, 0.2, 0.3)), dev(values(d, 0.8, 0.4))
     bf = torch.bfloat16
     results = []
-    for mask in (0xffffffff & ~capi.FROM_LENGTH if total < 1024 else 0xffffffff,
+    for mask in (0xffffffff & ~capi.FROM_LENGTH if total < 256 else 0xffffffff,
                  0xffffffff & ~capi.EIGHT_WAVE):
         cache = capi.KvCache(total, kh, d)
         outs = []
