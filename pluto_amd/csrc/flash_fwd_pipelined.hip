@@ -1,25 +1,23 @@
-// Causal flash attention forward for long bf16 sequences on gfx950: the
-// kernel whose main loop is a hand-scheduled instruction stream.
+// Causal flash attention forward for bf16 sequences on gfx950: the kernel
+// whose main loop is a hand-scheduled instruction stream.
 //
 // Same mathematics, operand layouts and results as flash_forward_kernel
 // (flash_fwd_mfma.hip; semantics of FlashAttentionForwardKernel,
 // src/llm/layers/attention.cc:98-170, and with the gate epilogue of
 // ForwardKernel, src/llm/layers/qwen_attention.cc:68-119).  What differs is who
-// orders the instructions.  A workgroup of eight waves owns 256 query rows,
-// 32 a wave.  The key tiles every one of those rows sees whole (all but the
-// last 256 keys of the causal range) are processed by ONE asm statement,
-// flash_fwd_loop.inc, written by gen_flash_fwd_loop.py: per 32-key block a
-// wave issues the S^T products of the next block, the softmax arithmetic of
-// the current one and the O^T products of the previous one interleaved
-// instruction by instruction, with its own LDS reads and waits, on fixed
-// registers.  The tiles that cross the diagonal (masks, waves with nothing
-// left to do) run the plain loop below, in C++.
+// orders the instructions.  A wave owns 32 query rows; all the key blocks it
+// sees, the ones the causal mask or the end of the keys cuts included, are
+// processed by ONE asm statement (flash_fwd_loop.inc for head widths 64 and
+// 128, flash_fwd_loop256.inc for 256, written by gen_flash_fwd_loop*.py): per
+// 32-key block a wave issues the S^T products of the next block, the softmax
+// arithmetic of the current one and the O^T products of the previous one
+// interleaved instruction by instruction, with its own LDS reads, waits and
+// global->LDS requests, on fixed registers.  Around the statement this file
+// loads Q, writes the output (through LDS, whole rows) and the row statistics,
+// and walks the list of tiles the launcher packed for the workgroup.
 #include "flash_fwd_mfma.h"
 #include "flash_fwd_loop.inc"
 #include "flash_fwd_loop256.inc"
-#ifndef TL
-#define TL(slot) do {} while (0)
-#endif
 #include "mfma_tile.h"
 
 #include <algorithm>
@@ -105,7 +103,6 @@ flash_forward_pipelined_kernel(FlashForwardArgs a_in, int unit_count, Schedule s
     head = (kv_unit % kv_heads) * a.group + slot % a.group;
     seq = kv_unit / kv_heads;
   }
-  TL(0);
   const int kv_head = head / a.group;
   const uint16_t* q_base = a.q + seq * a.q_seq_stride + head * a.q_head_stride;
   const uint16_t* k_base = a.k + seq * a.k_seq_stride + kv_head * a.k_head_stride;
@@ -181,7 +178,6 @@ flash_forward_pipelined_kernel(FlashForwardArgs a_in, int unit_count, Schedule s
   // (two blocks) starts with one.
   const uint32_t total_steps = __builtin_amdgcn_readfirstlane(
       static_cast<uint32_t>(blocks_of(q0 + BM - 32)) / (D == 256 ? 1 : 2));
-  TL(1);
   {
     // ---- the hand-scheduled loop ----------------------------------------------------
     const uint32_t k_tile_step = static_cast<uint32_t>(BN * a.k_row_stride * 2);
@@ -306,8 +302,6 @@ flash_forward_pipelined_kernel(FlashForwardArgs a_in, int unit_count, Schedule s
                    : FLASH_LOOP_D64_CLOBBERS);
     }
   }
-  TL(2);
-  TL(3);
   // ---- epilogue ------------------------------------------------------------------
   // The arithmetic of flash_forward_kernel's epilogue.  Every access goes
   // through a bounds-checked buffer descriptor instead of a branch: rows past
@@ -339,9 +333,6 @@ flash_forward_pipelined_kernel(FlashForwardArgs a_in, int unit_count, Schedule s
         const_cast<uint16_t*>(gate_base), 0,
         static_cast<int>(static_cast<long long>(a.q_rows - 1) * a.gate_row_stride * 2 + D * 2),
         0x00020000);
-#ifdef PLUTO_ABLATE_EPILOGUE
-    if (a.scale > 1e30f)
-#endif
     {
     const float l_used = l_acc[0] > 0.0f ? l_acc[0] : 1.0f;
     const float inverse = 1.0f / l_used;
@@ -354,7 +345,6 @@ flash_forward_pipelined_kernel(FlashForwardArgs a_in, int unit_count, Schedule s
     // Chunk c of row r sits at slot c ^ (r & 15): both directions spread over
     // the banks.
     unsigned char* rows_out = lds + 2 * kStageBytes + wave * (32 * D * 2);
-    TL(6);
     constexpr int kRowChunks = D / 8, kRowsAtOnce = 64 / kRowChunks;  // 16-byte pieces a row
     const int part = lane_here / kRowChunks, chunk = lane_here % kRowChunks;
     // every gate load is requested before the first store: a load returns
@@ -381,7 +371,6 @@ flash_forward_pipelined_kernel(FlashForwardArgs a_in, int unit_count, Schedule s
         *reinterpret_cast<uint2*>(rows_out + n * (D * 2) + ((chunk ^ (n & (kRowChunks - 1))) * 16) + 8 * h) = plain;
       }
     __builtin_amdgcn_s_waitcnt(0xC07F);
-    TL(7);
 #pragma unroll
     for (int i = 0; i < 32 / kRowsAtOnce; ++i) {
       const int r = kRowsAtOnce * i + part;
@@ -438,15 +427,6 @@ flash_forward_pipelined_kernel(FlashForwardArgs a_in, int unit_count, Schedule s
     }
     }
   }
-  TL(4);
-#ifdef PLUTO_TIMELINE
-  {
-    const tl_u32x2 tl_v = {static_cast<unsigned>(total_steps), 0u};
-    __builtin_amdgcn_raw_buffer_store_b64(
-        tl_v, __builtin_amdgcn_make_buffer_rsrc(timeline, 0, 4096 * 8 * 8, 0x00020000),
-        threadIdx.x == 0 ? ((blockIdx.x * 4 + entry) * 8 + 5) * 8 : 0x7fffffff, 0, 0);
-  }
-#endif
   // the next tile's fills must not overtake this tile's last LDS reads
   __syncthreads();
   }
@@ -471,10 +451,7 @@ struct ScheduleKey {
 // Cost of a query tile in key tiles: those it walks plus a fixed part (fills
 // in flight before the first product, the epilogue, the end-of-tile barriers)
 // that was measured at seven to eleven key tiles' time.
-#ifndef PLUTO_FIXED_COST
-#define PLUTO_FIXED_COST 8
-#endif
-constexpr int kFixedCost = PLUTO_FIXED_COST;
+constexpr int kFixedCost = 8;
 
 int tile_cost(const ScheduleKey& k, int q_tile) {
   const long long last_row = std::min<long long>((q_tile + 1LL) * k.tile_rows, k.q_rows) - 1;
