@@ -546,15 +546,14 @@ int pluto_hip_test_force_generic(int enabled);
  * attention forward, key-owned attention backward, split-K decode, delta-net
  * scan; 2 = the query-owned attention backward kernel; 4 = auxiliary kernels:
  * preparation, tables, combines; 16 = not a kernel: with this bit cleared the
- * attention forward at head widths 64, 128 and 256 keeps to its four-wave kernel
- * whatever the sequence length, which lets a test compare it with the
- * eight-wave kernel that long sequences take, and the key-owned attention
- * backward at head width 64 keeps to its compiler-scheduled kernel; 32 = not a
- * kernel either: with this bit cleared (and 16 set) that backward takes its
- * hand-scheduled kernel at every sequence length instead of from 4096 rows,
- * and the attention forward at head width 256 its own instead of from 256
- * rows, which lets a test compare each with the kernel it replaces, bit for
- * bit, on small shapes).  A benchmark
+ * attention forward and the key-owned attention backward keep to their
+ * compiler-scheduled kernels whatever the sequence length, which lets a test
+ * compare those with the kernels with hand-scheduled loops that longer
+ * sequences take (forward: from 2048 rows at head widths 64 and 128, from 256
+ * rows at 256; backward: from 4096 rows at head width 64); 32 = not a kernel
+ * either: with this bit cleared (and 16 set) the backward and the forward at
+ * head width 256 take their hand-scheduled kernels at every sequence length,
+ * which extends that comparison, bit for bit, to small shapes).  A benchmark
  * runs the whole call once, then times one class with events around the call.  Returns the previous mask;
  * the default, ~0u, runs everything.  Thread-local like the switch above, and
  * like it written by nothing on the product path. */

@@ -149,13 +149,15 @@ def test_mfma_heads_of_128(capi, oracle):
 
 
 @pytest.mark.parametrize("T, H, E, B", [(2100, 3, 384, 2), (2048, 5, 320, 3), (2301, 2, 128, 9),
-                                        (2048, 12, 768, 6), (4096, 4, 512, 3)])
+                                        (2048, 12, 768, 6), (4096, 4, 512, 3),
+                                        (256, 2, 512, 3), (301, 3, 768, 2), (2100, 2, 512, 2)])
 def test_long_sequences_take_the_eight_wave_kernel(capi, oracle, T, H, E, B):
-    # From 2048 rows on the forward at head widths 64 and 128 runs an eight-wave
-    # kernel (256-row tiles; here with the packed [rows, 3E] layout, several
-    # sequences and heads, lengths that are not a multiple of its tile, more
-    # and fewer tiles than compute units).  It must leave exactly what the
-    # four-wave kernel leaves, which the oracle pins.
+    # From 2048 rows on the forward at head widths 64 and 128 runs the kernel
+    # with the hand-scheduled loop (256-row tiles, 128 at width 64; here with the
+    # packed [rows, 3E] layout, several sequences and heads, lengths that are
+    # not a multiple of its tile, more and fewer tiles than compute units); at
+    # head width 256 from 256 rows (128-row tiles, one wave a SIMD).  It must
+    # leave exactly what the four-wave kernel leaves, which the oracle pins.
     rng = np.random.default_rng(31)
     host = rng.standard_normal((B * T, 3 * E)).astype(np.float32)
     x = torch.from_numpy(host).cuda().to(torch.bfloat16)
