@@ -572,6 +572,22 @@ unsigned pluto_hip_test_kernel_classes(unsigned mask);
 #define PLUTO_HIP_PATH_RECURRENCE 6   /* token-by-token delta-net */
 int pluto_hip_test_last_path(void);
 
+/* The tile lists the attention forward with the hand-scheduled loop would
+ * launch with for a shape, computed on the host alone (no device is touched):
+ * `items[w * *slots + e]` is entry e of workgroup w's list, (sequence *
+ * query_heads + head) * q_tiles + q_tile with q_tiles = ceil(q_rows /
+ * tile_rows), or 0xffff past the list's end; tile_rows is 256 at head width
+ * 128 and 128 at 64 and 256.  `workgroups_resident` is what the launcher
+ * derives from the device (compute units x workgroups a compute unit).
+ * Returns 0 and sets *workgroups (0: the launch numbers its tiles by
+ * workgroup index instead of lists) and *slots; PLUTO_HIP_EINVAL for a bad
+ * argument, PLUTO_HIP_ELIMIT when `capacity` entries do not hold the lists.
+ * Lets a test check, for any shape, that every tile is launched exactly once. */
+int pluto_hip_test_forward_schedule(int head_dim, int q_rows, int kv_rows, int start_position,
+                                    int query_heads, int group, int sequences,
+                                    int workgroups_resident, uint16_t* items, int capacity,
+                                    int* workgroups, int* slots);
+
 #ifdef __cplusplus
 }
 #endif

@@ -71,6 +71,8 @@ SIGNATURES = {
     "pluto_hip_test_force_generic": (_I, [_I]),
     "pluto_hip_test_kernel_classes": (ctypes.c_uint, [ctypes.c_uint]),
     "pluto_hip_test_last_path": (_I, []),
+    "pluto_hip_test_forward_schedule": (_I, [_I] * 8 + [ctypes.POINTER(ctypes.c_uint16), _I,
+                                                        ctypes.POINTER(_I), ctypes.POINTER(_I)]),
     "pluto_hip_abi_version": (_I, []),
     "pluto_hip_target_arch": (ctypes.c_char_p, []),
     "pluto_hip_executor_create": (_I, [ctypes.POINTER(_VP)]),

@@ -619,3 +619,28 @@ int launch_flash_forward_pipelined(hipStream_t stream, const FlashForwardArgs& a
 }
 
 }  // namespace pluto_hip
+
+extern "C" int pluto_hip_test_forward_schedule(int head_dim, int q_rows, int kv_rows,
+                                               int start_position, int query_heads, int group,
+                                               int sequences, int workgroups_resident,
+                                               uint16_t* items, int capacity, int* workgroups,
+                                               int* slots) {
+  using namespace pluto_hip;
+  if ((head_dim != 64 && head_dim != 128 && head_dim != 256) || q_rows <= 0 || kv_rows <= 0 ||
+      start_position < 0 || query_heads <= 0 || group <= 0 || query_heads % group != 0 ||
+      sequences <= 0 || workgroups_resident < 0 || !items || capacity < 0 || !workgroups || !slots)
+    return PLUTO_HIP_EINVAL;
+  ScheduleKey key;
+  key.q_rows = q_rows, key.kv_rows = kv_rows, key.start_position = start_position;
+  key.query_heads = query_heads, key.group = group, key.sequences = sequences;
+  key.tile_rows =
+      32 * (head_dim == 256 ? kWaves<256> : head_dim == 128 ? kWaves<128> : kWaves<64>);
+  key.workgroups = workgroups_resident;
+  static thread_local Schedule schedule;
+  *workgroups = build_schedule(key, schedule);
+  *slots = schedule.slots;
+  const long long entries = static_cast<long long>(*workgroups) * schedule.slots;
+  if (entries > capacity) return PLUTO_HIP_ELIMIT;
+  for (long long i = 0; i < entries; ++i) items[i] = schedule.item[i];
+  return 0;
+}
