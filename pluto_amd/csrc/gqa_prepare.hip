@@ -9,6 +9,7 @@
 // rounded results agree with it except on exact rounding ties.
 #include "gqa.h"
 #include "gqa_rotate.h"
+#include "mfma_tile.h"
 
 namespace pluto_hip {
 namespace {
@@ -114,32 +115,48 @@ prefill_prepare_bf16_kernel(PrefillPrepareArgs a) {
   const float4 w0 = *reinterpret_cast<const float4*>(weight + 8 * chunk);
   const float4 w1 = *reinterpret_cast<const float4*>(weight + 8 * chunk + 4);
   const float w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
-  float n[8];
+  // Rounding to bf16 is the hardware's conversion (round to nearest even, two
+  // values an instruction); a rounded pair stays packed until its values are
+  // needed again as floats.
+  uint32_t normalized[4];
 #pragma unroll
-  for (int e = 0; e < 8; ++e)
-    n[e] = round_to_bf16(static_cast<float>(x[e] * inverse * (1.0 + static_cast<double>(w[e]))));
-  // RoPE partner channels c +- half live `half / 8` lanes away.
+  for (int i = 0; i < 4; ++i)
+    normalized[i] = pack_bf16(
+        static_cast<float>(x[2 * i] * inverse * (1.0 + static_cast<double>(w[2 * i]))),
+        static_cast<float>(x[2 * i + 1] * inverse * (1.0 + static_cast<double>(w[2 * i + 1]))));
+  // RoPE partner channels c +- half live `half / 8` lanes away: four packed
+  // words travel instead of eight floats.
   const int first = 8 * chunk;
   const bool rotated = first < a.rotary_dim;
   const bool lower = first < half;
   const int lane = threadIdx.x % 64;
-  const int partner_lane = lower ? lane + half / 8 : lane - half / 8;
-  float result[8];
-  const float* cos_row = a.cosines + static_cast<long long>(row) * half + (lower ? first : first - half);
-  const float* sin_row = a.sines + static_cast<long long>(row) * half + (lower ? first : first - half);
+  const int partner_lane = rotated ? (lower ? lane + half / 8 : lane - half / 8) : lane;
+  uint32_t partner[4];
 #pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    const float np = __shfl(n[e], rotated ? partner_lane : lane, 64);
-    result[e] = n[e];
-    if (rotated) {
-      const float p = round_to_bf16(n[e] * cos_row[e]);
-      const float q = round_to_bf16(np * sin_row[e]);
-      result[e] = round_to_bf16(lower ? p - q : p + q);
+  for (int i = 0; i < 4; ++i) partner[i] = __shfl(normalized[i], partner_lane, 64);
+  uint32_t result[4] = {normalized[0], normalized[1], normalized[2], normalized[3]};
+  if (rotated) {
+    const long long table = static_cast<long long>(row) * half + (lower ? first : first - half);
+    const float4 c0 = *reinterpret_cast<const float4*>(a.cosines + table);
+    const float4 c1 = *reinterpret_cast<const float4*>(a.cosines + table + 4);
+    const float4 s0 = *reinterpret_cast<const float4*>(a.sines + table);
+    const float4 s1 = *reinterpret_cast<const float4*>(a.sines + table + 4);
+    const float cosine[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+    const float sine[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float n0 = __uint_as_float(normalized[i] << 16);
+      const float n1 = __uint_as_float(normalized[i] & 0xffff0000u);
+      const float p0 = __uint_as_float(partner[i] << 16);
+      const float p1 = __uint_as_float(partner[i] & 0xffff0000u);
+      const uint32_t own = pack_bf16(n0 * cosine[2 * i], n1 * cosine[2 * i + 1]);
+      const uint32_t other = pack_bf16(p0 * sine[2 * i], p1 * sine[2 * i + 1]);
+      const float a0 = __uint_as_float(own << 16), a1 = __uint_as_float(own & 0xffff0000u);
+      const float b0 = __uint_as_float(other << 16), b1 = __uint_as_float(other & 0xffff0000u);
+      result[i] = lower ? pack_bf16(a0 - b0, a1 - b1) : pack_bf16(a0 + b0, a1 + b1);
     }
   }
-  *reinterpret_cast<uint4*>(out + 8 * chunk) =
-      make_uint4(pack_bf16_bits(result[0], result[1]), pack_bf16_bits(result[2], result[3]),
-                 pack_bf16_bits(result[4], result[5]), pack_bf16_bits(result[6], result[7]));
+  *reinterpret_cast<uint4*>(out + 8 * chunk) = make_uint4(result[0], result[1], result[2], result[3]);
   if (!is_query) {
     const uint16_t* v_in = static_cast<const uint16_t*>(a.v) +
                            (static_cast<long long>(row) * a.key_value_heads + kv) * D;
