@@ -277,8 +277,10 @@ int pluto_hip_gqa_prefill_probabilities(void* stream,
  *   probabilities: optional HOST array of `batch` device pointers (entries may
  *             be NULL), each fp32 [qh, positions[b] + 1]
  *             (AttentionProbabilitiesKernel, cached_attention_ops.cc:131-178)
- *   split_tokens: tokens per split-K block (512 in the decode configuration;
- *             0 selects the default)
+ *   split_tokens: cache rows per split-K block: a multiple of 64 up to 512, or
+ *             1024 at head width 256; 0 selects the default (512, and 1024
+ *             at head width 256).  Anything else is PLUTO_HIP_EINVAL, and the
+ *             workspace size is then reported as 0.
  * Returns PLUTO_HIP_ERANGE if any positions[b] >= capacity; nothing is
  * queued in that case. */
 size_t pluto_hip_gqa_decode_workspace_bytes(const pluto_hip_attention_params* p,

@@ -142,7 +142,9 @@ PrefillBackwardLayout prefill_backward_layout(const pluto_hip_attention_params* 
   return l;
 }
 
-int split_or_default(int split_tokens) { return split_tokens == 0 ? 512 : split_tokens; }
+int split_or_default(int split_tokens, int head_dim) {
+  return split_tokens == 0 ? decode_split_default(head_dim) : split_tokens;
+}
 
 long long decode_blocks(int batch, const int* positions, int split) {
   long long blocks = 0;
@@ -464,8 +466,8 @@ static DecodeLayout decode_layout(const pluto_hip_attention_params* p, int batch
 size_t pluto_hip_gqa_decode_workspace_bytes(const pluto_hip_attention_params* p, int batch,
                                             const int* positions, int split_tokens) {
   if (validate_params(p) != 0 || batch <= 0 || !positions) return 0;
-  const int split = split_or_default(split_tokens);
-  if (split < 64 || split > 512 || split % 64 != 0) return 0;
+  const int split = split_or_default(split_tokens, p ? p->head_dim : 0);
+  if (!decode_split_valid(p->head_dim, split)) return 0;
   for (int b = 0; b < batch; ++b)
     if (positions[b] < 0) return 0;
   const long long blocks = decode_blocks(batch, positions, split);
@@ -487,7 +489,7 @@ static int decode_check(const pluto_hip_attention_params* p, int batch, int io_d
   // cached_attention_ops.cc:314-317: null pointers are rejected before any work.
   if (!q_gate || !k || !v || !q_norm || !k_norm || !out || !positions || !caches)
     return PLUTO_HIP_EINVAL;
-  if (split < 64 || split > 512 || split % 64 != 0) return PLUTO_HIP_EINVAL;
+  if (!decode_split_valid(p->head_dim, split)) return PLUTO_HIP_EINVAL;
   for (int b = 0; b < batch; ++b) {
     status = validate_cache(&caches[b], p);
     if (status != 0) return status;
@@ -519,7 +521,7 @@ int pluto_hip_gqa_decode(void* stream, const pluto_hip_attention_params* p, int 
                          const pluto_hip_kv_cache_view* caches, void* out,
                          float* const* probabilities, int split_tokens, void* workspace,
                          size_t workspace_bytes) {
-  const int split = split_or_default(split_tokens);
+  const int split = split_or_default(split_tokens, p ? p->head_dim : 0);
   const int status =
       decode_check(p, batch, io_dtype, q_gate, k, v, q_norm, k_norm, positions, caches, out, split);
   if (status != 0) return status;
@@ -544,7 +546,7 @@ int pluto_hip_gqa_decode_static(void* stream, const pluto_hip_attention_params* 
                                 const float* q_norm, const float* k_norm, const int* positions,
                                 const pluto_hip_kv_cache_view* caches, void* out,
                                 float* const* probabilities, int split_tokens) {
-  const int split = split_or_default(split_tokens);
+  const int split = split_or_default(split_tokens, p ? p->head_dim : 0);
   int status =
       decode_check(p, batch, io_dtype, q_gate, k, v, q_norm, k_norm, positions, caches, out, split);
   if (status != 0) return status;

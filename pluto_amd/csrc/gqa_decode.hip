@@ -31,6 +31,8 @@
 //           combines that pair's blocks in ascending order (a fixed order,
 //           whichever workgroup does it: bitwise repeatable), applies
 //           bf16(bf16(core) * bf16(sigmoid(gate))) and leaves the counter zero.
+#include <type_traits>
+
 #include "gqa.h"
 #include "gqa_rotate.h"
 #include "mfma_tile.h"
@@ -132,6 +134,43 @@ __device__ inline void prepare_head(const void* base, long long offset, int dtyp
     row[lane + 64 * i] = static_cast<uint16_t>(__float_as_uint(result[i]) >> 16);
 }
 
+// Compile-time loop: f(std::integral_constant<int, I>) for I = FIRST .. LAST-1.
+template <int FIRST, int LAST, class F>
+__device__ inline void static_for(F&& f) {
+  if constexpr (FIRST < LAST) {
+    f(std::integral_constant<int, FIRST>{});
+    static_for<FIRST + 1, LAST>(f);
+  }
+}
+
+// K rows requested without the compiler's knowledge of when they land: the
+// wave's vector-memory queue then holds K rows and V stage fills in an order
+// only this file knows, and wait_for_rows() says how many younger requests may
+// still be outstanding when a group's rows are needed (requests complete in
+// order).  Passing the registers through the wait ties every use to it.
+template <int KSTEPS>
+__device__ inline void request_rows(const uint16_t* row, bf16x8 (&dst)[KSTEPS]) {
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ++ks)
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst[ks]) : "v"(row + 32 * ks) : "memory");
+}
+template <int OUTSTANDING, int KSTEPS>
+__device__ inline void wait_for_rows(bf16x8 (&k)[KSTEPS]) {
+  static_assert(OUTSTANDING >= 0 && OUTSTANDING < 64);
+  static_assert(KSTEPS == 2 || KSTEPS == 4 || KSTEPS == 8);
+  if constexpr (KSTEPS == 2)
+    asm volatile("s_waitcnt vmcnt(%2)" : "+v"(k[0]), "+v"(k[1]) : "n"(OUTSTANDING) : "memory");
+  else if constexpr (KSTEPS == 4)
+    asm volatile("s_waitcnt vmcnt(%4)"
+                 : "+v"(k[0]), "+v"(k[1]), "+v"(k[2]), "+v"(k[3])
+                 : "n"(OUTSTANDING) : "memory");
+  else
+    asm volatile("s_waitcnt vmcnt(%8)"
+                 : "+v"(k[0]), "+v"(k[1]), "+v"(k[2]), "+v"(k[3]), "+v"(k[4]), "+v"(k[5]),
+                   "+v"(k[6]), "+v"(k[7])
+                 : "n"(OUTSTANDING) : "memory");
+}
+
 // What a workgroup knows about its (sequence, kv head, block).
 struct BlockContext {
   int tid, wave, lane, hq, n;
@@ -142,12 +181,45 @@ struct BlockContext {
 };
 
 constexpr int kStageRows = 16;  // V rows per LDS stage of a wave: one contraction step
-constexpr int kStages = 3;      // stages per wave: one in use, the others travelling
+// Stages per wave (one in use, the others travelling) and K groups requested
+// before they are used.  At head width 256 a group and a stage are 8 KiB a
+// wave each; two of either let two workgroups share a compute unit (64 KiB
+// of LDS and under 256 registers each), which covers one workgroup's start
+// and hand-over with the other's stream.
+constexpr int stages_of(int head_dim) { return head_dim == 256 ? 2 : 3; }
+constexpr int ahead_of(int head_dim) { return head_dim == 256 ? 2 : 4; }
+
+// Request order of a wave when the block size is a compile-time constant: K
+// groups 0 .. ahead-1 up front; score step j then requests group j + ahead,
+// and once the K rows run out the first V stages instead, one a step, so
+// that requests stay in flight from the last score steps into the first value
+// steps.  A group and a stage are the same number of requests per lane
+// (D / 32); ahead >= stages, so every first stage finds a step.
+struct RequestOrder {
+  int groups, ahead, stages;
+  constexpr int first_fill_step() const { return groups > ahead ? groups - ahead : 0; }
+  constexpr bool step_requests_rows(int step) const { return step + ahead < groups; }
+  constexpr bool step_requests_stage(int step) const {
+    const int stage = step - first_fill_step();
+    return !step_requests_rows(step) && stage >= 0 && stage < stages && stage < groups;
+  }
+  // Units (groups or stages) requested after K group `group` and before score
+  // step `group` waits for it.
+  constexpr int units_after_group(int group) const {
+    const int up_front = groups < ahead ? groups : ahead;
+    int after = group < up_front ? up_front - 1 - group : 0;
+    for (int step = 0; step < group; ++step) {
+      if (step_requests_rows(step)) after += step + ahead > group ? 1 : 0;
+      else if (step_requests_stage(step)) after += 1;
+    }
+    return after;
+  }
+};
 
 // LDS of a workgroup: per wave kStages stages of 16 V rows (later reused for
 // the waves' partial outputs and the combine's block weights).
 template <int D>
-constexpr int value_area_bytes() { return 4 * kStages * kStageRows * D * 2; }
+constexpr int value_area_bytes() { return 4 * stages_of(D) * kStageRows * D * 2; }
 
 // Prepare step, split-K attention over one block and the block's partial
 // results.  SPLIT: tokens per block when known at compile time (the loops
@@ -177,8 +249,10 @@ __device__ inline void decode_block(const DecodeArgs& a, const BlockContext& ctx
   constexpr int KSTEPS = D / 32;
   constexpr int KCH = D / 8;                       // 16-byte chunks per row
   constexpr int GROUPS = (SPLIT ? SPLIT : kMaxSplit) / 64;  // 16-token groups per wave at most
-  constexpr int kAhead = 4;  // K groups requested before they are used
   constexpr int FILLS = kStageRows * KCH / 64;     // 16-byte fills per lane and stage
+  constexpr int kStages = stages_of(D), kAhead = ahead_of(D);
+  constexpr RequestOrder kOrder = {GROUPS, kAhead, kStages};
+  static_assert(kAhead >= kStages);
   constexpr int kStageBytes = kStageRows * D * 2;
   constexpr int CB = D / 16;                       // 16-channel blocks of O^T
   float (*o_lds)[GROUP][D] = reinterpret_cast<float (*)[GROUP][D]>(value_area);
@@ -192,7 +266,8 @@ __device__ inline void decode_block(const DecodeArgs& a, const BlockContext& ctx
   const int groups = per_wave / 16;  // 16-token groups of this wave (<= GROUPS)
   const int wave_t0 = t0 + wave * per_wave;
 
-  // ---- the first two V stages are requested before anything else ----------
+  // ---- V stages: requested before anything else when the block size is only
+  // known at run time, between the last score steps otherwise ---------------
   unsigned char* stage_base = value_area + wave * kStages * kStageBytes;
   uint32_t fill_offset[FILLS];
 #pragma unroll
@@ -212,9 +287,11 @@ __device__ inline void decode_block(const DecodeArgs& a, const BlockContext& ctx
     for (int i = 0; i < FILLS; ++i)
       lds_fill<16>(rsrc, stage_base + (st % kStages) * kStageBytes + i * 1024, fill_offset[i]);
   };
+  if constexpr (SPLIT == 0) {
 #pragma unroll
-  for (int st = 0; st < kStages; ++st)
-    if (st < groups) fill(st);
+    for (int st = 0; st < kStages; ++st)
+      if (st < groups) fill(st);
+  }
 
   // ---- then the first K rows ------------------------------------------------
   // A operand row = lane % 16; rows beyond the valid prefix repeat its last row
@@ -229,10 +306,19 @@ __device__ inline void decode_block(const DecodeArgs& a, const BlockContext& ctx
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) dst[ks] = load_bf16x8(row + 32 * ks);
   };
+  auto request_k = [&](int grp, bf16x8 (&dst)[KSTEPS]) {
+    request_rows<KSTEPS>(keys + static_cast<long long>(k_token(grp)) * a.token_stride + 8 * hq,
+                         dst);
+  };
   bf16x8 k_rows[kAhead][KSTEPS];
 #pragma unroll
-  for (int grp = 0; grp < kAhead; ++grp)
-    if (grp < groups) load_k(grp, k_rows[grp]);
+  for (int grp = 0; grp < kAhead; ++grp) {
+    if constexpr (SPLIT == 0) {
+      if (grp < groups) load_k(grp, k_rows[grp]);
+    } else {
+      if (grp < GROUPS) request_k(grp, k_rows[grp]);
+    }
+  }
 
   // ---- prepare: the group's queries, and the new cache row ----------------
   {
@@ -293,29 +379,51 @@ __device__ inline void decode_block(const DecodeArgs& a, const BlockContext& ctx
   }
   floatx4 s[GROUPS];
   float local_max = kMasked;
+  auto score_group = [&](int grp, const bf16x8 (&rows)[KSTEPS]) {
+    floatx4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-  for (int grp = 0; grp < GROUPS; ++grp) {
-    s[grp] = floatx4{kMasked, kMasked, kMasked, kMasked};
-    if (grp < groups) {
-      floatx4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks) {
-        bf16x8 k_use = k_rows[grp % kAhead][ks];
-        if constexpr (LAST) k_use = k_token(grp) == position ? k_new[ks] : k_use;
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k_use, qf[ks], acc, 0, 0, 0);
-      }
-      // this group's registers take the rows of the group kAhead further on
-      if (grp + kAhead < groups) load_k(grp + kAhead, k_rows[grp % kAhead]);
-      // accumulator register r = (token 4*hq + r of the group, head n)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int t = wave_t0 + 16 * grp + 4 * hq + r;
-        const float v = (!LAST || t < length) ? acc[r] * scale2 : kMasked;
-        acc[r] = v;
-        local_max = fmaxf(local_max, v);
-      }
-      s[grp] = acc;
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      bf16x8 k_use = rows[ks];
+      if constexpr (LAST) k_use = k_token(grp) == position ? k_new[ks] : k_use;
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k_use, qf[ks], acc, 0, 0, 0);
     }
+    return acc;
+  };
+  // accumulator register r = (token 4*hq + r of the group, head n)
+  auto scaled = [&](int grp, floatx4 acc) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int t = wave_t0 + 16 * grp + 4 * hq + r;
+      const float v = (!LAST || t < length) ? acc[r] * scale2 : kMasked;
+      acc[r] = v;
+      local_max = fmaxf(local_max, v);
+    }
+    return acc;
+  };
+  if constexpr (SPLIT == 0) {
+#pragma unroll
+    for (int grp = 0; grp < GROUPS; ++grp) {
+      s[grp] = floatx4{kMasked, kMasked, kMasked, kMasked};
+      if (grp < groups) {
+        const floatx4 acc = score_group(grp, k_rows[grp % kAhead]);
+        // this group's registers take the rows of the group kAhead further on
+        if (grp + kAhead < groups) load_k(grp + kAhead, k_rows[grp % kAhead]);
+        s[grp] = scaled(grp, acc);
+      }
+    }
+  } else {
+    static_for<0, GROUPS>([&](auto index) {
+      constexpr int grp = decltype(index)::value;
+      wait_for_rows<kOrder.units_after_group(grp) * KSTEPS>(k_rows[grp % kAhead]);
+      const floatx4 acc = score_group(grp, k_rows[grp % kAhead]);
+      // this group's registers take the rows of the group kAhead further on;
+      // when the rows have run out, a V stage is requested in their place
+      if constexpr (kOrder.step_requests_rows(grp))
+        request_k(grp + kAhead, k_rows[grp % kAhead]);
+      else if constexpr (kOrder.step_requests_stage(grp))
+        fill(grp - kOrder.first_fill_step());
+      s[grp] = scaled(grp, acc);
+    });
   }
   // Each wave normalises its quarter of the block by its own maximum.
   local_max = fmaxf(local_max, __shfl_xor(local_max, 16, 64));
@@ -438,7 +546,7 @@ __device__ inline void decode_block(const DecodeArgs& a, const BlockContext& ctx
 
 template <int D, int GROUP>
 __global__ void __launch_bounds__(kThreads)
-__attribute__((amdgpu_waves_per_eu(D == 256 ? 1 : 3, D == 256 ? 1 : 3)))
+__attribute__((amdgpu_waves_per_eu(D == 256 ? 2 : 3, D == 256 ? 2 : 3)))
 decode_fused_kernel(DecodeArgs a, DecodeBatch batch) {
   __shared__ __attribute__((aligned(1024))) unsigned char value_area[value_area_bytes<D>()];
   float* shared_area = reinterpret_cast<float*>(value_area);
@@ -472,11 +580,12 @@ decode_fused_kernel(DecodeArgs a, DecodeBatch batch) {
   ctx.values = static_cast<uint16_t*>(batch.values[b]) + g * a.head_stride;
   ctx.slot = (a.block_base + block) * kh + g;
   const bool is_last = j == blocks_here - 1;  // this block holds row `position`
-  if (a.split_tokens == kMaxSplit) {
+  constexpr int kFixed = decode_split_default(D);
+  if (a.split_tokens == kFixed) {
     if (is_last)
-      decode_block<D, GROUP, kMaxSplit, true>(a, ctx, value_area, wave_max, wave_sum_lds, q_lds, new_row);
+      decode_block<D, GROUP, kFixed, true>(a, ctx, value_area, wave_max, wave_sum_lds, q_lds, new_row);
     else
-      decode_block<D, GROUP, kMaxSplit, false>(a, ctx, value_area, wave_max, wave_sum_lds, q_lds, new_row);
+      decode_block<D, GROUP, kFixed, false>(a, ctx, value_area, wave_max, wave_sum_lds, q_lds, new_row);
   } else {
     if (is_last)
       decode_block<D, GROUP, 0, true>(a, ctx, value_area, wave_max, wave_sum_lds, q_lds, new_row);
@@ -673,8 +782,7 @@ int launch_decode_fast(hipStream_t stream, const DecodeArgs& a, const DecodeBatc
   const long long blocks =
       static_cast<long long>(batch.block_start[batch.count]) * a.key_value_heads;
   if (blocks <= 0 || blocks > 0x7fffffffLL) return PLUTO_HIP_EINVAL;
-  if (a.split_tokens < 64 || a.split_tokens > kMaxSplit || a.split_tokens % 64 != 0)
-    return PLUTO_HIP_EINVAL;
+  if (!decode_split_valid(a.head_dim, a.split_tokens)) return PLUTO_HIP_EINVAL;
   if (a.rotary_dim / 2 > 128) return PLUTO_HIP_EUNSUPPORTED;
   if (!kernel_enabled(kMainKernel)) return 0;
   switch (a.head_dim) {

@@ -397,6 +397,54 @@ def test_config4_batched_decode(capi, oracle):
     assert torch.equal(out, again)
 
 
+@pytest.mark.parametrize("split", [0, 1024, 512, 192])
+def test_batched_decode_at_the_models_head_width(capi, oracle, split):
+    # cached_attention_ops.h:13-22: heads of 256 with 64 rotated channels.  The
+    # fused kernel is specialised for blocks of 1024 cache rows there (the
+    # default, split 0) and takes any other multiple of 64 up to 512 with its
+    # run-time loops; lengths on both sides of the block boundaries.
+    qh, kh, d, capacity = 12, 2, 256, 5120
+    kw = dict(query_heads=qh, key_value_heads=kh, head_dim=d, rotary_dim=64, capacity=capacity)
+    p, po = both_params(capi, oracle, **kw)
+    lengths = np.array([1, 700, 1024, 1025, 2049, 5000, 3072, 192, 193])
+    batch = len(lengths)
+    rng = np.random.default_rng(256)
+    gen = torch.Generator(device="cuda").manual_seed(256)
+    caches = []
+    for L in lengths:
+        c = capi.KvCache(capacity, kh, d, fill=float("nan"))
+        if L > 1:
+            c.keys[:, :L - 1] = torch.randn((kh, L - 1, d), generator=gen, device="cuda").to(torch.bfloat16)
+            c.values[:, :L - 1] = torch.randn((kh, L - 1, d), generator=gen, device="cuda").to(torch.bfloat16)
+        c.position = int(L - 1)
+        caches.append(c)
+    q_gate = oracle.bf16_round(rng.standard_normal((batch, qh, 2, d)).astype(np.float32))
+    k = oracle.bf16_round(rng.standard_normal((batch, kh, d)).astype(np.float32))
+    v = oracle.bf16_round(rng.standard_normal((batch, kh, d)).astype(np.float32))
+    qw, kw_ = values(d, 0.2, 0.3), values(d, 0.8, 0.4)
+    bf = torch.bfloat16
+    args = (p, dev(q_gate, bf), dev(k, bf), dev(v, bf), dev(qw), dev(kw_), caches)
+    out = capi.gqa_decode(*args, split_tokens=split, advance=False)
+    assert capi.last_path() == capi.PATH_SPLIT_K
+    torch.cuda.synchronize()
+    got = out.float().cpu().numpy()
+    assert np.all(np.isfinite(got))
+    for b in range(batch):
+        L = int(lengths[b])
+        keys = caches[b].keys[:, :L].float().cpu().numpy()
+        vals = caches[b].values[:, :L].float().cpu().numpy()
+        for h in range(kh):
+            near(keys[h, L - 1], oracle.gqa_normalize_rotate(po, L - 1, k[b, h], kw_), True)
+            np.testing.assert_array_equal(vals[h, L - 1], oracle.bf16_round(v[b, h]))
+        q = np.stack([oracle.gqa_normalize_rotate(po, L - 1, q_gate[b, h, 0], qw) for h in range(qh)])
+        near(got[b], oracle.gqa_attend(po, q, q_gate[b, :, 1], keys, vals), True)
+    with capi.force_generic():
+        generic = capi.gqa_decode(*args, split_tokens=split, advance=False)
+        torch.cuda.synchronize()
+    near(got, generic.float().cpu().numpy(), True)
+    assert torch.equal(out, capi.gqa_decode(*args, split_tokens=split, advance=False))
+
+
 def test_decode_more_than_one_launch_slice(capi, oracle):
     # 70 sequences > 64 per launch, ragged short lengths, split 64
     batch, qh, kh, d = 70, 4, 2, 64
@@ -460,6 +508,18 @@ def test_rejects_invalid_arguments_before_any_work(capi):
             capi.ptr(call[2]), capi.ptr(call[3]), capi.ptr(call[4]), pos, views,
             capi.ptr(t), None, 0, capi.ptr(ws), ws.numel())
         assert code == capi.EINVAL
+    # split-K blocks: multiples of 64 up to 512 rows, 1024 at head width 256 only
+    for split in (-64, 32, 100, 576, 1024, 2048):
+        with pytest.raises(capi.PlutoHipError) as info:
+            capi.gqa_decode(p, *args, [cache], out=t[:8].view(1, 2, 4), split_tokens=split)
+        assert info.value.code == capi.EINVAL and cache.position == 0
+        pos = (ctypes.c_int * 1)(0)
+        assert capi.lib().pluto_hip_gqa_decode_workspace_bytes(ctypes.byref(p), 1, pos, split) == 0
+    wide = capi.attention_params(query_heads=2, key_value_heads=1, head_dim=256, rotary_dim=64,
+                                 capacity=2)
+    pos = (ctypes.c_int * 1)(0)
+    assert capi.lib().pluto_hip_gqa_decode_workspace_bytes(ctypes.byref(wide), 1, pos, 1024) > 0
+    assert capi.lib().pluto_hip_gqa_decode_workspace_bytes(ctypes.byref(wide), 1, pos, 2048) == 0
     torch.cuda.synchronize()
     assert torch.all(t == -13.0)
 
