@@ -397,16 +397,21 @@ def test_config4_batched_decode(capi, oracle):
     assert torch.equal(out, again)
 
 
-@pytest.mark.parametrize("split", [0, 1024, 512, 192])
-def test_batched_decode_at_the_models_head_width(capi, oracle, split):
-    # cached_attention_ops.h:13-22: heads of 256 with 64 rotated channels.  The
-    # fused kernel is specialised for blocks of 1024 cache rows there (the
-    # default, split 0) and takes any other multiple of 64 up to 512 with its
-    # run-time loops; lengths on both sides of the block boundaries.
-    qh, kh, d, capacity = 12, 2, 256, 5120
-    kw = dict(query_heads=qh, key_value_heads=kh, head_dim=d, rotary_dim=64, capacity=capacity)
+@pytest.mark.parametrize("d,qh,kh,rotary,split", [
+    (256, 12, 2, 64, 0), (256, 12, 2, 64, 1024), (256, 12, 2, 64, 512), (256, 12, 2, 64, 192),
+    (256, 8, 1, 256, 0), (64, 8, 2, 16, 0), (64, 2, 2, 64, 512), (64, 4, 2, 32, 320),
+    (128, 8, 1, 32, 0), (128, 4, 4, 128, 0)])
+def test_batched_decode_block_sizes_and_head_widths(capi, oracle, d, qh, kh, rotary, split):
+    # cached_attention_ops.h:13-22: the model's heads are 256 wide with 64
+    # rotated channels.  The fused kernel is specialised for blocks of 1024
+    # cache rows there and of 512 at the narrower widths (the defaults, split
+    # 0), with a request order fixed at compile time, and takes any other
+    # multiple of 64 up to 512 with its run-time loops; groups of 1, 2, 4, 6
+    # and 8 query heads; lengths on both sides of the block boundaries.
+    capacity = 5120
+    kw = dict(query_heads=qh, key_value_heads=kh, head_dim=d, rotary_dim=rotary, capacity=capacity)
     p, po = both_params(capi, oracle, **kw)
-    lengths = np.array([1, 700, 1024, 1025, 2049, 5000, 3072, 192, 193])
+    lengths = np.array([1, 700, 1024, 1025, 2049, 5000, 3072, 192, 193, 512, 513])
     batch = len(lengths)
     rng = np.random.default_rng(256)
     gen = torch.Generator(device="cuda").manual_seed(256)
