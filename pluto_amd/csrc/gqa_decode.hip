@@ -216,6 +216,41 @@ struct RequestOrder {
   }
 };
 
+// The same order replayed as a queue, at compile time: every K group is
+// requested exactly once and before its score step; when step `group` waits
+// with units_after_group(group) units allowed outstanding, the group is no
+// longer among them but the unit right after it still is (the wait is exact,
+// not just safe); and when the value steps begin, the first
+// min(stages, groups) V stages, in order, are all that has been requested after
+// the last K group -- what the waits of the value steps count on.
+constexpr bool request_order_holds(int groups, int ahead, int stages) {
+  const RequestOrder order = {groups, ahead, stages};
+  int queue[64] = {};  // unit i of the queue: K group g as g, V stage s as 100 + s
+  int issued = 0;
+  for (int g = 0; g < groups && g < ahead; ++g) queue[issued++] = g;
+  for (int step = 0; step < groups; ++step) {
+    int at = -1;
+    for (int i = 0; i < issued; ++i)
+      if (queue[i] == step) at = at < 0 ? i : 64;
+    if (at < 0 || at >= 64) return false;  // not requested yet, or twice
+    if (issued - 1 - at != order.units_after_group(step)) return false;
+    if (order.step_requests_rows(step)) queue[issued++] = step + ahead;
+    else if (order.step_requests_stage(step)) queue[issued++] = 100 + step - order.first_fill_step();
+    if (issued > 60) return false;
+  }
+  const int first_stages = stages < groups ? stages : groups;
+  if (issued != groups + first_stages) return false;
+  for (int s = 0; s < first_stages; ++s)
+    if (queue[groups + s] != 100 + s) return false;  // stages follow every K group, in order
+  return true;
+}
+constexpr bool request_orders_hold() {
+  for (int groups = 1; groups <= 16; ++groups)
+    if (!request_order_holds(groups, 4, 3) || !request_order_holds(groups, 2, 2)) return false;
+  return true;
+}
+static_assert(request_orders_hold(), "the hand-counted waits of the score steps");
+
 // LDS of a workgroup: per wave kStages stages of 16 V rows (later reused for
 // the waves' partial outputs and the combine's block weights).
 template <int D>
