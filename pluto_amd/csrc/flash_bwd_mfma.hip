@@ -122,7 +122,9 @@ flash_dq_kernel(GenericBackwardArgs a, float* __restrict__ lse2,
     tile_fill<D, LOADS>(lds, wave, k_base, 3LL * E, 0, T, fill);
     tile_fill<D, LOADS>(lds + kTileBytes, wave, v_base, 3LL * E, 0, T, fill);
 
-    const int q_row = q0 + 32 * wave + n;
+    const int wave_first_row = q0 + 32 * wave;
+    const int q_row = wave_first_row + n;
+    uint4* copy_area = reinterpret_cast<uint4*>(lds + kStageBytes) + wave * 32 * KCH;
     // Rows beyond the sequence are clamped to its last row and never stored.
     const int q_load = min(q_row, T - 1);
     bf16x8 qf[KS], gf[KS];
@@ -146,8 +148,19 @@ flash_dq_kernel(GenericBackwardArgs a, float* __restrict__ lse2,
       }
       const uint4 bits = make_uint4(packed[0], packed[1], packed[2], packed[3]);
       gf[ks] = as_bf16x8(bits);
-      if (q_row < T)
-        *reinterpret_cast<uint4*>(gb_base + static_cast<long long>(q_row) * E + c) = bits;
+      copy_area[n * KCH + ((2 * ks + h) ^ (n & 7))] = bits;
+    }
+    // The bf16 copy of dO leaves through LDS (the wave's slice of the stage
+    // that no fill has been issued into yet): a lane holds 16-byte pieces of its
+    // own row, and stored from there a store instruction touches 32 lines;
+    // from LDS it writes whole rows (25 MB in 17 us against 5 us).
+#pragma unroll
+    for (int i = 0; i < 32 * KCH / 64; ++i) {
+      const int at = i * 64 + lane, row = at / KCH, chunk = at % KCH;
+      const uint4 bits = copy_area[row * KCH + (chunk ^ (row & 7))];
+      if (wave_first_row + row < T)
+        *reinterpret_cast<uint4*>(gb_base + static_cast<long long>(wave_first_row + row) * E +
+                                  8 * chunk) = bits;
     }
     // delta of attention.cc:283-291 (uses the stored, rounded output)
     const float row_delta = half_swap_sum(partial);
@@ -165,7 +178,6 @@ flash_dq_kernel(GenericBackwardArgs a, float* __restrict__ lse2,
 #pragma unroll
       for (int i = 0; i < 16; ++i) dq_acc[db][i] = 0.0f;
 
-    const int wave_first_row = q0 + 32 * wave;
     const int wave_last_key = wave_first_row + 31;
 
     for (int tile = 0; tile < tiles; ++tile) {
@@ -228,19 +240,41 @@ flash_dq_kernel(GenericBackwardArgs a, float* __restrict__ lse2,
         }
       }
     }
-    if (q_row < T) {
-      float* dst = a.d_qkv + (seq_row0 + q_row) * 3 * E + head * D;
+    // dQ leaves through LDS as dK and dV do in the key-owned kernel: 64 columns
+    // at a time, 32 rows x 64 floats a wave, pieces swizzled by row, so that
+    // every store instruction writes whole rows.
+    __syncthreads();  // every wave is done with the tile stages
+    {
+      static_assert(4 * 32 * 64 * 4 <= 2 * kStageBytes, "the stages hold one step of the workgroup");
+      constexpr int kPieces = 16;  // 16-byte pieces in 64 columns
+      float4* area = reinterpret_cast<float4*>(lds) + wave * 32 * kPieces;
+      const int out_piece = lane % kPieces, out_row = lane / kPieces;
 #pragma unroll
-      for (int db = 0; db < DB; ++db)
+      for (int half = 0; half < D / 64; ++half) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          float4 value;
-          value.x = dq_acc[db][4 * j + 0] * a.scale;
-          value.y = dq_acc[db][4 * j + 1] * a.scale;
-          value.z = dq_acc[db][4 * j + 2] * a.scale;
-          value.w = dq_acc[db][4 * j + 3] * a.scale;
-          *reinterpret_cast<float4*>(dst + 32 * db + 8 * j + 4 * h) = value;
+        for (int d2 = 0; d2 < 2; ++d2)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const floatx16& acc = dq_acc[2 * half + d2];
+            float4 value;
+            value.x = acc[4 * j + 0] * a.scale;
+            value.y = acc[4 * j + 1] * a.scale;
+            value.z = acc[4 * j + 2] * a.scale;
+            value.w = acc[4 * j + 3] * a.scale;
+            const int piece = 8 * d2 + 2 * j + h;
+            area[n * kPieces + (piece ^ (n % kPieces))] = value;
+          }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the wave reads what its own lanes wrote
+        float* dst = a.d_qkv + (seq_row0 + wave_first_row) * 3 * E + head * D + 64 * half;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const int row = 4 * i + out_row;
+          const float4 value = area[row * kPieces + (out_piece ^ (row % kPieces))];
+          if (wave_first_row + row < T)
+            *reinterpret_cast<float4*>(dst + static_cast<long long>(row) * 3 * E + 4 * out_piece) = value;
         }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // before the area is overwritten
+      }
     }
     __syncthreads();  // the next pass refills stage 0
   }
