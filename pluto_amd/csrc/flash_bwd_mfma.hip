@@ -240,41 +240,19 @@ flash_dq_kernel(GenericBackwardArgs a, float* __restrict__ lse2,
         }
       }
     }
-    // dQ leaves through LDS as dK and dV do in the key-owned kernel: 64 columns
-    // at a time, 32 rows x 64 floats a wave, pieces swizzled by row, so that
-    // every store instruction writes whole rows.
-    __syncthreads();  // every wave is done with the tile stages
-    {
-      static_assert(4 * 32 * 64 * 4 <= 2 * kStageBytes, "the stages hold one step of the workgroup");
-      constexpr int kPieces = 16;  // 16-byte pieces in 64 columns
-      float4* area = reinterpret_cast<float4*>(lds) + wave * 32 * kPieces;
-      const int out_piece = lane % kPieces, out_row = lane / kPieces;
+    if (q_row < T) {
+      float* dst = a.d_qkv + (seq_row0 + q_row) * 3 * E + head * D;
 #pragma unroll
-      for (int half = 0; half < D / 64; ++half) {
+      for (int db = 0; db < DB; ++db)
 #pragma unroll
-        for (int d2 = 0; d2 < 2; ++d2)
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const floatx16& acc = dq_acc[2 * half + d2];
-            float4 value;
-            value.x = acc[4 * j + 0] * a.scale;
-            value.y = acc[4 * j + 1] * a.scale;
-            value.z = acc[4 * j + 2] * a.scale;
-            value.w = acc[4 * j + 3] * a.scale;
-            const int piece = 8 * d2 + 2 * j + h;
-            area[n * kPieces + (piece ^ (n % kPieces))] = value;
-          }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the wave reads what its own lanes wrote
-        float* dst = a.d_qkv + (seq_row0 + wave_first_row) * 3 * E + head * D + 64 * half;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          const int row = 4 * i + out_row;
-          const float4 value = area[row * kPieces + (out_piece ^ (row % kPieces))];
-          if (wave_first_row + row < T)
-            *reinterpret_cast<float4*>(dst + static_cast<long long>(row) * 3 * E + 4 * out_piece) = value;
+        for (int j = 0; j < 4; ++j) {
+          float4 value;
+          value.x = dq_acc[db][4 * j + 0] * a.scale;
+          value.y = dq_acc[db][4 * j + 1] * a.scale;
+          value.z = dq_acc[db][4 * j + 2] * a.scale;
+          value.w = dq_acc[db][4 * j + 3] * a.scale;
+          *reinterpret_cast<float4*>(dst + 32 * db + 8 * j + 4 * h) = value;
         }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // before the area is overwritten
-      }
     }
     __syncthreads();  // the next pass refills stage 0
   }
