@@ -82,6 +82,11 @@ flash_dq_kernel(GenericBackwardArgs a, float* __restrict__ lse2,
   constexpr int kTileBytes = BN * D * 2, kStageBytes = 2 * kTileBytes;
   constexpr int kBlockBytes = 32 * D * 2;
   __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * kStageBytes];
+  // 4 KiB a wave that no other wave touches (64-wide heads, where three
+  // workgroups of 48 KiB still share a compute unit): rows on their way out are
+  // reordered here without a barrier
+  constexpr bool kOwnArea = D == 64;
+  __shared__ __attribute__((aligned(16))) uint4 own_area[kOwnArea ? 4 * 256 : 1];
 
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
   const int h = lane / 32, n = lane % 32;
@@ -124,7 +129,8 @@ flash_dq_kernel(GenericBackwardArgs a, float* __restrict__ lse2,
 
     const int wave_first_row = q0 + 32 * wave;
     const int q_row = wave_first_row + n;
-    uint4* copy_area = reinterpret_cast<uint4*>(lds + kStageBytes) + wave * 32 * KCH;
+    uint4* copy_area = kOwnArea ? own_area + wave * 256
+                                : reinterpret_cast<uint4*>(lds + kStageBytes) + wave * 32 * KCH;
     // Rows beyond the sequence are clamped to its last row and never stored.
     const int q_load = min(q_row, T - 1);
     bf16x8 qf[KS], gf[KS];
@@ -240,7 +246,33 @@ flash_dq_kernel(GenericBackwardArgs a, float* __restrict__ lse2,
         }
       }
     }
-    if (q_row < T) {
+    if constexpr (kOwnArea) {
+      // dQ leaves through the wave's own area, 32 columns at a time: a store
+      // instruction then writes eight whole 128-byte half rows instead of
+      // 32-byte pieces of 32 rows
+      float4* area = reinterpret_cast<float4*>(own_area) + wave * 256;
+      float* dst = a.d_qkv + (seq_row0 + wave_first_row) * 3 * E + head * D;
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          float4 value;
+          value.x = dq_acc[db][4 * j + 0] * a.scale;
+          value.y = dq_acc[db][4 * j + 1] * a.scale;
+          value.z = dq_acc[db][4 * j + 2] * a.scale;
+          value.w = dq_acc[db][4 * j + 3] * a.scale;
+          area[n * 8 + ((2 * j + h) ^ (n & 7))] = value;
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int row = 8 * i + lane / 8, piece = lane % 8;
+          const float4 value = area[row * 8 + (piece ^ (row & 7))];
+          if (wave_first_row + row < T)
+            *reinterpret_cast<float4*>(dst + static_cast<long long>(row) * 3 * E + 32 * db +
+                                       4 * piece) = value;
+        }
+      }
+    } else if (q_row < T) {
       float* dst = a.d_qkv + (seq_row0 + q_row) * 3 * E + head * D;
 #pragma unroll
       for (int db = 0; db < DB; ++db)
