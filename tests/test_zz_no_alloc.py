@@ -86,6 +86,19 @@ def test_two_calls_in_a_row_second_one_smaller(capi):
     run_both(capi, p, make_case(capi, 13, batch, qh, kh, d, capacity, lengths), lengths, 512)
 
 
+def test_the_models_head_width_on_both_block_size_paths(capi):
+    """Heads of 256 (cached_attention_ops.h:13-22): the default block of 1024
+    rows takes the kernel's compile-time request order, 512 its run-time loops;
+    the same scratch serves both, one call after the other."""
+    batch, qh, kh, d, capacity = 6, 12, 2, 256, 4096
+    p = capi.attention_params(qh, kh, d, 64, capacity=capacity)
+    lengths = np.array([4096, 1, 1024, 1025, 2500, 300])
+    run_both(capi, p, make_case(capi, 31, batch, qh, kh, d, capacity, lengths), lengths, 0)
+    lengths = np.array([700, 3000, 513, 4096, 64, 1024])
+    run_both(capi, p, make_case(capi, 32, batch, qh, kh, d, capacity, lengths), lengths, 512)
+    run_both(capi, p, make_case(capi, 33, batch, qh, kh, d, capacity, lengths), lengths, 1024)
+
+
 def test_reset_then_another_call(capi):
     """pluto_hip_gqa_decode_static_reset between two calls: the second call starts
     from cleared arrival counters and still matches the workspace entry point."""
