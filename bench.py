@@ -454,10 +454,14 @@ def decode_block(torch, capi):
     attention_out = torch.empty((batch, width), dtype=bf, device="cuda")
     decode_ws = capi.gqa_decode_workspace(p, positions, 0)
 
+    def project_many(matrices, x, outs):
+        # the projections of one input in one call, as the host's branches run them
+        capi.dense_imported_forward_many(capi.MATRIX_FP8_E4M3, [m["w"] for m in matrices],
+                                         [m["s"] for m in matrices], x, matrices[0]["ws"], outs)
+
     def attention_in():
-        project(wq, hidden, q_gate.view(batch, -1))
-        project(wk, hidden, k_new.view(batch, -1))
-        project(wv, hidden, v_new.view(batch, -1))
+        project_many([wq, wk, wv], hidden,
+                     [q_gate.view(batch, -1), k_new.view(batch, -1), v_new.view(batch, -1)])
 
     def attention_core():
         capi.gqa_decode(p, q_gate, k_new, v_new, qn, kn, caches, positions=positions,
@@ -484,10 +488,7 @@ def decode_block(torch, capi):
     mixed = [None]
 
     def delta_in():
-        project(wqkv, hidden, qkv)
-        project(wz, hidden, z)
-        project(wa, hidden, a)
-        project(wb, hidden, b)
+        project_many([wqkv, wz, wa, wb], hidden, [qkv, z, a, b])
 
     def delta_core():
         mixed[0] = states.step(qkv, z, a, b, conv, a_log, dt_bias, norm)

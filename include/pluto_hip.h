@@ -51,7 +51,9 @@ const char* pluto_hip_error_string(int code);
  *   2: pluto_hip_gdn_step_batch takes io_dtype and void* activations; the
  *      decode workspace starts with the arrival counters;
  *      pluto_hip_dense_imported_workspace_bytes grew.
- *   3: pluto_hip_gqa_decode_static_reset added. */
+ *   3: pluto_hip_gqa_decode_static_reset added.
+ *      (pluto_hip_dense_imported_forward_many was added without a bump:
+ *      nothing that existed changed.) */
 #define PLUTO_HIP_ABI_VERSION 3
 int pluto_hip_abi_version(void);
 const char* pluto_hip_target_arch(void);
@@ -530,6 +532,28 @@ int pluto_hip_dense_imported_forward_batch(void* stream, int storage,
                                            int input_dim, int output_dim,
                                            void* output, void* workspace,
                                            size_t workspace_bytes);
+/* `matrices` (1..8) such projections of the SAME tokens in one call: the query
+ * | gate, key and value projections of an attention branch, or the four input
+ * projections of a delta-net branch, which the reference's block applies to
+ * one hidden row one after the other (qwen/model.cc:174-274, each a
+ * FullyConnectedLayer of its own; no single call of the reference
+ * corresponds to this).  weights, scales (FP8 only, else NULL or all NULL),
+ * output_dims and outputs are HOST arrays of `matrices` entries; all matrices
+ * share storage and input_dim.  outputs[i] is bf16 [tokens, output_dims[i]] and
+ * bit for bit what pluto_hip_dense_imported_forward_batch gives for matrix i;
+ * the tokens are prepared once and every pass of 32 tokens is one launch
+ * over all matrices (one call a matrix costs a fixed 14 us at 32 tokens,
+ * whatever its size).  Workspace as for the batch call. */
+#define PLUTO_HIP_IMPORTED_MAX_MATRICES 8
+int pluto_hip_dense_imported_forward_many(void* stream, int storage,
+                                          int matrices,
+                                          const void* const* weights,
+                                          const float* const* scales,
+                                          const int* output_dims,
+                                          const void* input, int tokens,
+                                          int input_dim, void* const* outputs,
+                                          void* workspace,
+                                          size_t workspace_bytes);
 
 /* ------------------------------------------------------------------------
  * Test support.  No counterpart in the reference.

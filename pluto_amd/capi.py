@@ -142,6 +142,9 @@ SIGNATURES = {
     "pluto_hip_dense_imported_batch_workspace_bytes": (_SZ, [_I, _I]),
     "pluto_hip_dense_imported_forward_batch": (_I, [_VP, _I, _VP, _VP, _VP, _I, _I, _I, _VP, _VP,
                                                     _SZ]),
+    "pluto_hip_dense_imported_forward_many": (_I, [_VP, _I, _I, ctypes.POINTER(_VP),
+                                                   ctypes.POINTER(_VP), ctypes.POINTER(_I), _VP,
+                                                   _I, _I, ctypes.POINTER(_VP), _VP, _SZ]),
     "pluto_hip_gdn_recurrence": (_I, [_VP, ctypes.POINTER(DeltaParams), _I, _I, _VP, _VP,
                                       _VP, _VP, _VP, _I, ctypes.c_float, _VP, _VP, _I]),
 }
@@ -621,3 +624,28 @@ def dense_imported_forward_batch(storage, weights, scales, x, workspace=None, ou
         stream or current_stream(), storage, ptr(weights), None if scales is None else ptr(scales),
         ptr(x), tokens, input_dim, output_dim, ptr(out), ptr(workspace), workspace.numel()))
     return out
+
+
+def dense_imported_forward_many(storage, weights, scales, x, workspace=None, outs=None,
+                                stream=None):
+    """Several imported projections of the same tokens in one call: weights a list
+    of [out_i, in] matrices, scales a list of the same length (entries None unless
+    FP8); returns the list of bf16 [tokens, out_i] results."""
+    count = len(weights)
+    input_dim = weights[0].shape[1]
+    tokens = x.shape[0]
+    if workspace is None:
+        bytes_needed = lib().pluto_hip_dense_imported_batch_workspace_bytes(tokens, input_dim)
+        workspace = torch.empty(max(bytes_needed, 1), dtype=torch.uint8, device=x.device)
+    if outs is None:
+        outs = [torch.empty((tokens, w.shape[0]), dtype=torch.bfloat16, device=x.device)
+                for w in weights]
+    pointers = ctypes.c_void_p * count
+    scale_list = scales if scales is not None else [None] * count
+    check(lib().pluto_hip_dense_imported_forward_many(
+        stream or current_stream(), storage, count,
+        pointers(*[w.data_ptr() for w in weights]),
+        pointers(*[None if s is None else s.data_ptr() for s in scale_list]),
+        (ctypes.c_int * count)(*[w.shape[0] for w in weights]), ptr(x), tokens, input_dim,
+        pointers(*[o.data_ptr() for o in outs]), ptr(workspace), workspace.numel()))
+    return outs

@@ -254,13 +254,30 @@ __device__ inline uint32_t fp8_pair_to_bf16(uint32_t word) {
 
 constexpr int kTileWaves = 8;  // waves that split a tile's contraction
 
-// AHEAD (FP8 only): blocks of a wave whose weight loads are issued together.
-template <bool FP8, int AHEAD = 1>
-__global__ void __launch_bounds__(64 * kTileWaves) imported_tile_kernel(TileArgs a) {
-  __shared__ float partial[kTileWaves - 1][16][64];
+// Several matrices applied to the same tokens in one launch: workgroup b works
+// on matrix i with first_block[i] <= b < first_block[i + 1], tile b - first_block[i].
+constexpr int kManyMax = 8;
+struct TileManyArgs {
+  const void* weights[kManyMax];
+  const float* weight_scales[kManyMax];
+  uint16_t* out[kManyMax];
+  int rows[kManyMax];
+  int first_block[kManyMax + 1];
+  int matrices = 0;
+  const uint16_t* tokens = nullptr;
+  const float* token_scales = nullptr;
+  int cols = 0, count = 0;
+};
+
+// One tile: 32 rows of the matrix times up to 32 tokens, the contraction split
+// over the workgroup's waves.  AHEAD (FP8 only): blocks of a wave whose weight
+// loads are issued together.
+template <bool FP8, int AHEAD>
+__device__ __forceinline__ void imported_tile(const TileArgs& a, int tile,
+                                              float (*partial)[16][64]) {
   const int lane = threadIdx.x % 64, n = lane % 32, h = lane / 32;
   const int wave = threadIdx.x / 64;
-  const int row_base = blockIdx.x * 32;
+  const int row_base = tile * 32;
   const int row = min(row_base + n, a.rows - 1);   // rows and tokens past the end repeat
   const int token = min(n, a.count - 1);           // the last one and are not stored
   const int groups = a.cols / kGroup;
@@ -362,6 +379,30 @@ __global__ void __launch_bounds__(64 * kTileWaves) imported_tile_kernel(TileArgs
     }
 }
 
+template <bool FP8, int AHEAD = 1>
+__global__ void __launch_bounds__(64 * kTileWaves) imported_tile_kernel(TileArgs a) {
+  __shared__ float partial[kTileWaves - 1][16][64];
+  imported_tile<FP8, AHEAD>(a, blockIdx.x, partial);
+}
+
+template <bool FP8, int AHEAD = 1>
+__global__ void __launch_bounds__(64 * kTileWaves) imported_tile_many_kernel(TileManyArgs m) {
+  __shared__ float partial[kTileWaves - 1][16][64];
+  int which = 0;
+  while (which + 1 < m.matrices && static_cast<int>(blockIdx.x) >= m.first_block[which + 1])
+    ++which;
+  TileArgs a;
+  a.weights = m.weights[which];
+  a.weight_scales = m.weight_scales[which];
+  a.tokens = m.tokens;
+  a.token_scales = m.token_scales;
+  a.out = m.out[which];
+  a.cols = m.cols;
+  a.rows = m.rows[which];
+  a.count = m.count;
+  imported_tile<FP8, AHEAD>(a, blockIdx.x - m.first_block[which], partial);
+}
+
 template <int AHEAD>
 void launch_fp8_tiles_ahead(hipStream_t s, const TileArgs& t, int blocks) {
   imported_tile_kernel<true, AHEAD><<<blocks, 64 * kTileWaves, 0, s>>>(t);
@@ -379,6 +420,25 @@ void launch_fp8_tiles(hipStream_t s, const TileArgs& t, int blocks) {
     case 6: return launch_fp8_tiles_ahead<6>(s, t, blocks);
     case 7: return launch_fp8_tiles_ahead<7>(s, t, blocks);
     default: return launch_fp8_tiles_ahead<8>(s, t, blocks);
+  }
+}
+
+template <int AHEAD>
+void launch_fp8_tiles_many_ahead(hipStream_t s, const TileManyArgs& t, int blocks) {
+  imported_tile_many_kernel<true, AHEAD><<<blocks, 64 * kTileWaves, 0, s>>>(t);
+}
+
+void launch_fp8_tiles_many(hipStream_t s, const TileManyArgs& t, int blocks) {
+  const int groups = t.cols / kGroup;
+  switch (std::min(8, (groups + kTileWaves - 1) / kTileWaves)) {
+    case 1: return launch_fp8_tiles_many_ahead<1>(s, t, blocks);
+    case 2: return launch_fp8_tiles_many_ahead<2>(s, t, blocks);
+    case 3: return launch_fp8_tiles_many_ahead<3>(s, t, blocks);
+    case 4: return launch_fp8_tiles_many_ahead<4>(s, t, blocks);
+    case 5: return launch_fp8_tiles_many_ahead<5>(s, t, blocks);
+    case 6: return launch_fp8_tiles_many_ahead<6>(s, t, blocks);
+    case 7: return launch_fp8_tiles_many_ahead<7>(s, t, blocks);
+    default: return launch_fp8_tiles_many_ahead<8>(s, t, blocks);
   }
 }
 
@@ -486,6 +546,53 @@ int launch_dense_imported_forward(hipStream_t s, int storage, const void* weight
   return launch_status();
 }
 
+// Several matrices of one storage kind and input width applied to the same
+// tokens: the tokens are prepared once and every pass of 32 tokens is one
+// launch over the tiles of all matrices.  Takes the matrix-core path only
+// (tile_path()); the caller falls back to one call a matrix otherwise.
+int launch_dense_imported_forward_many(hipStream_t s, int storage, int matrices,
+                                       const void* const* weights, const float* const* scales,
+                                       const int* output_dims, const void* input, int tokens,
+                                       int input_dim, void* const* outputs, void* workspace) {
+  const bool fp8 = storage == PLUTO_HIP_MATRIX_FP8_E4M3;
+  TileManyArgs t;
+  t.matrices = matrices;
+  t.cols = input_dim;
+  t.tokens = static_cast<const uint16_t*>(input);
+  t.first_block[0] = 0;
+  for (int i = 0; i < kManyMax; ++i) {
+    const bool used = i < matrices;
+    t.weights[i] = used ? weights[i] : nullptr;
+    t.weight_scales[i] = used && fp8 ? scales[i] : nullptr;
+    t.out[i] = used ? static_cast<uint16_t*>(outputs[i]) : nullptr;
+    t.rows[i] = used ? output_dims[i] : 0;
+    t.first_block[i + 1] = t.first_block[i] + (used ? (output_dims[i] + 31) / 32 : 0);
+  }
+  if (fp8) {
+    const dim3 groups(static_cast<unsigned>((input_dim + kGroup - 1) / kGroup),
+                      static_cast<unsigned>(tokens));
+    uint16_t* values = static_cast<uint16_t*>(workspace);
+    float* token_scales = reinterpret_cast<float*>(static_cast<char*>(workspace) +
+                                                   tile_values_bytes(tokens, input_dim));
+    imported_token_fp8_kernel<<<groups, kGroup, 0, s>>>(static_cast<const uint16_t*>(input),
+                                                        input_dim, values, token_scales);
+    t.tokens = values;
+    t.token_scales = token_scales;
+  }
+  const int blocks = t.first_block[matrices];
+  for (int done = 0; done < tokens; done += 32) {
+    t.count = tokens - done < 32 ? tokens - done : 32;
+    if (fp8)
+      launch_fp8_tiles_many(s, t, blocks);
+    else
+      imported_tile_many_kernel<false><<<blocks, 64 * kTileWaves, 0, s>>>(t);
+    t.tokens += static_cast<size_t>(32) * input_dim;
+    if (fp8) t.token_scales += static_cast<size_t>(32) * (input_dim / kGroup);
+    for (int i = 0; i < matrices; ++i) t.out[i] += static_cast<size_t>(32) * output_dims[i];
+  }
+  return launch_status();
+}
+
 }  // namespace pluto_hip
 
 using namespace pluto_hip;
@@ -538,6 +645,44 @@ int pluto_hip_dense_imported_forward_batch(void* stream, int storage, const void
     return PLUTO_HIP_EWORKSPACE;
   return launch_dense_imported_forward(static_cast<hipStream_t>(stream), storage, weights, scales,
                                        input, tokens, input_dim, output_dim, output, workspace);
+}
+
+int pluto_hip_dense_imported_forward_many(void* stream, int storage, int matrices,
+                                          const void* const* weights,
+                                          const float* const* scales, const int* output_dims,
+                                          const void* input, int tokens, int input_dim,
+                                          void* const* outputs, void* workspace,
+                                          size_t workspace_bytes) {
+  if (matrices <= 0 || matrices > PLUTO_HIP_IMPORTED_MAX_MATRICES || !weights || !output_dims ||
+      !outputs || !input)
+    return PLUTO_HIP_EINVAL;
+  const bool fp8 = storage == PLUTO_HIP_MATRIX_FP8_E4M3;
+  if (fp8 && !scales) return PLUTO_HIP_EINVAL;
+  long long tiles = 0;
+  for (int i = 0; i < matrices; ++i) {
+    const int status = validate_imported(storage, fp8 ? scales[i] : nullptr, tokens, input_dim,
+                                         output_dims[i]);
+    if (status != 0) return status;
+    if (!fp8 && scales && scales[i]) return PLUTO_HIP_EINVAL;
+    if (!weights[i] || !outputs[i]) return PLUTO_HIP_EINVAL;
+    tiles += (output_dims[i] + 31) / 32;
+  }
+  if (tiles > 0x7fffffffLL) return PLUTO_HIP_EINVAL;
+  if (!workspace || workspace_bytes < dense_imported_workspace_bytes(tokens, input_dim))
+    return PLUTO_HIP_EWORKSPACE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (tile_path(storage, tokens, input_dim))
+    return launch_dense_imported_forward_many(s, storage, matrices, weights, scales, output_dims,
+                                              input, tokens, input_dim, outputs, workspace);
+  // few tokens, FP32 matrices or a ragged width: one call a matrix, same results
+  for (int i = 0; i < matrices; ++i) {
+    const int status = launch_dense_imported_forward(s, storage, weights[i],
+                                                     fp8 ? scales[i] : nullptr, input, tokens,
+                                                     input_dim, output_dims[i], outputs[i],
+                                                     workspace);
+    if (status != 0) return status;
+  }
+  return 0;
 }
 
 }  // extern "C"

@@ -66,6 +66,35 @@ Status ProjectionSet::Run(int which, const void* input, void* output) const {
       "imported projection launch");
 }
 
+Status ProjectionSet::RunFirst(int count, const void* input) const {
+  bool alike = count <= PLUTO_HIP_IMPORTED_MAX_MATRICES;
+  for (int i = 1; i < count && alike; ++i)
+    alike = *layers_[i]->imported_storage() == *layers_[0]->imported_storage() &&
+            layers_[i]->input_dim() == layers_[0]->input_dim();
+  if (!alike) {
+    for (int which = 0; which < count; ++which)
+      RETURN_IF_ERROR(Run(which, input, stage(which)));
+    return OkStatus();
+  }
+  const void* weights[PLUTO_HIP_IMPORTED_MAX_MATRICES];
+  const float* scales[PLUTO_HIP_IMPORTED_MAX_MATRICES];
+  int output_dims[PLUTO_HIP_IMPORTED_MAX_MATRICES];
+  void* outputs[PLUTO_HIP_IMPORTED_MAX_MATRICES];
+  for (int i = 0; i < count; ++i) {
+    const Span<Buffer> buffers = layers_[i]->weights();
+    weights[i] = buffers[0].data();
+    scales[i] = buffers.size() == 2 ? static_cast<const float*>(buffers[1].data()) : nullptr;
+    output_dims[i] = layers_[i]->output_dim();
+    outputs[i] = stage(i);
+  }
+  return hip::HipStatus(
+      pluto_hip_dense_imported_forward_many(
+          executor_->stream(), StorageCode(*layers_[0]->imported_storage()), count, weights,
+          scales, output_dims, input, batch_, layers_[0]->input_dim(), outputs,
+          workspace_[0].data(), workspace_[0].size_bytes()),
+      "imported projections launch");
+}
+
 }  // namespace internal
 
 namespace {
@@ -140,8 +169,7 @@ StatusOr<FwdResult> BatchedFullAttentionBranch::fwd_impl(hip::Executor& executor
       return ResourceExhaustedError("full-attention cache capacity reached");
   ASSIGN_OR_RETURN(auto result, Buffer::Allocate(executor, inputs[0].size_bytes()));
   const void* hidden = inputs[0].data();
-  for (int which = 0; which < 3; ++which)
-    RETURN_IF_ERROR(projections_.Run(which, hidden, projections_.stage(which)));
+  RETURN_IF_ERROR(projections_.RunFirst(3, hidden));
   RETURN_IF_ERROR(cached_attention_ops::CachedAttentionStepBatchBFloat16(
       executor, parameters_, Span<KeyValueCache* const>(borrowed_.data(), borrowed_.size()),
       projections_.stage(0), projections_.stage(1), projections_.stage(2),
@@ -206,8 +234,7 @@ StatusOr<FwdResult> BatchedDeltaNetBranch::fwd_impl(hip::Executor& executor,
   RETURN_IF_ERROR(CheckHidden(executor_, executor, inputs, batch(), width));
   ASSIGN_OR_RETURN(auto result, Buffer::Allocate(executor, inputs[0].size_bytes()));
   const void* hidden = inputs[0].data();
-  for (int which = 0; which < 4; ++which)
-    RETURN_IF_ERROR(projections_.Run(which, hidden, projections_.stage(which)));
+  RETURN_IF_ERROR(projections_.RunFirst(4, hidden));
   auto weight = [this](int i) { return static_cast<const float*>(weights_[i].data()); };
   RETURN_IF_ERROR(state_->StepBFloat16(projections_.stage(0), projections_.stage(1),
                                        projections_.stage(2), projections_.stage(3), weight(0),

@@ -42,6 +42,10 @@ class ProjectionSet {
                                         const std::vector<std::pair<int, int>>& shape);
   // Projection `which` of `batch` bf16 rows at `input`, into `output`.
   Status Run(int which, const void* input, void* output) const;
+  // Projections 0 .. count-1 of the same rows into their stages: one call when
+  // they share a storage kind (the loader gives a model's matrices one), one
+  // call each otherwise; the results are the same bits either way.
+  Status RunFirst(int count, const void* input) const;
   void* stage(int which) const { return stages_[which].data(); }
   int output_dim(int which) const { return layers_[which]->output_dim(); }
 

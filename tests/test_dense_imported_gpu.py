@@ -174,6 +174,72 @@ def test_matrix_core_batch_matches_the_oracle(capi, oracle):
             assert np.mean(got[t] != want) <= 0.05, (storage, t)
 
 
+@pytest.mark.parametrize("cols,tokens", [(512, 32), (512, 40), (1024, 33), (512, 5), (263, 11)])
+def test_several_matrices_of_one_input_match_the_single_calls(capi, oracle, cols, tokens):
+    """The query | gate, key and value projections of a block (qwen/model.cc:174-274)
+    see the same rows: pluto_hip_dense_imported_forward_many prepares the tokens
+    once and walks the tiles of all matrices in one launch a pass.  Bit for
+    bit the batch call's results for every matrix, on the matrix-core path
+    (partial passes, partial row tiles, a matrix smaller than a tile) and on the
+    vector path it falls back to (few tokens, ragged widths, FP32 weights)."""
+    heights = [70, 1000, 32, 7, 129]
+    rng = np.random.default_rng(cols * 3 + tokens)
+    x = bf16_tensor(oracle, rng.standard_normal((tokens, cols)))
+    sources = [rng.standard_normal((rows, cols)).astype(np.float32) for rows in heights]
+    scales = [torch.from_numpy(rng.uniform(0.5, 2.0, ((rows + 127) // 128, (cols + 127) // 128))
+                               .astype(np.float32)).cuda() for rows in heights]
+    cases = [(capi.MATRIX_F32, [torch.from_numpy(w).cuda() for w in sources], None),
+             (capi.MATRIX_BF16, [torch.from_numpy(w).cuda().to(torch.bfloat16) for w in sources], None),
+             (capi.MATRIX_FP8_E4M3,
+              [torch.from_numpy(oracle.f32_to_fp8_e4m3(w)).cuda() for w in sources], scales)]
+    for storage, weights, s in cases:
+        many = capi.dense_imported_forward_many(storage, weights, s, x)
+        for i, w in enumerate(weights):
+            single = capi.dense_imported_forward_batch(storage, w, None if s is None else s[i], x)
+            torch.cuda.synchronize()
+            assert torch.isfinite(single.float()).all()
+            assert torch.equal(many[i].view(torch.int16), single.view(torch.int16)), (storage, i)
+    # one matrix is the batch call
+    storage, weights, s = cases[2]
+    alone = capi.dense_imported_forward_many(storage, weights[1:2], s[1:2], x)[0]
+    assert torch.equal(alone, capi.dense_imported_forward_batch(storage, weights[1], s[1], x))
+
+
+def test_several_matrices_rejections(capi):
+    import ctypes
+    lib = capi.lib()
+    w = torch.zeros((32, 128), dtype=torch.bfloat16, device="cuda")
+    x = torch.zeros((16, 128), dtype=torch.bfloat16, device="cuda")
+    y = torch.full((16, 32), -3.0, dtype=torch.bfloat16, device="cuda")
+    ws = torch.zeros(1 << 16, dtype=torch.uint8, device="cuda")
+    s = torch.ones(1, dtype=torch.float32, device="cuda")
+    stream = capi.current_stream()
+    pointers = ctypes.c_void_p * 9
+
+    def call(storage=capi.MATRIX_BF16, count=2, weights=(w, w), scales=None, dims=(32, 32),
+             outs=(y, y), tokens=16, cols=128, workspace_bytes=1 << 16, null_arrays=False):
+        w_list = pointers(*[t.data_ptr() for t in weights])
+        o_list = pointers(*[t.data_ptr() for t in outs])
+        s_list = None if scales is None else pointers(*[None if t is None else t.data_ptr()
+                                                        for t in scales])
+        return lib.pluto_hip_dense_imported_forward_many(
+            stream, storage, count, None if null_arrays else w_list, s_list,
+            (ctypes.c_int * 9)(*dims), capi.ptr(x), tokens, cols, o_list, capi.ptr(ws),
+            workspace_bytes)
+
+    assert call() == 0
+    assert call(count=0) == capi.EINVAL and call(count=9, weights=(w,) * 9, dims=(32,) * 9,
+                                                 outs=(y,) * 9) == capi.EINVAL
+    assert call(null_arrays=True) == capi.EINVAL
+    assert call(dims=(32, 0)) == capi.EINVAL and call(cols=0) == capi.EINVAL
+    assert call(tokens=0) == capi.EINVAL and call(tokens=4097) == capi.EINVAL
+    assert call(storage=capi.MATRIX_FP8_E4M3) == capi.EINVAL            # FP8 without scales
+    assert call(storage=capi.MATRIX_FP8_E4M3, scales=(s, None)) == capi.EINVAL
+    assert call(scales=(s, s)) == capi.EINVAL                             # scales without FP8
+    assert call(workspace_bytes=4) == capi.EWORKSPACE
+    torch.cuda.synchronize()
+
+
 def test_rejects_bad_arguments(capi):
     lib = capi.lib()
     w = torch.zeros(6, dtype=torch.float32, device="cuda")
