@@ -60,13 +60,13 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E (published)
 # kept as profiles/*_hbm_traffic.md.  None = not measured.
 MEASURED_TRAFFIC_BYTES = {
     # (workload, kernel group): (bytes read + written, commit the counters were read at)
-    ("mha_train_bf16", "flash_forward_kernel<64>"): (99.1e6 + 26.7e6, "588f4ef"),
-    ("mha_train_bf16", "flash_dq_kernel<64>"): (179.4e6 + 77.1e6, "588f4ef"),
-    ("mha_train_bf16", "flash_dkv_kernel<64>"): (154.5e6 + 100.7e6, "588f4ef"),
-    ("gqa_prefill", "flash_forward_pipelined_kernel<128>"): (184.6e6 + 88.1e6, "588f4ef"),
-    ("gqa_prefill_d256", "flash_forward_pipelined_kernel<256>"): (444.8e6 + 100.9e6, "588f4ef"),
-    ("gqa_decode", "decode_fused_kernel<128,6>"): (1044.2e6 + 13.0e6, "588f4ef"),
-    ("gdn_scan", "gdn_chunk_scan"): (524.7e6 + 138.5e6, "588f4ef"),
+    ("mha_train_bf16", "flash_forward_kernel<64>"): (99.1e6 + 26.7e6, "4f26c5a"),
+    ("mha_train_bf16", "flash_dq_kernel<64>"): (179.5e6 + 77.1e6, "4f26c5a"),
+    ("mha_train_bf16", "flash_dkv_kernel<64>"): (154.5e6 + 100.7e6, "4f26c5a"),
+    ("gqa_prefill", "flash_forward_pipelined_kernel<128>"): (184.6e6 + 88.1e6, "4f26c5a"),
+    ("gqa_prefill_d256", "flash_forward_pipelined_kernel<256>"): (444.8e6 + 100.9e6, "4f26c5a"),
+    ("gqa_decode", "decode_fused_kernel<128,6>"): (1044.2e6 + 13.0e6, "4f26c5a"),
+    ("gdn_scan", "gdn_chunk_scan"): (524.5e6 + 138.8e6, "4f26c5a"),
 }
 
 NAMES = ["mha_train_bf16", "mha_fwd_fp32", "gqa_prefill", "gqa_decode", "gdn_scan"]
