@@ -343,11 +343,14 @@ def test_long_prefill_kernels_agree_bit_for_bit(capi, oracle, lengths, d):
     assert_close_bf16(got[-3:], want["out"][total - 3:total], "last rows of the long prefill")
 
 
-def test_config4_batched_decode(capi, oracle):
+@pytest.mark.parametrize("d,rotary,split", [(128, 32, 512), (256, 64, 0)])
+def test_config4_batched_decode(capi, oracle, d, rotary, split):
     # batch 32, context length ~ U[1024, 32768] (seed 3), 24 query heads, 4 KV
-    # heads, D=128, bf16 cache, split-K over 512-token blocks.
-    batch, qh, kh, d, capacity = 32, 24, 4, 128, 32768
-    kw = dict(query_heads=qh, key_value_heads=kh, head_dim=d, rotary_dim=32, capacity=capacity)
+    # heads, D=128, bf16 cache, split-K over 512-token blocks; and the same
+    # batch at the model's own head width (cached_attention_ops.h:13-22: 256,
+    # 64 rotated channels) with the default blocks of 1024 rows.
+    batch, qh, kh, capacity = 32, 24, 4, 32768
+    kw = dict(query_heads=qh, key_value_heads=kh, head_dim=d, rotary_dim=rotary, capacity=capacity)
     p, po = both_params(capi, oracle, **kw)
     rng = np.random.default_rng(3)
     lengths = 1024 + np.floor(rng.random(batch) * 31745).astype(int)
@@ -366,7 +369,7 @@ def test_config4_batched_decode(capi, oracle):
     qw, kw_ = values(d, 0.2, 0.3), values(d, 0.8, 0.4)
     bf = torch.bfloat16
     out = capi.gqa_decode(p, dev(q_gate, bf), dev(k, bf), dev(v, bf), dev(qw), dev(kw_), caches,
-                          split_tokens=512, advance=False)
+                          split_tokens=split, advance=False)
     assert capi.last_path() == capi.PATH_SPLIT_K
     torch.cuda.synchronize()
     got = out.float().cpu().numpy()
@@ -388,12 +391,12 @@ def test_config4_batched_decode(capi, oracle):
     # all sequences: against the any-shape FP32-arithmetic kernels
     with capi.force_generic():
         out2 = capi.gqa_decode(p, dev(q_gate, bf), dev(k, bf), dev(v, bf), dev(qw), dev(kw_), caches,
-                               split_tokens=512, advance=False)
+                               split_tokens=split, advance=False)
         torch.cuda.synchronize()
     near(got, out2.float().cpu().numpy(), True)
     # bitwise repeatable (fixed-order split-K combine)
     again = capi.gqa_decode(p, dev(q_gate, bf), dev(k, bf), dev(v, bf), dev(qw), dev(kw_), caches,
-                            split_tokens=512, advance=False)
+                            split_tokens=split, advance=False)
     assert torch.equal(out, again)
 
 
